@@ -1,0 +1,182 @@
+/*
+ * saga_hip.h - C ABI of the MI355X (gfx950) kernel library behind Saga's "hip" engine.
+ *
+ * Every entry point enqueues work on the given HIP stream and returns immediately.
+ * Plain pointers and sizes only: no C++ types, no exceptions, no torch types.
+ * Return value: 0 on success, a negative SAGA_HIP_E* code for a rejected argument,
+ * or a positive hipError_t from the runtime.
+ *
+ * Each declaration cites the reference code whose role it takes (paths relative to
+ * the reference tree).  The callers in the reference design are the exec() methods
+ * of the backend's operation objects (src/cuda/cuda_dnn.cpp, cuda_optimizer.cpp).
+ */
+#ifndef SAGA_HIP_H
+#define SAGA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* A hipStream_t, passed opaque so that C callers need no HIP headers. */
+typedef void *saga_stream_t;
+
+/* Element types; values equal saga::Tensor::DataType (saga.hpp:161-168). */
+enum SagaDType {
+    SAGA_U8 = 0,
+    SAGA_HALF = 1,
+    SAGA_FLOAT = 2,
+    SAGA_INT64 = 3,
+    SAGA_I32 = 4,
+    SAGA_I16 = 5
+};
+
+enum SagaError {
+    SAGA_HIP_OK = 0,
+    SAGA_HIP_EINVAL = -1,       /* malformed argument (null pointer, negative size ...) */
+    SAGA_HIP_ESHAPE = -2,       /* operand shapes do not agree */
+    SAGA_HIP_EUNSUPPORTED = -3, /* valid but not implemented (dtype / layout combination) */
+    SAGA_HIP_EWORKSPACE = -4    /* workspace missing or too small */
+};
+
+/*
+ * A tensor as the kernels see it: logical dims are always (N, C, H, W) (rank-2 tensors
+ * use H = W = 1) and the strides, in elements, carry the physical layout: NCHW, NHWC,
+ * or a channel slice of a wider tensor (how concat is realised).
+ * Takes the role of cudnnTensorDescriptor_t + device pointer (src/cuda/cuda_tensor.cpp:560-583).
+ */
+typedef struct SagaTensorView {
+    void *ptr;
+    int32_t dims[4];
+    int64_t strides[4];
+    int32_t dtype; /* enum SagaDType */
+} SagaTensorView;
+
+/* Square pad / stride / dilation as in src/cuda/cuda_dnn.cpp:227-235. */
+typedef struct SagaConvParams {
+    int32_t pad;
+    int32_t stride;
+    int32_t dilation;
+    int32_t group;
+} SagaConvParams;
+
+/* Flags returned to the host by the optimizer; layout of CudaAux (src/cuda/cuda_aux.hpp:5-10). */
+typedef struct SagaAux {
+    uint32_t range;
+    uint32_t inf;
+    uint32_t nan;
+    uint32_t anomaly;
+} SagaAux;
+
+enum SagaConvKind { SAGA_CONV_FWD = 0, SAGA_CONV_BWD_DATA = 1, SAGA_CONV_BWD_FILTER = 2 };
+enum SagaActMode { SAGA_ACT_RELU = 0, SAGA_ACT_SIGMOID = 1, SAGA_ACT_TANH = 2, SAGA_ACT_SWISH = 3, SAGA_ACT_LEAKYRELU = 4 };
+enum SagaPoolMode { SAGA_POOL_MAX = 0, SAGA_POOL_AVG = 1 };
+
+/* Epilogue / fusion flags for the batch-norm entry points. */
+enum SagaBnFlags {
+    SAGA_BN_RELU = 1, /* y = relu(bn(x) [+ z]) ; backward masks dy by y > 0 */
+    SAGA_BN_ADD = 2   /* z is added before the activation; backward also emits dz */
+};
+
+const char *saga_hip_error_string(int code);
+
+/* Library / device bring-up; returns the number of compute units of `device` in *cus (may be NULL). */
+int saga_hip_init(int device, int *cus);
+
+/* ---- convolution: cudnnConvolutionForward / BackwardData / BackwardFilter
+ *      (src/cuda/cuda_dnn.cpp:338-347, :467-476, :419-428).  Cross-correlation.
+ *      w has logical dims (K, C/group, R, S); for NHWC programs it is stored K,R,S,C
+ *      (strides say so).  out = alpha * conv + beta * out.
+ *      Transposed convolution is the same three calls with roles exchanged
+ *      (src/cuda/cuda_dnn.cpp:542-574). */
+size_t saga_hip_conv2d_workspace_size(int kind, const SagaTensorView *x, const SagaTensorView *w,
+                                      const SagaTensorView *y, const SagaConvParams *p);
+int saga_hip_conv2d_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y,
+                        const SagaConvParams *p, float alpha, float beta, void *workspace, size_t ws_bytes,
+                        saga_stream_t stream);
+int saga_hip_conv2d_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx,
+                             const SagaConvParams *p, float alpha, float beta, void *workspace, size_t ws_bytes,
+                             saga_stream_t stream);
+int saga_hip_conv2d_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, const SagaTensorView *dw,
+                               const SagaConvParams *p, float alpha, float beta, void *workspace,
+                               size_t ws_bytes, saga_stream_t stream);
+
+/* y[n,c,:,:] += b[c] : cudnnAddTensor of a {1,C,1,1} bias (src/cuda/cuda_dnn.cpp:39-68). b is fp32 or y's type. */
+int saga_hip_bias_add(const SagaTensorView *y, const SagaTensorView *b, saga_stream_t stream);
+/* db[c] = beta*db + sum_{n,h,w} dy : cudnnConvolutionBackwardBias (src/cuda/cuda_dnn.cpp:378-385). */
+int saga_hip_bias_bwd(const SagaTensorView *dy, const SagaTensorView *db, float beta, saga_stream_t stream);
+
+/* ---- GEMM: cublasSgemm / cublasHgemm as used by the fc node (src/cuda/cuda_dnn.cpp:1001-1025).
+ *      Row-major: C[M,N] = alpha * op(A) * op(B) + beta * C, op(A) is MxK, op(B) is KxN;
+ *      trans flag set means the matrix is stored transposed (A as KxM, B as NxK).
+ *      fp16 operands accumulate in fp32. */
+int saga_hip_gemm(int transA, int transB, int M, int N, int K, float alpha, const void *A, int lda, const void *B,
+                  int ldb, float beta, void *C, int ldc, int dtype, saga_stream_t stream);
+
+/* ---- batch normalisation (spatial, per channel; s,b,m,v and saved statistics are fp32 [C]).
+ *      infer: cudnnBatchNormalizationForwardInference (src/cuda/cuda_dnn.cpp:1641-1651);
+ *      train: ...ForwardTraining / ForwardTrainingEx with BN, BN_ACTIVATION, BN_ADD_ACTIVATION
+ *             (src/cuda/cuda_dnn.cpp:1689-1709, :2041-2069);
+ *      bwd:   ...Backward / BackwardEx (src/cuda/cuda_dnn.cpp:1754-1766, :2138-2163).
+ *      z / dz may be NULL unless SAGA_BN_ADD is set.  save_invstd holds 1/sqrt(var+eps).
+ *      Running variance is updated with the unbiased batch variance. */
+int saga_hip_bn_infer(const SagaTensorView *x, const SagaTensorView *z, const SagaTensorView *y, const float *s,
+                      const float *b, const float *m, const float *v, float eps, int flags, saga_stream_t stream);
+size_t saga_hip_bn_workspace_size(const SagaTensorView *x);
+int saga_hip_bn_train_fwd(const SagaTensorView *x, const SagaTensorView *z, const SagaTensorView *y,
+                          const float *s, const float *b, float *run_m, float *run_v, float *save_mean,
+                          float *save_invstd, float eps, float expavg, int flags, void *workspace,
+                          size_t ws_bytes, saga_stream_t stream);
+int saga_hip_bn_bwd(const SagaTensorView *x, const SagaTensorView *y, const SagaTensorView *dy,
+                    const SagaTensorView *dx, const SagaTensorView *dz, const float *s, const float *save_mean,
+                    const float *save_invstd, float *ds, float *db, float beta_dx, float beta_dz, float beta_p,
+                    int flags, void *workspace, size_t ws_bytes, saga_stream_t stream);
+
+/* ---- activations: cudnnActivationForward / Backward (src/cuda/cuda_dnn.cpp:631-638, :668-676),
+ *      leaky relu kernel (src/cuda/cuda_kernels.cu:478-495).  y = act(x) + beta*y ; dx = dy*act'(x) + beta*dx. */
+int saga_hip_act_fwd(int mode, float alpha, const SagaTensorView *x, const SagaTensorView *y, float beta,
+                     saga_stream_t stream);
+int saga_hip_act_bwd(int mode, float alpha, const SagaTensorView *x, const SagaTensorView *y,
+                     const SagaTensorView *dy, const SagaTensorView *dx, float beta, saga_stream_t stream);
+
+/* ---- pooling: cudnnPoolingForward / Backward, MAX and AVERAGE_COUNT_INCLUDE_PADDING
+ *      (src/cuda/cuda_dnn.cpp:820-836, :858-866).  idx (optional, I32, dims of y) receives the
+ *      flat h*W+w position of each window's maximum, first maximum in scan order. */
+int saga_hip_pool_fwd(int mode, const SagaTensorView *x, const SagaTensorView *y, const SagaTensorView *idx,
+                      int size, int pad, int stride, saga_stream_t stream);
+int saga_hip_pool_bwd(int mode, const SagaTensorView *x, const SagaTensorView *y, const SagaTensorView *dy,
+                      const SagaTensorView *dx, int size, int pad, int stride, float beta, saga_stream_t stream);
+
+/* y = a + b : cudnnOpTensor ADD (src/cuda/cuda_dnn.cpp:1866-1875). */
+int saga_hip_add(const SagaTensorView *a, const SagaTensorView *b, const SagaTensorView *y, saga_stream_t stream);
+/* dst = alpha*src + beta*dst : cudnnTransformTensor (src/cuda/cuda_dnn.cpp:72-99); also layout conversion. */
+int saga_hip_axpby(const SagaTensorView *src, const SagaTensorView *dst, float alpha, float beta,
+                   saga_stream_t stream);
+/* dst = (float)src * scale : convert kernels (src/cuda/cuda_kernels.cu:102-151). */
+int saga_hip_convert(const SagaTensorView *src, const SagaTensorView *dst, float scale, saga_stream_t stream);
+/* softmax over C at every (n,h,w): cudnnSoftmaxForward ACCURATE / MODE_CHANNEL (src/cuda/cuda_dnn.cpp:1937-1945). */
+int saga_hip_softmax(const SagaTensorView *x, const SagaTensorView *y, saga_stream_t stream);
+
+/* ---- classifier head: catclassifier_fwd / catclassifier_bwd (src/cuda/cuda_kernels.cu:11-96).
+ *      x is [N,C] with contiguous rows; pred/labels are int32 [N]; loss fp32 [N] (may be NULL). */
+int saga_hip_catclassifier_fwd(const SagaTensorView *x, int32_t *pred, saga_stream_t stream);
+int saga_hip_catclassifier_bwd(const SagaTensorView *x, const SagaTensorView *dx, const int32_t *pred,
+                               const int32_t *labels, float *loss, float scale, saga_stream_t stream);
+
+/* ---- optimizer: adam_float / adam_mixed (src/cuda/cuda_kernels.cu:159-250).
+ *      b1t = 1/(1-0.9^t), b2t = 1/(1-0.999^t) are computed by the caller (src/cuda/cuda_optimizer.cpp:79-80).
+ *      aux points to a SagaAux in device-visible memory. */
+int saga_hip_adam_f32(size_t n, float *w, const float *g, float *m, float *v, float b1t, float b2t, float lr,
+                      float lambda, SagaAux *aux, saga_stream_t stream);
+int saga_hip_adam_mixed(size_t n, float alpha, void *w_half, const void *g_half, float *m, float *v, float *c,
+                        float b1t, float b2t, float lr, float lambda, SagaAux *aux, saga_stream_t stream);
+
+/* Fills `bytes` bytes with the byte `value` using a kernel (safe inside captured graphs). */
+int saga_hip_fill(void *ptr, int value, size_t bytes, saga_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SAGA_HIP_H */

@@ -1,0 +1,705 @@
+// Batch normalisation for gfx950: inference, training forward (with optional fused
+// residual add + relu) and backward.  Everything here is HBM-bound.
+//
+// Channels-last tensors are walked as rows of C contiguous channels: a 256-thread block is
+// shaped (CVB channel-vectors) x (RB rows); lanes along x read consecutive 16-byte vectors so
+// each wavefront touches whole rows, and every thread keeps its channel's parameters in
+// registers for all the rows it visits.  Per-channel sums are reduced thread -> LDS ->
+// per-block partials in the workspace -> one small finalize kernel, so the data is read
+// exactly twice in training forward (statistics, then normalise) and backward.
+//
+// Statistics are accumulated on values shifted by the channel's first element, which removes
+// the cancellation in E[x^2] - E[x]^2 when |mean| >> stddev.
+#include "common.hpp"
+
+namespace {
+
+template <typename T, int VN> struct VecT;
+template <> struct VecT<half_t, 8> { typedef half8_t type; };
+template <> struct VecT<float, 4> { typedef float4_t type; };
+template <> struct VecT<half_t, 1> { typedef half_t type; };
+template <> struct VecT<float, 1> { typedef float type; };
+
+template <typename T, int VN> struct Ld {
+    typedef typename VecT<T, VN>::type V;
+    static __device__ __forceinline__ void load(const T *p, float (&o)[VN])
+    {
+        if constexpr(VN == 1) {
+            o[0] = (float)*p;
+        } else {
+            const V v = *(const V *)p;
+#pragma unroll
+            for(int j = 0; j < VN; j++)
+                o[j] = (float)v[j];
+        }
+    }
+    static __device__ __forceinline__ void store(T *p, const float (&o)[VN])
+    {
+        if constexpr(VN == 1) {
+            *p = (T)o[0];
+        } else {
+            V v;
+#pragma unroll
+            for(int j = 0; j < VN; j++)
+                v[j] = (T)o[j];
+            *(V *)p = v;
+        }
+    }
+};
+
+struct Shape {
+    int cvb;  // channel vectors per block (power of two <= 64)
+    int rb;   // rows per block = 256 / cvb
+    int gy;   // blocks along channels
+    int gx;   // blocks along rows
+};
+
+static Shape plan(int64_t rows, int cvec)
+{
+    Shape s;
+    s.cvb = 1;
+    while(s.cvb < cvec && s.cvb < 64)
+        s.cvb <<= 1;
+    s.rb = 256 / s.cvb;
+    s.gy = (cvec + s.cvb - 1) / s.cvb;
+    int64_t want = (rows + (int64_t)s.rb * 4 - 1) / ((int64_t)s.rb * 4);
+    int cap = 2048 / s.gy;
+    if(cap < 1)
+        cap = 1;
+    if(want > cap)
+        want = cap;
+    if(want < 1)
+        want = 1;
+    s.gx = (int)want;
+    return s;
+}
+
+// ---------------------------------------------------------------- channels-last kernels
+
+// y = x*scale[c] + shift[c] (+ z) (relu).  MODE 0: scale/shift from s,b,m,v (inference);
+// MODE 1: scale/shift precomputed in ss[0..C), ss[C..2C) (training, second pass).
+template <typename T, int VN, int MODE>
+__global__ void __launch_bounds__(256)
+    bn_apply_cl(const T *__restrict__ x, int64_t px, const T *__restrict__ z, int64_t pz, T *__restrict__ y, int64_t py,
+                const float *__restrict__ s, const float *__restrict__ b, const float *__restrict__ m,
+                const float *__restrict__ v, const float *__restrict__ ss, float eps, int64_t rows, int C, int cvb,
+                int flags)
+{
+    const int tx = threadIdx.x % cvb, ty = threadIdx.x / cvb, rb = 256 / cvb;
+    const int c0 = (blockIdx.y * cvb + tx) * VN;
+    if(c0 >= C)
+        return;
+    float sc[VN], sh[VN];
+#pragma unroll
+    for(int j = 0; j < VN; j++) {
+        if(MODE == 0) {
+            sc[j] = s[c0 + j] * rsqrtf(v[c0 + j] + eps);
+            sh[j] = b[c0 + j] - m[c0 + j] * sc[j];
+        } else {
+            sc[j] = ss[c0 + j];
+            sh[j] = ss[C + c0 + j];
+        }
+    }
+    const bool relu = flags & SAGA_BN_RELU, add = flags & SAGA_BN_ADD;
+    for(int64_t r = (int64_t)blockIdx.x * rb + ty; r < rows; r += (int64_t)gridDim.x * rb) {
+        float xv[VN], zv[VN];
+        Ld<T, VN>::load(x + r * px + c0, xv);
+        if(add)
+            Ld<T, VN>::load(z + r * pz + c0, zv);
+#pragma unroll
+        for(int j = 0; j < VN; j++) {
+            float o = xv[j] * sc[j] + sh[j];
+            if(add)
+                o += zv[j];
+            if(relu)
+                o = (o != o) ? o : fmaxf(o, 0.0f);
+            xv[j] = o;
+        }
+        Ld<T, VN>::store(y + r * py + c0, xv);
+    }
+}
+
+// Pass 1 of training forward: per-block partial sums of (x-K) and (x-K)^2, K = x[row 0].
+template <typename T, int VN>
+__global__ void __launch_bounds__(256)
+    bn_stats_cl(const T *__restrict__ x, int64_t px, float *__restrict__ partial, int64_t rows, int C, int cvb)
+{
+    __shared__ float red[256 * VN * 2];
+    const int tx = threadIdx.x % cvb, ty = threadIdx.x / cvb, rb = 256 / cvb;
+    const int c0 = (blockIdx.y * cvb + tx) * VN;
+    float a0[VN], a1[VN], k[VN];
+#pragma unroll
+    for(int j = 0; j < VN; j++)
+        a0[j] = a1[j] = 0.0f;
+    if(c0 < C) {
+        Ld<T, VN>::load(x + c0, k);
+        for(int64_t r = (int64_t)blockIdx.x * rb + ty; r < rows; r += (int64_t)gridDim.x * rb) {
+            float xv[VN];
+            Ld<T, VN>::load(x + r * px + c0, xv);
+#pragma unroll
+            for(int j = 0; j < VN; j++) {
+                const float d = xv[j] - k[j];
+                a0[j] += d;
+                a1[j] += d * d;
+            }
+        }
+    }
+#pragma unroll
+    for(int j = 0; j < VN; j++) {
+        red[(ty * cvb + tx) * VN * 2 + j] = a0[j];
+        red[(ty * cvb + tx) * VN * 2 + VN + j] = a1[j];
+    }
+    __syncthreads();
+    if(ty == 0 && c0 < C) {
+        for(int t = 1; t < rb; t++) {
+#pragma unroll
+            for(int j = 0; j < VN; j++) {
+                a0[j] += red[(t * cvb + tx) * VN * 2 + j];
+                a1[j] += red[(t * cvb + tx) * VN * 2 + VN + j];
+            }
+        }
+        float *o = partial + ((int64_t)blockIdx.x * C + c0) * 2;
+#pragma unroll
+        for(int j = 0; j < VN; j++) {
+            o[j * 2] = a0[j];
+            o[j * 2 + 1] = a1[j];
+        }
+    }
+}
+
+// Finalize: mean, biased variance, invstd, running statistics, fused scale/shift.
+template <typename T>
+__global__ void __launch_bounds__(256)
+    bn_stats_finalize(const float *__restrict__ partial, int gx, const T *__restrict__ xrow0, int64_t kstride,
+                      const float *__restrict__ s, const float *__restrict__ b, float *run_m, float *run_v,
+                      float *save_mean, float *save_invstd, float *ss, double M, int C, float eps, float expavg)
+{
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if(c >= C)
+        return;
+    double s0 = 0, s1 = 0;
+    for(int g = 0; g < gx; g++) {
+        s0 += partial[((int64_t)g * C + c) * 2];
+        s1 += partial[((int64_t)g * C + c) * 2 + 1];
+    }
+    const double k = (double)(float)xrow0[c * kstride];
+    const double dm = s0 / M;
+    double var = s1 / M - dm * dm;
+    if(var < 0)
+        var = 0;
+    const double mean = k + dm;
+    const float inv = (float)(1.0 / sqrt(var + (double)eps));
+    if(save_mean)
+        save_mean[c] = (float)mean;
+    if(save_invstd)
+        save_invstd[c] = inv;
+    if(run_m)
+        run_m[c] = (float)((1.0 - expavg) * run_m[c] + expavg * mean);
+    if(run_v) {
+        const double unb = M > 1 ? var * M / (M - 1.0) : var;
+        run_v[c] = (float)((1.0 - expavg) * run_v[c] + expavg * unb);
+    }
+    const float sc = s[c] * inv;
+    ss[c] = sc;
+    ss[C + c] = b[c] - (float)mean * sc;
+}
+
+// Pass 1 of backward: partial sums of dy' and dy'*(x-mean); dy' = dy masked by y>0 when fused relu.
+template <typename T, int VN>
+__global__ void __launch_bounds__(256)
+    bn_bwd_stats_cl(const T *__restrict__ x, int64_t px, const T *__restrict__ y, int64_t py, const T *__restrict__ dy,
+                    int64_t pdy, const float *__restrict__ save_mean, float *__restrict__ partial, int64_t rows, int C,
+                    int cvb, int flags)
+{
+    __shared__ float red[256 * VN * 2];
+    const int tx = threadIdx.x % cvb, ty = threadIdx.x / cvb, rb = 256 / cvb;
+    const int c0 = (blockIdx.y * cvb + tx) * VN;
+    const bool relu = flags & SAGA_BN_RELU;
+    float a0[VN], a1[VN], mean[VN];
+#pragma unroll
+    for(int j = 0; j < VN; j++)
+        a0[j] = a1[j] = 0.0f;
+    if(c0 < C) {
+#pragma unroll
+        for(int j = 0; j < VN; j++)
+            mean[j] = save_mean[c0 + j];
+        for(int64_t r = (int64_t)blockIdx.x * rb + ty; r < rows; r += (int64_t)gridDim.x * rb) {
+            float xv[VN], gv[VN], yv[VN];
+            Ld<T, VN>::load(x + r * px + c0, xv);
+            Ld<T, VN>::load(dy + r * pdy + c0, gv);
+            if(relu)
+                Ld<T, VN>::load(y + r * py + c0, yv);
+#pragma unroll
+            for(int j = 0; j < VN; j++) {
+                float g = gv[j];
+                if(relu && !(yv[j] > 0.0f))
+                    g = 0.0f;
+                a0[j] += g;
+                a1[j] += g * (xv[j] - mean[j]);
+            }
+        }
+    }
+#pragma unroll
+    for(int j = 0; j < VN; j++) {
+        red[(ty * cvb + tx) * VN * 2 + j] = a0[j];
+        red[(ty * cvb + tx) * VN * 2 + VN + j] = a1[j];
+    }
+    __syncthreads();
+    if(ty == 0 && c0 < C) {
+        for(int t = 1; t < rb; t++) {
+#pragma unroll
+            for(int j = 0; j < VN; j++) {
+                a0[j] += red[(t * cvb + tx) * VN * 2 + j];
+                a1[j] += red[(t * cvb + tx) * VN * 2 + VN + j];
+            }
+        }
+        float *o = partial + ((int64_t)blockIdx.x * C + c0) * 2;
+#pragma unroll
+        for(int j = 0; j < VN; j++) {
+            o[j * 2] = a0[j];
+            o[j * 2 + 1] = a1[j];
+        }
+    }
+}
+
+// coef[0..C) = s*invstd ; coef[C..2C) = db/M ; coef[2C..3C) = ds*invstd/M ; writes ds, db.
+__global__ void __launch_bounds__(256)
+    bn_bwd_finalize(const float *__restrict__ partial, int gx, const float *__restrict__ s,
+                    const float *__restrict__ save_invstd, float *ds, float *db, float *coef, double M, int C,
+                    float beta_p)
+{
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if(c >= C)
+        return;
+    double s0 = 0, s1 = 0;
+    for(int g = 0; g < gx; g++) {
+        s0 += partial[((int64_t)g * C + c) * 2];
+        s1 += partial[((int64_t)g * C + c) * 2 + 1];
+    }
+    const double inv = save_invstd[c];
+    const double dsv = s1 * inv;
+    ds[c] = (float)(beta_p != 0.0f ? dsv + (double)beta_p * ds[c] : dsv);
+    db[c] = (float)(beta_p != 0.0f ? s0 + (double)beta_p * db[c] : s0);
+    coef[c] = (float)(s[c] * inv);
+    coef[C + c] = (float)(s0 / M);
+    coef[2 * C + c] = (float)(dsv * inv / M);
+}
+
+// Pass 2 of backward: dx = s*invstd*(dy' - db/M - (x-mean)*invstd*ds/M) ; dz = dy'.
+template <typename T, int VN>
+__global__ void __launch_bounds__(256)
+    bn_bwd_apply_cl(const T *__restrict__ x, int64_t px, const T *__restrict__ y, int64_t py, const T *__restrict__ dy,
+                    int64_t pdy, T *__restrict__ dx, int64_t pdx, T *__restrict__ dz, int64_t pdz,
+                    const float *__restrict__ save_mean, const float *__restrict__ coef, int64_t rows, int C, int cvb,
+                    int flags, float beta_dx, float beta_dz)
+{
+    const int tx = threadIdx.x % cvb, ty = threadIdx.x / cvb, rb = 256 / cvb;
+    const int c0 = (blockIdx.y * cvb + tx) * VN;
+    if(c0 >= C)
+        return;
+    const bool relu = flags & SAGA_BN_RELU;
+    float mean[VN], a[VN], k0[VN], k1[VN];
+#pragma unroll
+    for(int j = 0; j < VN; j++) {
+        mean[j] = save_mean[c0 + j];
+        a[j] = coef[c0 + j];
+        k0[j] = coef[C + c0 + j];
+        k1[j] = coef[2 * C + c0 + j];
+    }
+    for(int64_t r = (int64_t)blockIdx.x * rb + ty; r < rows; r += (int64_t)gridDim.x * rb) {
+        float xv[VN], gv[VN], yv[VN], ov[VN];
+        Ld<T, VN>::load(x + r * px + c0, xv);
+        Ld<T, VN>::load(dy + r * pdy + c0, gv);
+        if(relu) {
+            Ld<T, VN>::load(y + r * py + c0, yv);
+#pragma unroll
+            for(int j = 0; j < VN; j++)
+                if(!(yv[j] > 0.0f))
+                    gv[j] = 0.0f;
+        }
+        if(beta_dx != 0.0f)
+            Ld<T, VN>::load(dx + r * pdx + c0, ov);
+#pragma unroll
+        for(int j = 0; j < VN; j++) {
+            const float v = a[j] * (gv[j] - k0[j] - (xv[j] - mean[j]) * k1[j]);
+            xv[j] = beta_dx != 0.0f ? v + beta_dx * ov[j] : v;
+        }
+        Ld<T, VN>::store(dx + r * pdx + c0, xv);
+        if(dz) {
+            if(beta_dz != 0.0f) {
+                Ld<T, VN>::load(dz + r * pdz + c0, ov);
+#pragma unroll
+                for(int j = 0; j < VN; j++)
+                    gv[j] += beta_dz * ov[j];
+            }
+            Ld<T, VN>::store(dz + r * pdz + c0, gv);
+        }
+    }
+}
+
+// ---------------------------------------------------------------- channels-first kernels
+// One block per channel; HW runs are contiguous, lanes stride along them.
+
+template <typename T> __device__ __forceinline__ void block_sum2(float &a, float &b)
+{
+    __shared__ float red[2][4];
+    a = wave_sum(a);
+    b = wave_sum(b);
+    __syncthreads();
+    if((threadIdx.x & 63) == 0) {
+        red[0][threadIdx.x >> 6] = a;
+        red[1][threadIdx.x >> 6] = b;
+    }
+    __syncthreads();
+    a = red[0][0] + red[0][1] + red[0][2] + red[0][3];
+    b = red[1][0] + red[1][1] + red[1][2] + red[1][3];
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+    bn_stats_cf(const T *__restrict__ x, int64_t npitch, int N, int C, int64_t HW, const float *__restrict__ s,
+                const float *__restrict__ b, float *run_m, float *run_v, float *save_mean, float *save_invstd,
+                float *ss, float eps, float expavg)
+{
+    const int c = blockIdx.x;
+    const float k = (float)x[(int64_t)c * HW];
+    float a0 = 0, a1 = 0;
+    for(int n = 0; n < N; n++) {
+        const T *p = x + n * npitch + (int64_t)c * HW;
+        for(int64_t i = threadIdx.x; i < HW; i += 256) {
+            const float d = (float)p[i] - k;
+            a0 += d;
+            a1 += d * d;
+        }
+    }
+    block_sum2<T>(a0, a1);
+    if(threadIdx.x == 0) {
+        const double M = (double)N * HW;
+        const double dm = a0 / M;
+        double var = a1 / M - dm * dm;
+        if(var < 0)
+            var = 0;
+        const double mean = k + dm;
+        const float inv = (float)(1.0 / sqrt(var + (double)eps));
+        if(save_mean)
+            save_mean[c] = (float)mean;
+        if(save_invstd)
+            save_invstd[c] = inv;
+        if(run_m)
+            run_m[c] = (float)((1.0 - expavg) * run_m[c] + expavg * mean);
+        if(run_v) {
+            const double unb = M > 1 ? var * M / (M - 1.0) : var;
+            run_v[c] = (float)((1.0 - expavg) * run_v[c] + expavg * unb);
+        }
+        const float sc = s[c] * inv;
+        ss[c] = sc;
+        ss[C + c] = b[c] - (float)mean * sc;
+    }
+}
+
+template <typename T, int MODE>
+__global__ void __launch_bounds__(256)
+    bn_apply_cf(const T *__restrict__ x, int64_t npx, const T *__restrict__ z, int64_t npz, T *__restrict__ y,
+                int64_t npy, const float *__restrict__ s, const float *__restrict__ b, const float *__restrict__ m,
+                const float *__restrict__ v, const float *__restrict__ ss, float eps, int N, int C, int64_t HW,
+                int flags)
+{
+    const int64_t total = (int64_t)N * C * HW;
+    const bool relu = flags & SAGA_BN_RELU, add = flags & SAGA_BN_ADD;
+    for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t nc = i / HW, hw = i - nc * HW;
+        const int c = (int)(nc % C);
+        const int64_t n = nc / C;
+        float sc, sh;
+        if(MODE == 0) {
+            sc = s[c] * rsqrtf(v[c] + eps);
+            sh = b[c] - m[c] * sc;
+        } else {
+            sc = ss[c];
+            sh = ss[C + c];
+        }
+        float o = (float)x[n * npx + (int64_t)c * HW + hw] * sc + sh;
+        if(add)
+            o += (float)z[n * npz + (int64_t)c * HW + hw];
+        if(relu)
+            o = (o != o) ? o : fmaxf(o, 0.0f);
+        y[n * npy + (int64_t)c * HW + hw] = (T)o;
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+    bn_bwd_cf(const T *__restrict__ x, int64_t npx, const T *__restrict__ y, int64_t npy, const T *__restrict__ dy,
+              int64_t npdy, T *__restrict__ dx, int64_t npdx, T *__restrict__ dz, int64_t npdz,
+              const float *__restrict__ s, const float *__restrict__ save_mean, const float *__restrict__ save_invstd,
+              float *ds, float *db, int N, int C, int64_t HW, int flags, float beta_dx, float beta_dz, float beta_p)
+{
+    const int c = blockIdx.x;
+    const bool relu = flags & SAGA_BN_RELU;
+    const float mean = save_mean[c], inv = save_invstd[c];
+    float a0 = 0, a1 = 0;
+    for(int n = 0; n < N; n++) {
+        const int64_t o = (int64_t)c * HW;
+        for(int64_t i = threadIdx.x; i < HW; i += 256) {
+            float g = (float)dy[n * npdy + o + i];
+            if(relu && !((float)y[n * npy + o + i] > 0.0f))
+                g = 0.0f;
+            a0 += g;
+            a1 += g * ((float)x[n * npx + o + i] - mean);
+        }
+    }
+    block_sum2<T>(a0, a1);
+    const double M = (double)N * HW;
+    const float dsv = a1 * inv;
+    const float a = s[c] * inv, k0 = (float)(a0 / M), k1 = (float)(dsv * inv / M);
+    for(int n = 0; n < N; n++) {
+        const int64_t o = (int64_t)c * HW;
+        for(int64_t i = threadIdx.x; i < HW; i += 256) {
+            float g = (float)dy[n * npdy + o + i];
+            if(relu && !((float)y[n * npy + o + i] > 0.0f))
+                g = 0.0f;
+            const float v = a * (g - k0 - ((float)x[n * npx + o + i] - mean) * k1);
+            T *pd = dx + n * npdx + o + i;
+            *pd = (T)(beta_dx != 0.0f ? v + beta_dx * (float)*pd : v);
+            if(dz) {
+                T *pz = dz + n * npdz + o + i;
+                *pz = (T)(beta_dz != 0.0f ? g + beta_dz * (float)*pz : g);
+            }
+        }
+    }
+    if(threadIdx.x == 0) {
+        ds[c] = beta_p != 0.0f ? dsv + beta_p * ds[c] : dsv;
+        db[c] = beta_p != 0.0f ? a0 + beta_p * db[c] : a0;
+    }
+}
+
+// ---------------------------------------------------------------- host side
+
+struct Views {
+    bool cl;
+    CLInfo lx, ly, lz, ldy, ldx, ldz;
+    CFInfo fx, fy, fz, fdy, fdx, fdz;
+};
+
+static int vec_width(int dtype, int C, std::initializer_list<const SagaTensorView *> vs,
+                     std::initializer_list<int64_t> pitches)
+{
+    const int vn = dtype == SAGA_HALF ? 8 : 4;
+    if(C % vn)
+        return 1;
+    for(auto v : vs)
+        if(v && !aligned16(v->ptr))
+            return 1;
+    for(auto p : pitches)
+        if(p % vn)
+            return 1;
+    return vn;
+}
+
+static size_t ws_floats(int64_t rows, int C, int dtype)
+{
+    // partials for the widest plan (vector width 1 gives the most blocks along y) + 3*C coefficients
+    size_t best = 0;
+    for(int vn : {1, dtype == SAGA_HALF ? 8 : 4}) {
+        if(C % vn)
+            continue;
+        Shape sh = plan(rows, C / vn);
+        size_t need = (size_t)sh.gx * C * 2;
+        if(need > best)
+            best = need;
+    }
+    return best + 3 * (size_t)C + 64;
+}
+
+} // namespace
+
+extern "C" {
+
+size_t saga_hip_bn_workspace_size(const SagaTensorView *x)
+{
+    if(!x)
+        return 0;
+    const int64_t rows = (int64_t)x->dims[0] * x->dims[2] * x->dims[3];
+    return ws_floats(rows, x->dims[1], x->dtype) * sizeof(float);
+}
+
+int saga_hip_bn_infer(const SagaTensorView *x, const SagaTensorView *z, const SagaTensorView *y, const float *s,
+                      const float *b, const float *m, const float *v, float eps, int flags, saga_stream_t stream)
+{
+    if(!valid_view(x) || !valid_view(y) || !s || !b || !m || !v)
+        return SAGA_HIP_EINVAL;
+    const bool add = flags & SAGA_BN_ADD;
+    if(add && !valid_view(z))
+        return SAGA_HIP_EINVAL;
+    if(!same_dims(x, y) || (add && !same_dims(x, z)))
+        return SAGA_HIP_ESHAPE;
+    if(x->dtype != y->dtype || (add && z->dtype != x->dtype) || (x->dtype != SAGA_HALF && x->dtype != SAGA_FLOAT))
+        return SAGA_HIP_EUNSUPPORTED;
+    hipStream_t st = as_stream(stream);
+    CLInfo lx, ly, lz = {};
+    CFInfo fx, fy, fz = {};
+    if(as_channels_last(x, &lx) && as_channels_last(y, &ly) && (!add || as_channels_last(z, &lz))) {
+        const int vn = vec_width(x->dtype, lx.C, {x, y, add ? z : nullptr}, {lx.pitch, ly.pitch, add ? lz.pitch : 0});
+        Shape sh = plan(lx.rows, lx.C / vn);
+        dim3 grid(sh.gx, sh.gy);
+#define GO(T, VN)                                                                                                 \
+    bn_apply_cl<T, VN, 0><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, add ? (const T *)z->ptr : nullptr,      \
+                                                lz.pitch, (T *)y->ptr, ly.pitch, s, b, m, v, nullptr, eps, lx.rows, \
+                                                lx.C, sh.cvb, flags)
+        if(x->dtype == SAGA_HALF) {
+            if(vn == 8) GO(half_t, 8); else GO(half_t, 1);
+        } else {
+            if(vn == 4) GO(float, 4); else GO(float, 1);
+        }
+#undef GO
+    } else if(as_channels_first(x, &fx) && as_channels_first(y, &fy) && (!add || as_channels_first(z, &fz))) {
+        const int64_t total = (int64_t)fx.N * fx.C * fx.HW;
+        const int g = grid_for(total, 256, 256 * 32);
+        if(x->dtype == SAGA_HALF)
+            bn_apply_cf<half_t, 0><<<g, 256, 0, st>>>((const half_t *)x->ptr, fx.npitch,
+                                                      add ? (const half_t *)z->ptr : nullptr, fz.npitch,
+                                                      (half_t *)y->ptr, fy.npitch, s, b, m, v, nullptr, eps, fx.N,
+                                                      fx.C, fx.HW, flags);
+        else
+            bn_apply_cf<float, 0><<<g, 256, 0, st>>>((const float *)x->ptr, fx.npitch,
+                                                     add ? (const float *)z->ptr : nullptr, fz.npitch,
+                                                     (float *)y->ptr, fy.npitch, s, b, m, v, nullptr, eps, fx.N, fx.C,
+                                                     fx.HW, flags);
+    } else {
+        return SAGA_HIP_EUNSUPPORTED;
+    }
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
+int saga_hip_bn_train_fwd(const SagaTensorView *x, const SagaTensorView *z, const SagaTensorView *y,
+                          const float *s, const float *b, float *run_m, float *run_v, float *save_mean,
+                          float *save_invstd, float eps, float expavg, int flags, void *workspace,
+                          size_t ws_bytes, saga_stream_t stream)
+{
+    if(!valid_view(x) || !valid_view(y) || !s || !b)
+        return SAGA_HIP_EINVAL;
+    const bool add = flags & SAGA_BN_ADD;
+    if(add && !valid_view(z))
+        return SAGA_HIP_EINVAL;
+    if(!same_dims(x, y) || (add && !same_dims(x, z)))
+        return SAGA_HIP_ESHAPE;
+    if(x->dtype != y->dtype || (add && z->dtype != x->dtype) || (x->dtype != SAGA_HALF && x->dtype != SAGA_FLOAT))
+        return SAGA_HIP_EUNSUPPORTED;
+    if(!workspace || ws_bytes < saga_hip_bn_workspace_size(x))
+        return SAGA_HIP_EWORKSPACE;
+    hipStream_t st = as_stream(stream);
+    float *ws = (float *)workspace;
+    CLInfo lx, ly, lz = {};
+    CFInfo fx, fy, fz = {};
+    if(as_channels_last(x, &lx) && as_channels_last(y, &ly) && (!add || as_channels_last(z, &lz))) {
+        const int C = lx.C;
+        const int vn = vec_width(x->dtype, C, {x, y, add ? z : nullptr}, {lx.pitch, ly.pitch, add ? lz.pitch : 0});
+        Shape sh = plan(lx.rows, C / vn);
+        dim3 grid(sh.gx, sh.gy);
+        float *partial = ws, *ss = ws + (size_t)sh.gx * C * 2;
+#define GO(T, VN)                                                                                                   \
+    do {                                                                                                            \
+        bn_stats_cl<T, VN><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, partial, lx.rows, C, sh.cvb);           \
+        bn_stats_finalize<T><<<(C + 255) / 256, 256, 0, st>>>(partial, sh.gx, (const T *)x->ptr, 1, s, b, run_m,      \
+                                                              run_v, save_mean, save_invstd, ss, (double)lx.rows, C, \
+                                                              eps, expavg);                                         \
+        bn_apply_cl<T, VN, 1><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, add ? (const T *)z->ptr : nullptr,   \
+                                                    lz.pitch, (T *)y->ptr, ly.pitch, nullptr, nullptr, nullptr,     \
+                                                    nullptr, ss, eps, lx.rows, C, sh.cvb, flags);                   \
+    } while(0)
+        if(x->dtype == SAGA_HALF) {
+            if(vn == 8) GO(half_t, 8); else GO(half_t, 1);
+        } else {
+            if(vn == 4) GO(float, 4); else GO(float, 1);
+        }
+#undef GO
+    } else if(as_channels_first(x, &fx) && as_channels_first(y, &fy) && (!add || as_channels_first(z, &fz))) {
+        const int C = fx.C;
+        float *ss = ws;
+        const int64_t total = (int64_t)fx.N * C * fx.HW;
+        const int g = grid_for(total, 256, 256 * 32);
+#define GO(T)                                                                                                      \
+    do {                                                                                                           \
+        bn_stats_cf<T><<<C, 256, 0, st>>>((const T *)x->ptr, fx.npitch, fx.N, C, fx.HW, s, b, run_m, run_v,          \
+                                          save_mean, save_invstd, ss, eps, expavg);                                \
+        bn_apply_cf<T, 1><<<g, 256, 0, st>>>((const T *)x->ptr, fx.npitch, add ? (const T *)z->ptr : nullptr,        \
+                                             fz.npitch, (T *)y->ptr, fy.npitch, nullptr, nullptr, nullptr, nullptr, \
+                                             ss, eps, fx.N, C, fx.HW, flags);                                      \
+    } while(0)
+        if(x->dtype == SAGA_HALF) GO(half_t); else GO(float);
+#undef GO
+    } else {
+        return SAGA_HIP_EUNSUPPORTED;
+    }
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
+int saga_hip_bn_bwd(const SagaTensorView *x, const SagaTensorView *y, const SagaTensorView *dy,
+                    const SagaTensorView *dx, const SagaTensorView *dz, const float *s, const float *save_mean,
+                    const float *save_invstd, float *ds, float *db, float beta_dx, float beta_dz, float beta_p,
+                    int flags, void *workspace, size_t ws_bytes, saga_stream_t stream)
+{
+    if(!valid_view(x) || !valid_view(dy) || !valid_view(dx) || !s || !save_mean || !save_invstd || !ds || !db)
+        return SAGA_HIP_EINVAL;
+    const bool relu = flags & SAGA_BN_RELU;
+    if(relu && !valid_view(y))
+        return SAGA_HIP_EINVAL;
+    if(dz && !valid_view(dz))
+        return SAGA_HIP_EINVAL;
+    if(!same_dims(x, dy) || !same_dims(x, dx) || (relu && !same_dims(x, y)) || (dz && !same_dims(x, dz)))
+        return SAGA_HIP_ESHAPE;
+    const int dt = x->dtype;
+    if((dt != SAGA_HALF && dt != SAGA_FLOAT) || dy->dtype != dt || dx->dtype != dt || (relu && y->dtype != dt) ||
+       (dz && dz->dtype != dt))
+        return SAGA_HIP_EUNSUPPORTED;
+    if(!workspace || ws_bytes < saga_hip_bn_workspace_size(x))
+        return SAGA_HIP_EWORKSPACE;
+    hipStream_t st = as_stream(stream);
+    float *ws = (float *)workspace;
+    CLInfo lx, ly = {}, ldy, ldx, ldz = {};
+    CFInfo fx, fy = {}, fdy, fdx, fdz = {};
+    if(as_channels_last(x, &lx) && as_channels_last(dy, &ldy) && as_channels_last(dx, &ldx) &&
+       (!relu || as_channels_last(y, &ly)) && (!dz || as_channels_last(dz, &ldz))) {
+        const int C = lx.C;
+        const int vn = vec_width(dt, C, {x, dy, dx, relu ? y : nullptr, dz},
+                                 {lx.pitch, ldy.pitch, ldx.pitch, relu ? ly.pitch : 0, dz ? ldz.pitch : 0});
+        Shape sh = plan(lx.rows, C / vn);
+        dim3 grid(sh.gx, sh.gy);
+        float *partial = ws, *coef = ws + (size_t)sh.gx * C * 2;
+#define GO(T, VN)                                                                                                    \
+    do {                                                                                                             \
+        bn_bwd_stats_cl<T, VN><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, relu ? (const T *)y->ptr : nullptr,  \
+                                                     ly.pitch, (const T *)dy->ptr, ldy.pitch, save_mean, partial,    \
+                                                     lx.rows, C, sh.cvb, flags);                                     \
+        bn_bwd_finalize<<<(C + 255) / 256, 256, 0, st>>>(partial, sh.gx, s, save_invstd, ds, db, coef,                \
+                                                         (double)lx.rows, C, beta_p);                                \
+        bn_bwd_apply_cl<T, VN><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, relu ? (const T *)y->ptr : nullptr,  \
+                                                     ly.pitch, (const T *)dy->ptr, ldy.pitch, (T *)dx->ptr,          \
+                                                     ldx.pitch, dz ? (T *)dz->ptr : nullptr, ldz.pitch, save_mean,   \
+                                                     coef, lx.rows, C, sh.cvb, flags, beta_dx, beta_dz);             \
+    } while(0)
+        if(dt == SAGA_HALF) {
+            if(vn == 8) GO(half_t, 8); else GO(half_t, 1);
+        } else {
+            if(vn == 4) GO(float, 4); else GO(float, 1);
+        }
+#undef GO
+    } else if(as_channels_first(x, &fx) && as_channels_first(dy, &fdy) && as_channels_first(dx, &fdx) &&
+              (!relu || as_channels_first(y, &fy)) && (!dz || as_channels_first(dz, &fdz))) {
+#define GO(T)                                                                                                         \
+    bn_bwd_cf<T><<<fx.C, 256, 0, st>>>((const T *)x->ptr, fx.npitch, relu ? (const T *)y->ptr : nullptr, fy.npitch,     \
+                                       (const T *)dy->ptr, fdy.npitch, (T *)dx->ptr, fdx.npitch,                      \
+                                       dz ? (T *)dz->ptr : nullptr, fdz.npitch, s, save_mean, save_invstd, ds, db,    \
+                                       fx.N, fx.C, fx.HW, flags, beta_dx, beta_dz, beta_p)
+        if(dt == SAGA_HALF) GO(half_t); else GO(float);
+#undef GO
+    } else {
+        return SAGA_HIP_EUNSUPPORTED;
+    }
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
+} // extern "C"

@@ -1,0 +1,104 @@
+// Convolution entry points: argument checking, geometry, and the choice between the MFMA
+// implicit-GEMM kernels and the direct fallback.
+#include "conv.hpp"
+
+#include <stdlib.h>
+
+namespace {
+
+static int conv_dim(int in, int k, int pad, int stride, int dil) { return 1 + (in + 2 * pad - ((k - 1) * dil + 1)) / stride; }
+
+// x: (N,C,H,W)  w: (K,C/group,R,S)  y: (N,K,P,Q)
+static int geometry(const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y, const SagaConvParams *p,
+                    ConvGeom *g)
+{
+    if(!valid_view(x) || !valid_view(w) || !valid_view(y) || !p)
+        return SAGA_HIP_EINVAL;
+    if(p->stride < 1 || p->pad < 0 || p->dilation < 1 || p->group < 1)
+        return SAGA_HIP_EINVAL;
+    g->N = x->dims[0]; g->C = x->dims[1]; g->H = x->dims[2]; g->W = x->dims[3];
+    g->K = w->dims[0]; g->R = w->dims[2]; g->S = w->dims[3];
+    g->pad = p->pad; g->stride = p->stride; g->dil = p->dilation; g->group = p->group;
+    g->P = conv_dim(g->H, g->R, g->pad, g->stride, g->dil);
+    g->Q = conv_dim(g->W, g->S, g->pad, g->stride, g->dil);
+    if(g->C % g->group || g->K % g->group || w->dims[1] != g->C / g->group)
+        return SAGA_HIP_ESHAPE;
+    if(y->dims[0] != g->N || y->dims[1] != g->K || y->dims[2] != g->P || y->dims[3] != g->Q || g->P < 1 || g->Q < 1)
+        return SAGA_HIP_ESHAPE;
+    if(x->dtype != w->dtype || x->dtype != y->dtype || (x->dtype != SAGA_HALF && x->dtype != SAGA_FLOAT))
+        return SAGA_HIP_EUNSUPPORTED;
+    return 0;
+}
+
+static bool force_direct()
+{
+    static int v = -1;
+    if(v < 0) {
+        const char *e = getenv("SAGA_HIP_FORCE_DIRECT");
+        v = (e && *e && *e != '0') ? 1 : 0;
+    }
+    return v == 1;
+}
+
+} // namespace
+
+extern "C" {
+
+size_t saga_hip_conv2d_workspace_size(int kind, const SagaTensorView *x, const SagaTensorView *w,
+                                      const SagaTensorView *y, const SagaConvParams *p)
+{
+    ConvGeom g;
+    if(geometry(x, w, y, p, &g))
+        return 0;
+    return conv_mfma_workspace(kind, x, w, y, g);
+}
+
+int saga_hip_conv2d_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y,
+                        const SagaConvParams *p, float alpha, float beta, void *workspace, size_t ws_bytes,
+                        saga_stream_t stream)
+{
+    ConvGeom g;
+    int r = geometry(x, w, y, p, &g);
+    if(r)
+        return r;
+    if(!force_direct()) {
+        r = conv_mfma_fwd(x, w, y, g, alpha, beta, workspace, ws_bytes, as_stream(stream));
+        if(r != SAGA_HIP_EUNSUPPORTED)
+            return r;
+    }
+    return conv_direct_fwd(x, w, y, g, alpha, beta, as_stream(stream));
+}
+
+int saga_hip_conv2d_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx,
+                             const SagaConvParams *p, float alpha, float beta, void *workspace, size_t ws_bytes,
+                             saga_stream_t stream)
+{
+    ConvGeom g;
+    int r = geometry(dx, w, dy, p, &g);
+    if(r)
+        return r;
+    if(!force_direct()) {
+        r = conv_mfma_bwd_data(dy, w, dx, g, alpha, beta, workspace, ws_bytes, as_stream(stream));
+        if(r != SAGA_HIP_EUNSUPPORTED)
+            return r;
+    }
+    return conv_direct_bwd_data(dy, w, dx, g, alpha, beta, as_stream(stream));
+}
+
+int saga_hip_conv2d_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, const SagaTensorView *dw,
+                               const SagaConvParams *p, float alpha, float beta, void *workspace,
+                               size_t ws_bytes, saga_stream_t stream)
+{
+    ConvGeom g;
+    int r = geometry(x, dw, dy, p, &g);
+    if(r)
+        return r;
+    if(!force_direct()) {
+        r = conv_mfma_bwd_filter(x, dy, dw, g, alpha, beta, workspace, ws_bytes, as_stream(stream));
+        if(r != SAGA_HIP_EUNSUPPORTED)
+            return r;
+    }
+    return conv_direct_bwd_filter(x, dy, dw, g, alpha, beta, as_stream(stream));
+}
+
+} // extern "C"

@@ -1,0 +1,29 @@
+// Internal interfaces between the convolution dispatcher and its kernel families.
+#pragma once
+#include "common.hpp"
+
+struct ConvGeom {
+    int N, C, H, W;    // input (x / dx)
+    int K, R, S;       // filters
+    int P, Q;          // output (y / dy)
+    int pad, stride, dil, group;
+};
+
+// Direct (non-MFMA) kernels: any dtype in {half, float}, any strides, groups, dilation.
+int conv_direct_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y, const ConvGeom &g,
+                    float alpha, float beta, hipStream_t st);
+int conv_direct_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx,
+                         const ConvGeom &g, float alpha, float beta, hipStream_t st);
+int conv_direct_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, const SagaTensorView *dw,
+                           const ConvGeom &g, float alpha, float beta, hipStream_t st);
+
+// MFMA implicit-GEMM kernels (fp16, channels-last).  Each returns SAGA_HIP_EUNSUPPORTED when the
+// problem is outside what it covers, and the dispatcher falls back to the direct kernels.
+size_t conv_mfma_workspace(int kind, const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y,
+                           const ConvGeom &g);
+int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y, const ConvGeom &g,
+                  float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st);
+int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx,
+                       const ConvGeom &g, float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st);
+int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, const SagaTensorView *dw,
+                         const ConvGeom &g, float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st);

@@ -1,0 +1,370 @@
+// Implicit-GEMM convolution on the gfx950 matrix cores (fp16 in, fp32 accumulate), for
+// channels-last activations and K,R,S,C filters.
+//
+//   forward        y[m, k]  = sum_{tap, c} x[pix(m, tap), c] * w[k, tap, c]      m = (n, p, q)
+//   backward data  dx[m, c] = sum_{tap, k} dy[pix'(m, tap), k] * wT[c, tap, k]   m = (n, h, w)
+//   backward filt  dw[k, tap, c] = sum_m dy[m, k] * x[pix(m, tap), c]
+//
+// Forward and backward-data share one kernel: a GEMM whose A operand is gathered on the fly
+// (im2col is never materialised) and whose B operand is a row-major [Ngemm][taps*Cred] matrix
+// with the reduction index contiguous - exactly the K,R,S,C filter for forward, and a
+// transposed copy (C,R,S,K) made in the workspace for backward-data.
+//
+// Tiling: 256 threads = 4 wavefronts; each wavefront owns a (TM*32) x (TN*32) patch built
+// from v_mfma_f32_32x32x16_f16 tiles; the block tile is staged through LDS in slices of
+// BK = 32 reduction elements, double buffered, with the next slice's global loads issued
+// before the current slice's MFMAs.  All global loads are 16-byte vectors along the channel
+// axis (the contiguous axis of NHWC), LDS rows are padded to 40 halfs so that the 16-byte
+// fragment reads of a wavefront spread over the banks.
+// Blocks are renumbered so that consecutive tiles land on the same XCD and share its L2.
+#include "conv.hpp"
+
+namespace {
+
+constexpr int BK = 32;        // reduction elements per LDS slice
+constexpr int LDK = BK + 8;   // padded LDS row, in halfs (80 bytes, keeps 16-byte alignment)
+
+struct GatherArgs {
+    const half_t *a;   // gathered operand (x for forward, dy for backward data)
+    const half_t *b;   // [Ngemm][taps * Cred]
+    half_t *out;       // [M][ldo]
+    int M;             // output rows = N * OH * OW
+    int Ngemm;         // output channels
+    int Cred;          // channels of the gathered tensor (reduction per tap)
+    int IH, IW;        // gathered tensor spatial size
+    int OH, OW;        // output spatial size
+    int R, S;
+    int pad, stride, dil;
+    int sshift;        // log2(stride), backward data only
+    int lda;           // row pitch of the gathered tensor (elements)
+    int ldo;           // row pitch of the output
+    float alpha, beta;
+    int nblk_n;        // number of block columns
+    int nblocks;
+};
+
+__device__ __forceinline__ int xcd_remap(int b, int nblocks)
+{
+    // hardware hands consecutive workgroup ids to the 8 XCDs round-robin; give each XCD a
+    // contiguous range of tiles instead
+    const int per = nblocks >> 3, rem = nblocks & 7;
+    const int xcd = b & 7, slot = b >> 3;
+    const int base = xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per;
+    return base + slot;
+}
+
+template <int BM, int BN, int WGM, int WGN, bool BWD>
+__global__ void __launch_bounds__(256) conv_gather_gemm(GatherArgs g)
+{
+    constexpr int WTM = BM / WGM, WTN = BN / WGN; // wavefront tile
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    constexpr int AV = BM / 64, BV = BN / 64;     // 16-byte vectors per thread per slice
+    static_assert(WGM * WGN == 4, "four wavefronts");
+    static_assert(BM % 64 == 0 && BN % 64 == 0, "tile");
+
+    __shared__ __attribute__((aligned(16))) half_t As[2][BM * LDK];
+    __shared__ __attribute__((aligned(16))) half_t Bs[2][BN * LDK];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int bid = xcd_remap(blockIdx.x, g.nblocks);
+    const int bm = bid / g.nblk_n, bn = bid - bm * g.nblk_n;
+    const int m0 = bm * BM, n0 = bn * BN;
+
+    // ---- per-thread load coordinates: vector column kv (8 halfs), rows tid/4 + 64*j
+    const int kv = (tid & 3) * 8;
+    const int lrow = tid >> 2;
+    int a_base[AV], a_y[AV], a_x[AV];
+    bool a_ok[AV];
+#pragma unroll
+    for(int j = 0; j < AV; j++) {
+        const int m = m0 + lrow + 64 * j;
+        a_ok[j] = m < g.M;
+        const int mm = a_ok[j] ? m : 0;
+        const int ox = mm % g.OW;
+        const int t = mm / g.OW;
+        const int oy = t % g.OH;
+        const int n = t / g.OH;
+        a_base[j] = n * g.IH * g.IW;
+        if(BWD) {
+            a_y[j] = oy + g.pad;
+            a_x[j] = ox + g.pad;
+        } else {
+            a_y[j] = oy * g.stride - g.pad;
+            a_x[j] = ox * g.stride - g.pad;
+        }
+    }
+    const int ktot = g.R * g.S * g.Cred;
+    int b_off[BV];
+    bool b_ok[BV];
+#pragma unroll
+    for(int j = 0; j < BV; j++) {
+        const int n = n0 + lrow + 64 * j;
+        b_ok[j] = n < g.Ngemm;
+        b_off[j] = (b_ok[j] ? n : 0) * ktot;
+    }
+
+    half8_t ra[AV], rb[BV];
+    const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    // slice iterator: tap (r, s) and channel offset c0
+    int r = 0, s = 0, c0 = 0;
+    const int csteps = (g.Cred + BK - 1) / BK;
+    const int KT = g.R * g.S * csteps;
+
+    auto load_slice = [&]() {
+        const int c = c0 + kv;
+        const bool cok = c < g.Cred;
+#pragma unroll
+        for(int j = 0; j < AV; j++) {
+            int iy, ix;
+            bool ok = a_ok[j] && cok;
+            if(BWD) {
+                const int ty = a_y[j] - r * g.dil, tx = a_x[j] - s * g.dil;
+                ok = ok && ty >= 0 && tx >= 0 && ((ty | tx) & (g.stride - 1)) == 0;
+                iy = ty >> g.sshift;
+                ix = tx >> g.sshift;
+            } else {
+                iy = a_y[j] + r * g.dil;
+                ix = a_x[j] + s * g.dil;
+                ok = ok && iy >= 0 && ix >= 0;
+            }
+            ok = ok && iy < g.IH && ix < g.IW;
+            ra[j] = zero;
+            if(ok)
+                ra[j] = *(const half8_t *)(g.a + (int64_t)(a_base[j] + iy * g.IW + ix) * g.lda + c);
+        }
+        const int kb = (r * g.S + s) * g.Cred + c;
+#pragma unroll
+        for(int j = 0; j < BV; j++) {
+            rb[j] = zero;
+            if(b_ok[j] && cok)
+                rb[j] = *(const half8_t *)(g.b + b_off[j] + kb);
+        }
+    };
+    auto advance = [&]() {
+        c0 += BK;
+        if(c0 >= g.Cred) {
+            c0 = 0;
+            if(++s == g.S) {
+                s = 0;
+                ++r;
+            }
+        }
+    };
+    auto store_slice = [&](int st) {
+#pragma unroll
+        for(int j = 0; j < AV; j++)
+            *(half8_t *)(&As[st][(lrow + 64 * j) * LDK + kv]) = ra[j];
+#pragma unroll
+        for(int j = 0; j < BV; j++)
+            *(half8_t *)(&Bs[st][(lrow + 64 * j) * LDK + kv]) = rb[j];
+    };
+
+    float16_t acc[TM][TN];
+#pragma unroll
+    for(int i = 0; i < TM; i++)
+#pragma unroll
+        for(int j = 0; j < TN; j++)
+#pragma unroll
+            for(int v = 0; v < 16; v++)
+                acc[i][j][v] = 0.0f;
+
+    const int wm = (wave / WGN) * WTM, wn = (wave % WGN) * WTN;
+    const int frow = lane & 31, fk = (lane >> 5) * 8;
+
+    load_slice();
+    store_slice(0);
+    __syncthreads();
+
+    for(int kt = 0; kt < KT; kt++) {
+        const int cur = kt & 1;
+        if(kt + 1 < KT) {
+            advance();
+            load_slice();
+        }
+#pragma unroll
+        for(int kk = 0; kk < BK; kk += 16) {
+            half8_t fa[TM], fb[TN];
+#pragma unroll
+            for(int i = 0; i < TM; i++)
+                fa[i] = *(const half8_t *)(&As[cur][(wm + i * 32 + frow) * LDK + kk + fk]);
+#pragma unroll
+            for(int j = 0; j < TN; j++)
+                fb[j] = *(const half8_t *)(&Bs[cur][(wn + j * 32 + frow) * LDK + kk + fk]);
+#pragma unroll
+            for(int i = 0; i < TM; i++)
+#pragma unroll
+                for(int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+        if(kt + 1 < KT)
+            store_slice(cur ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: accumulator element v of a 32x32 tile sits at row 8*(v/4) + 4*(lane/32) + v%4,
+    // column lane%32
+    const int ecol = lane & 31, erow = (lane >> 5) * 4;
+#pragma unroll
+    for(int i = 0; i < TM; i++) {
+#pragma unroll
+        for(int j = 0; j < TN; j++) {
+            const int n = n0 + wn + j * 32 + ecol;
+            if(n >= g.Ngemm)
+                continue;
+#pragma unroll
+            for(int v = 0; v < 16; v++) {
+                const int m = m0 + wm + i * 32 + (v >> 2) * 8 + erow + (v & 3);
+                if(m >= g.M)
+                    continue;
+                half_t *o = g.out + (int64_t)m * g.ldo + n;
+                float val = g.alpha * acc[i][j][v];
+                if(g.beta != 0.0f)
+                    val += g.beta * (float)*o;
+                *o = (half_t)val;
+            }
+        }
+    }
+}
+
+// w (K, C, R, S logical; stored K,R,S,C) -> wT stored C,R,S,K
+__global__ void __launch_bounds__(256) transpose_filter(const half_t *__restrict__ w, half_t *__restrict__ wt, int K, int C, int RS)
+{
+    const int64_t total = (int64_t)K * C * RS;
+    for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        // i enumerates the destination: (c, tap, k) with k fastest
+        const int k = (int)(i % K);
+        const int tap = (int)((i / K) % RS);
+        const int c = (int)(i / ((int64_t)K * RS));
+        wt[i] = w[((int64_t)k * RS + tap) * C + c];
+    }
+}
+
+static bool krsc_dense(const SagaTensorView *w)
+{
+    const int C = w->dims[1], R = w->dims[2], S = w->dims[3];
+    if(C > 1 && w->strides[1] != 1)
+        return false;
+    if(S > 1 && w->strides[3] != C)
+        return false;
+    if(R > 1 && w->strides[2] != (int64_t)S * C)
+        return false;
+    if(w->dims[0] > 1 && w->strides[0] != (int64_t)R * S * C)
+        return false;
+    return true;
+}
+
+static int ilog2_exact(int v)
+{
+    int s = 0;
+    while((1 << s) < v)
+        s++;
+    return (1 << s) == v ? s : -1;
+}
+
+template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
+{
+    // tile choice by output-channel count; M tiles are 128 or 256 rows
+    if(g.Ngemm > 64) {
+        constexpr int BM = 128, BN = 128;
+        g.nblk_n = (g.Ngemm + BN - 1) / BN;
+        g.nblocks = ((g.M + BM - 1) / BM) * g.nblk_n;
+        conv_gather_gemm<BM, BN, 2, 2, BWD><<<g.nblocks, 256, 0, st>>>(g);
+    } else {
+        constexpr int BM = 256, BN = 64;
+        g.nblk_n = (g.Ngemm + BN - 1) / BN;
+        g.nblocks = ((g.M + BM - 1) / BM) * g.nblk_n;
+        conv_gather_gemm<BM, BN, 4, 1, BWD><<<g.nblocks, 256, 0, st>>>(g);
+    }
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
+static bool common_ok(const SagaTensorView *act_in, const SagaTensorView *w, const SagaTensorView *act_out,
+                      const ConvGeom &g, CLInfo *li, CLInfo *lo)
+{
+    if(act_in->dtype != SAGA_HALF || g.group != 1)
+        return false;
+    if(!as_channels_last(act_in, li) || !as_channels_last(act_out, lo) || !krsc_dense(w))
+        return false;
+    if(li->C % 8 || li->pitch % 8 || !aligned16(act_in->ptr) || !aligned16(w->ptr))
+        return false;
+    // 32-bit element offsets inside the kernels
+    if(li->rows * li->pitch >= (int64_t)1 << 31 || lo->rows * lo->pitch >= (int64_t)1 << 31)
+        return false;
+    if((int64_t)g.K * g.R * g.S * g.C >= (int64_t)1 << 31)
+        return false;
+    return true;
+}
+
+} // namespace
+
+size_t conv_mfma_workspace(int kind, const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y,
+                           const ConvGeom &g)
+{
+    if(x->dtype != SAGA_HALF)
+        return 0;
+    if(kind == SAGA_CONV_BWD_DATA)
+        return (size_t)g.K * g.C * g.R * g.S * sizeof(half_t) + 256;
+    return 0;
+}
+
+int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y, const ConvGeom &g,
+                  float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st)
+{
+    CLInfo lx, ly;
+    if(!common_ok(x, w, y, g, &lx, &ly))
+        return SAGA_HIP_EUNSUPPORTED;
+    GatherArgs a;
+    a.a = (const half_t *)x->ptr;
+    a.b = (const half_t *)w->ptr;
+    a.out = (half_t *)y->ptr;
+    a.M = (int)ly.rows;
+    a.Ngemm = g.K;
+    a.Cred = g.C;
+    a.IH = g.H; a.IW = g.W; a.OH = g.P; a.OW = g.Q;
+    a.R = g.R; a.S = g.S;
+    a.pad = g.pad; a.stride = g.stride; a.dil = g.dil; a.sshift = 0;
+    a.lda = (int)lx.pitch;
+    a.ldo = (int)ly.pitch;
+    a.alpha = alpha; a.beta = beta;
+    return launch_gather<false>(a, st);
+}
+
+int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx,
+                       const ConvGeom &g, float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st)
+{
+    CLInfo ldy, ldx;
+    if(!common_ok(dy, w, dx, g, &ldy, &ldx))
+        return SAGA_HIP_EUNSUPPORTED;
+    const int sshift = ilog2_exact(g.stride);
+    if(sshift < 0)
+        return SAGA_HIP_EUNSUPPORTED;
+    const size_t need = (size_t)g.K * g.C * g.R * g.S * sizeof(half_t);
+    if(!ws || ws_bytes < need || !aligned16(ws))
+        return SAGA_HIP_EWORKSPACE;
+    half_t *wt = (half_t *)ws;
+    const int64_t total = (int64_t)g.K * g.C * g.R * g.S;
+    transpose_filter<<<grid_for(total, 256, 256 * 16), 256, 0, st>>>((const half_t *)w->ptr, wt, g.K, g.C, g.R * g.S);
+    GatherArgs a;
+    a.a = (const half_t *)dy->ptr;
+    a.b = wt;
+    a.out = (half_t *)dx->ptr;
+    a.M = (int)ldx.rows;
+    a.Ngemm = g.C;
+    a.Cred = g.K;
+    a.IH = g.P; a.IW = g.Q; a.OH = g.H; a.OW = g.W;
+    a.R = g.R; a.S = g.S;
+    a.pad = g.pad; a.stride = g.stride; a.dil = g.dil; a.sshift = sshift;
+    a.lda = (int)ldy.pitch;
+    a.ldo = (int)ldx.pitch;
+    a.alpha = alpha; a.beta = beta;
+    return launch_gather<true>(a, st);
+}
+
+int conv_mfma_bwd_filter(const SagaTensorView *, const SagaTensorView *, const SagaTensorView *, const ConvGeom &,
+                         float, float, void *, size_t, hipStream_t)
+{
+    return SAGA_HIP_EUNSUPPORTED;
+}

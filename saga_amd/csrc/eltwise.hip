@@ -1,0 +1,493 @@
+// Element-wise kernels: activations, add, axpby (transform), convert, bias add, fill.
+// All are HBM-bound: the fast paths move 16 bytes per lane per access and keep every
+// wavefront on consecutive addresses; odd layouts fall back to a strided gather.
+#include "common.hpp"
+
+namespace {
+
+// ---------------------------------------------------------------- functors (fp32 math)
+
+struct ActFwd {
+    int mode;
+    float alpha, beta;
+    __device__ float operator()(float x, float, float old) const
+    {
+        float r;
+        switch(mode) {
+        case SAGA_ACT_RELU: r = (x != x) ? x : fmaxf(x, 0.0f); break;
+        case SAGA_ACT_SIGMOID: r = 1.0f / (1.0f + __expf(-x)); break;
+        case SAGA_ACT_TANH: r = tanhf(x); break;
+        case SAGA_ACT_SWISH: r = x / (1.0f + __expf(-x)); break;
+        default: r = x > 0 ? x : x * alpha; break;
+        }
+        return beta != 0.0f ? r + beta * old : r;
+    }
+};
+
+// a = x (relu, swish, leaky) or y (sigmoid, tanh); b = dy
+struct ActBwd {
+    int mode;
+    float alpha, beta;
+    __device__ float operator()(float a, float dy, float old) const
+    {
+        float d;
+        switch(mode) {
+        case SAGA_ACT_RELU: d = a > 0 ? 1.0f : 0.0f; break;
+        case SAGA_ACT_SIGMOID: d = a * (1.0f - a); break;
+        case SAGA_ACT_TANH: d = 1.0f - a * a; break;
+        case SAGA_ACT_SWISH: {
+            const float sg = 1.0f / (1.0f + __expf(-a));
+            d = sg + a * sg * (1.0f - sg);
+            break;
+        }
+        default: d = a > 0 ? 1.0f : alpha; break;
+        }
+        const float r = d * dy;
+        return beta != 0.0f ? r + beta * old : r;
+    }
+};
+
+struct AddFn {
+    __device__ float operator()(float a, float b, float) const { return a + b; }
+};
+
+struct AxpbyFn {
+    float alpha, beta;
+    __device__ float operator()(float a, float, float old) const
+    {
+        const float r = alpha * a;
+        return beta != 0.0f ? r + beta * old : r;
+    }
+};
+
+// ---------------------------------------------------------------- kernels
+
+template <typename T> struct Vec;
+template <> struct Vec<half_t> {
+    typedef half8_t type;
+    static constexpr int n = 8;
+};
+template <> struct Vec<float> {
+    typedef float4_t type;
+    static constexpr int n = 4;
+};
+
+// Flat, dense, same layout for every operand: 16-byte vectors, grid-stride.
+template <typename T, int NIN, bool READ_OLD, typename F>
+__global__ void __launch_bounds__(256) ew_flat(T *__restrict__ out, const T *__restrict__ a, const T *__restrict__ b,
+                                               int64_t nvec, int64_t total, F f)
+{
+    typedef typename Vec<T>::type V;
+    constexpr int VN = Vec<T>::n;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += stride) {
+        V va = ((const V *)a)[i];
+        V vb = NIN > 1 ? ((const V *)b)[i] : va;
+        V vo = READ_OLD ? ((const V *)out)[i] : va;
+        V r;
+#pragma unroll
+        for(int j = 0; j < VN; j++)
+            r[j] = (T)f((float)va[j], (float)vb[j], (float)vo[j]);
+        ((V *)out)[i] = r;
+    }
+    // tail
+    const int64_t base = nvec * VN;
+    for(int64_t i = base + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const float va = (float)a[i];
+        const float vb = NIN > 1 ? (float)b[i] : va;
+        const float vo = READ_OLD ? (float)out[i] : 0.0f;
+        out[i] = (T)f(va, vb, vo);
+    }
+}
+
+// Channels-last rows with individual pitches (channel slices): vectors along C.
+template <typename T, int NIN, bool READ_OLD, typename F>
+__global__ void __launch_bounds__(256)
+    ew_rows(T *__restrict__ out, int64_t po, const T *__restrict__ a, int64_t pa, const T *__restrict__ b, int64_t pb,
+            int64_t rows, int cvec, F f)
+{
+    typedef typename Vec<T>::type V;
+    constexpr int VN = Vec<T>::n;
+    const int64_t total = rows * cvec;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int64_t r = i / cvec;
+        const int c = (int)(i - r * cvec) * VN;
+        V va = *(const V *)(a + r * pa + c);
+        V vb = NIN > 1 ? *(const V *)(b + r * pb + c) : va;
+        V vo = READ_OLD ? *(const V *)(out + r * po + c) : va;
+        V res;
+#pragma unroll
+        for(int j = 0; j < VN; j++)
+            res[j] = (T)f((float)va[j], (float)vb[j], (float)vo[j]);
+        *(V *)(out + r * po + c) = res;
+    }
+}
+
+// Anything else: one element per lane, addresses from the 4-D strides.  `cl` selects the
+// decode order so that neighbouring lanes are neighbours in the output's memory.
+template <typename TO, typename TA, typename TB, int NIN, bool READ_OLD, typename F>
+__global__ void __launch_bounds__(256) ew_strided(DView out, DView a, DView b, int64_t total, int cl, F f)
+{
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    const int N = out.d[0], C = out.d[1], H = out.d[2], W = out.d[3];
+    (void)N;
+    for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        int n, c, h, w;
+        int64_t t = i;
+        if(cl) {
+            c = (int)(t % C);
+            t /= C;
+            w = (int)(t % W);
+            t /= W;
+            h = (int)(t % H);
+            n = (int)(t / H);
+        } else {
+            w = (int)(t % W);
+            t /= W;
+            h = (int)(t % H);
+            t /= H;
+            c = (int)(t % C);
+            n = (int)(t / C);
+        }
+        const int64_t oa = n * a.s[0] + c * a.s[1] + h * a.s[2] + w * a.s[3];
+        const int64_t oo = n * out.s[0] + c * out.s[1] + h * out.s[2] + w * out.s[3];
+        const float va = (float)((const TA *)a.ptr)[oa];
+        float vb = va;
+        if(NIN > 1) {
+            const int64_t ob = n * b.s[0] + c * b.s[1] + h * b.s[2] + w * b.s[3];
+            vb = (float)((const TB *)b.ptr)[ob];
+        }
+        TO *po = (TO *)out.ptr + oo;
+        const float vo = READ_OLD ? (float)*po : 0.0f;
+        *po = (TO)f(va, vb, vo);
+    }
+}
+
+static bool same_strides(const SagaTensorView *a, const SagaTensorView *b)
+{
+    for(int i = 0; i < 4; i++)
+        if(a->dims[i] > 1 && a->strides[i] != b->strides[i])
+            return false;
+    return true;
+}
+
+static bool dense(const SagaTensorView *v)
+{
+    CLInfo cl;
+    CFInfo cf;
+    if(as_channels_last(v, &cl) && cl.pitch == cl.C)
+        return true;
+    if(as_channels_first(v, &cf) && cf.npitch == (int64_t)cf.C * cf.HW)
+        return true;
+    return false;
+}
+
+// Dispatch for same-dtype unary / binary element-wise ops.
+template <typename T, int NIN, bool READ_OLD, typename F>
+int launch_ew_t(const SagaTensorView *out, const SagaTensorView *a, const SagaTensorView *b, F f, hipStream_t st)
+{
+    const int64_t total = view_elements(out);
+    constexpr int VN = Vec<T>::n;
+    const bool al = aligned16(out->ptr) && aligned16(a->ptr) && (NIN < 2 || aligned16(b->ptr));
+    if(dense(out) && same_strides(out, a) && (NIN < 2 || same_strides(out, b)) && al) {
+        const int64_t nvec = total / VN;
+        ew_flat<T, NIN, READ_OLD, F><<<grid_for(nvec ? nvec : 1, 256, 256 * 16), 256, 0, st>>>(
+            (T *)out->ptr, (const T *)a->ptr, (const T *)(NIN > 1 ? b->ptr : a->ptr), nvec, total, f);
+        SAGA_CHECK_LAUNCH();
+        return 0;
+    }
+    CLInfo co, ca, cb;
+    if(al && as_channels_last(out, &co) && as_channels_last(a, &ca) && (NIN < 2 || as_channels_last(b, &cb)) &&
+       co.C % VN == 0 && co.pitch % VN == 0 && ca.pitch % VN == 0 && (NIN < 2 || cb.pitch % VN == 0)) {
+        const int cvec = co.C / VN;
+        ew_rows<T, NIN, READ_OLD, F><<<grid_for(co.rows * cvec, 256, 256 * 16), 256, 0, st>>>(
+            (T *)out->ptr, co.pitch, (const T *)a->ptr, ca.pitch, (const T *)(NIN > 1 ? b->ptr : a->ptr),
+            NIN > 1 ? cb.pitch : ca.pitch, co.rows, cvec, f);
+        SAGA_CHECK_LAUNCH();
+        return 0;
+    }
+    const int cl = (out->dims[1] == 1 || out->strides[1] == 1) ? 1 : 0;
+    ew_strided<T, T, T, NIN, READ_OLD, F><<<grid_for(total, 256, 256 * 32), 256, 0, st>>>(
+        dview(out), dview(a), dview(NIN > 1 ? b : a), total, cl, f);
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
+template <int NIN, typename F>
+int launch_ew(const SagaTensorView *out, const SagaTensorView *a, const SagaTensorView *b, bool read_old, F f,
+              hipStream_t st)
+{
+    if(!valid_view(out) || !valid_view(a) || (NIN > 1 && !valid_view(b)))
+        return SAGA_HIP_EINVAL;
+    if(!same_dims(out, a) || (NIN > 1 && !same_dims(out, b)))
+        return SAGA_HIP_ESHAPE;
+    if(out->dtype != a->dtype || (NIN > 1 && out->dtype != b->dtype))
+        return SAGA_HIP_EUNSUPPORTED;
+    if(out->dtype == SAGA_HALF)
+        return read_old ? launch_ew_t<half_t, NIN, true, F>(out, a, b, f, st)
+                        : launch_ew_t<half_t, NIN, false, F>(out, a, b, f, st);
+    if(out->dtype == SAGA_FLOAT)
+        return read_old ? launch_ew_t<float, NIN, true, F>(out, a, b, f, st)
+                        : launch_ew_t<float, NIN, false, F>(out, a, b, f, st);
+    return SAGA_HIP_EUNSUPPORTED;
+}
+
+struct ScaleFn {
+    float scale;
+    __device__ float operator()(float a, float, float) const { return a * scale; }
+};
+
+template <typename TS, typename TD>
+int launch_convert(const SagaTensorView *src, const SagaTensorView *dst, float scale, hipStream_t st)
+{
+    const int64_t total = view_elements(dst);
+    const int cl = (dst->dims[1] == 1 || dst->strides[1] == 1) ? 1 : 0;
+    ew_strided<TD, TS, TS, 1, false, ScaleFn><<<grid_for(total, 256, 256 * 32), 256, 0, st>>>(
+        dview(dst), dview(src), dview(src), total, cl, ScaleFn{scale});
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
+// y[row, c] += b[c] on channels-last rows.
+template <typename T, typename TB>
+__global__ void __launch_bounds__(256) bias_add_cl(T *y, int64_t pitch, const TB *b, int64_t rows, int C)
+{
+    const int64_t total = rows * C;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int64_t r = i / C;
+        const int c = (int)(i - r * C);
+        T *p = y + r * pitch + c;
+        *p = (T)((float)*p + (float)b[c]);
+    }
+}
+
+template <typename T, typename TB>
+__global__ void __launch_bounds__(256) bias_add_cf(T *y, int64_t npitch, const TB *b, int N, int C, int64_t HW)
+{
+    const int64_t total = (int64_t)N * C * HW;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int64_t nc = i / HW;
+        const int c = (int)(nc % C);
+        const int64_t n = nc / C;
+        T *p = y + n * npitch + (int64_t)c * HW + (i - nc * HW);
+        *p = (T)((float)*p + (float)b[c]);
+    }
+}
+
+// db[c] = beta*db[c] + sum over rows, channels-last: one block handles 64 channels x all rows
+// striped over 4 waves; lanes read consecutive channels.
+template <typename T, typename TB>
+__global__ void __launch_bounds__(256) bias_bwd_cl(const T *dy, int64_t pitch, TB *db, int64_t rows, int C, float beta)
+{
+    __shared__ float part[4][64];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int c = blockIdx.x * 64 + lane;
+    float acc = 0;
+    if(c < C)
+        for(int64_t r = wv; r < rows; r += 4)
+            acc += (float)dy[r * pitch + c];
+    part[wv][lane] = acc;
+    __syncthreads();
+    if(wv == 0 && c < C) {
+        const float s = part[0][lane] + part[1][lane] + part[2][lane] + part[3][lane];
+        db[c] = (TB)(beta != 0.0f ? s + beta * (float)db[c] : s);
+    }
+}
+
+template <typename T, typename TB>
+__global__ void __launch_bounds__(256) bias_bwd_cf(const T *dy, int64_t npitch, TB *db, int N, int C, int64_t HW, float beta)
+{
+    __shared__ float part[4];
+    const int c = blockIdx.x;
+    float acc = 0;
+    for(int n = 0; n < N; n++) {
+        const T *p = dy + n * npitch + (int64_t)c * HW;
+        for(int64_t i = threadIdx.x; i < HW; i += 256)
+            acc += (float)p[i];
+    }
+    acc = wave_sum(acc);
+    if((threadIdx.x & 63) == 0)
+        part[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if(threadIdx.x == 0) {
+        const float s = part[0] + part[1] + part[2] + part[3];
+        db[c] = (TB)(beta != 0.0f ? s + beta * (float)db[c] : s);
+    }
+}
+
+__global__ void __launch_bounds__(256) fill_bytes(uint8_t *p, uint8_t v, size_t n)
+{
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const size_t i0 = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t v4 = v * 0x01010101u;
+    const size_t head = (size_t)((16 - ((uintptr_t)p & 15)) & 15);
+    const size_t h = head < n ? head : n;
+    for(size_t i = i0; i < h; i += stride)
+        p[i] = v;
+    uint4 *q = (uint4 *)(p + h);
+    const size_t nv = (n - h) / 16;
+    for(size_t i = i0; i < nv; i += stride)
+        q[i] = make_uint4(v4, v4, v4, v4);
+    for(size_t i = h + nv * 16 + i0; i < n; i += stride)
+        p[i] = v;
+}
+
+} // namespace
+
+extern "C" {
+
+int saga_hip_act_fwd(int mode, float alpha, const SagaTensorView *x, const SagaTensorView *y, float beta,
+                     saga_stream_t stream)
+{
+    if(mode < SAGA_ACT_RELU || mode > SAGA_ACT_LEAKYRELU)
+        return SAGA_HIP_EINVAL;
+    return launch_ew<1>(y, x, nullptr, beta != 0.0f, ActFwd{mode, alpha, beta}, as_stream(stream));
+}
+
+int saga_hip_act_bwd(int mode, float alpha, const SagaTensorView *x, const SagaTensorView *y,
+                     const SagaTensorView *dy, const SagaTensorView *dx, float beta, saga_stream_t stream)
+{
+    if(mode < SAGA_ACT_RELU || mode > SAGA_ACT_LEAKYRELU)
+        return SAGA_HIP_EINVAL;
+    const bool uses_y = mode == SAGA_ACT_SIGMOID || mode == SAGA_ACT_TANH;
+    const SagaTensorView *a = uses_y ? y : x;
+    return launch_ew<2>(dx, a, dy, beta != 0.0f, ActBwd{mode, alpha, beta}, as_stream(stream));
+}
+
+int saga_hip_add(const SagaTensorView *a, const SagaTensorView *b, const SagaTensorView *y, saga_stream_t stream)
+{
+    return launch_ew<2>(y, a, b, false, AddFn{}, as_stream(stream));
+}
+
+int saga_hip_axpby(const SagaTensorView *src, const SagaTensorView *dst, float alpha, float beta,
+                   saga_stream_t stream)
+{
+    return launch_ew<1>(dst, src, nullptr, beta != 0.0f, AxpbyFn{alpha, beta}, as_stream(stream));
+}
+
+int saga_hip_convert(const SagaTensorView *src, const SagaTensorView *dst, float scale, saga_stream_t stream)
+{
+    if(!valid_view(src) || !valid_view(dst))
+        return SAGA_HIP_EINVAL;
+    if(!same_dims(src, dst))
+        return SAGA_HIP_ESHAPE;
+    hipStream_t st = as_stream(stream);
+    const int s = src->dtype, d = dst->dtype;
+    if(s == d && (s == SAGA_HALF || s == SAGA_FLOAT))
+        return saga_hip_axpby(src, dst, scale, 0.0f, stream);
+    if(s == SAGA_U8 && d == SAGA_FLOAT) return launch_convert<uint8_t, float>(src, dst, scale, st);
+    if(s == SAGA_U8 && d == SAGA_HALF) return launch_convert<uint8_t, half_t>(src, dst, scale, st);
+    if(s == SAGA_I16 && d == SAGA_HALF) return launch_convert<int16_t, half_t>(src, dst, scale, st);
+    if(s == SAGA_I16 && d == SAGA_FLOAT) return launch_convert<int16_t, float>(src, dst, scale, st);
+    if(s == SAGA_FLOAT && d == SAGA_HALF) return launch_convert<float, half_t>(src, dst, scale, st);
+    if(s == SAGA_HALF && d == SAGA_FLOAT) return launch_convert<half_t, float>(src, dst, scale, st);
+    return SAGA_HIP_EUNSUPPORTED;
+}
+
+int saga_hip_bias_add(const SagaTensorView *y, const SagaTensorView *b, saga_stream_t stream)
+{
+    if(!valid_view(y) || !valid_view(b))
+        return SAGA_HIP_EINVAL;
+    if(view_elements(b) != y->dims[1])
+        return SAGA_HIP_ESHAPE;
+    hipStream_t st = as_stream(stream);
+    const int64_t total = view_elements(y);
+    CLInfo cl;
+    CFInfo cf;
+#define BIAS_ADD(T, TB)                                                                                       \
+    if(as_channels_last(y, &cl))                                                                              \
+        bias_add_cl<T, TB><<<grid_for(total, 256, 256 * 32), 256, 0, st>>>((T *)y->ptr, cl.pitch,               \
+                                                                           (const TB *)b->ptr, cl.rows, cl.C); \
+    else if(as_channels_first(y, &cf))                                                                        \
+        bias_add_cf<T, TB><<<grid_for(total, 256, 256 * 32), 256, 0, st>>>((T *)y->ptr, cf.npitch,              \
+                                                                           (const TB *)b->ptr, cf.N, cf.C, cf.HW); \
+    else                                                                                                      \
+        return SAGA_HIP_EUNSUPPORTED;
+    if(y->dtype == SAGA_HALF && b->dtype == SAGA_HALF) {
+        BIAS_ADD(half_t, half_t)
+    } else if(y->dtype == SAGA_HALF && b->dtype == SAGA_FLOAT) {
+        BIAS_ADD(half_t, float)
+    } else if(y->dtype == SAGA_FLOAT && b->dtype == SAGA_FLOAT) {
+        BIAS_ADD(float, float)
+    } else
+        return SAGA_HIP_EUNSUPPORTED;
+#undef BIAS_ADD
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
+int saga_hip_bias_bwd(const SagaTensorView *dy, const SagaTensorView *db, float beta, saga_stream_t stream)
+{
+    if(!valid_view(dy) || !valid_view(db))
+        return SAGA_HIP_EINVAL;
+    if(view_elements(db) != dy->dims[1])
+        return SAGA_HIP_ESHAPE;
+    hipStream_t st = as_stream(stream);
+    CLInfo cl;
+    CFInfo cf;
+#define BIAS_BWD(T, TB)                                                                                     \
+    if(as_channels_last(dy, &cl))                                                                           \
+        bias_bwd_cl<T, TB><<<(cl.C + 63) / 64, 256, 0, st>>>((const T *)dy->ptr, cl.pitch, (TB *)db->ptr,     \
+                                                             cl.rows, cl.C, beta);                          \
+    else if(as_channels_first(dy, &cf))                                                                     \
+        bias_bwd_cf<T, TB><<<cf.C, 256, 0, st>>>((const T *)dy->ptr, cf.npitch, (TB *)db->ptr, cf.N, cf.C,   \
+                                                 cf.HW, beta);                                              \
+    else                                                                                                    \
+        return SAGA_HIP_EUNSUPPORTED;
+    if(dy->dtype == SAGA_HALF && db->dtype == SAGA_HALF) {
+        BIAS_BWD(half_t, half_t)
+    } else if(dy->dtype == SAGA_HALF && db->dtype == SAGA_FLOAT) {
+        BIAS_BWD(half_t, float)
+    } else if(dy->dtype == SAGA_FLOAT && db->dtype == SAGA_FLOAT) {
+        BIAS_BWD(float, float)
+    } else
+        return SAGA_HIP_EUNSUPPORTED;
+#undef BIAS_BWD
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
+int saga_hip_fill(void *ptr, int value, size_t bytes, saga_stream_t stream)
+{
+    if(!ptr && bytes)
+        return SAGA_HIP_EINVAL;
+    if(bytes == 0)
+        return 0;
+    fill_bytes<<<grid_for((int64_t)(bytes / 16 + 1), 256, 256 * 16), 256, 0, as_stream(stream)>>>(
+        (uint8_t *)ptr, (uint8_t)value, bytes);
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
+const char *saga_hip_error_string(int code)
+{
+    switch(code) {
+    case SAGA_HIP_OK: return "ok";
+    case SAGA_HIP_EINVAL: return "invalid argument";
+    case SAGA_HIP_ESHAPE: return "operand shapes do not agree";
+    case SAGA_HIP_EUNSUPPORTED: return "unsupported dtype or layout";
+    case SAGA_HIP_EWORKSPACE: return "workspace missing or too small";
+    }
+    if(code > 0)
+        return hipGetErrorString((hipError_t)code);
+    return "unknown error";
+}
+
+int saga_hip_init(int device, int *cus)
+{
+    hipError_t e = hipSetDevice(device);
+    if(e != hipSuccess)
+        return (int)e;
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, device);
+    if(e != hipSuccess)
+        return (int)e;
+    if(cus)
+        *cus = prop.multiProcessorCount;
+    return 0;
+}
+
+} // extern "C"

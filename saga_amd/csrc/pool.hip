@@ -1,0 +1,315 @@
+// Max / average pooling, forward and backward, for any 4-D strides.
+// Channels-last tensors are processed in vectors of channels (16-byte loads, lanes on
+// consecutive channel groups); everything else runs one element per lane with w fastest.
+// Backward is a gather over the windows that cover each input position, so no atomics are
+// needed and fp16 gradients are summed in fp32 registers.
+#include "common.hpp"
+
+namespace {
+
+template <typename T, int VN> struct PV {
+    static __device__ __forceinline__ void load(const T *p, float (&o)[VN])
+    {
+        if constexpr(VN == 1) {
+            o[0] = (float)*p;
+        } else if constexpr(sizeof(T) == 2) {
+            const half8_t v = *(const half8_t *)p;
+#pragma unroll
+            for(int j = 0; j < VN; j++)
+                o[j] = (float)v[j];
+        } else {
+            const float4_t v = *(const float4_t *)p;
+#pragma unroll
+            for(int j = 0; j < VN; j++)
+                o[j] = v[j];
+        }
+    }
+    static __device__ __forceinline__ void store(T *p, const float (&o)[VN])
+    {
+        if constexpr(VN == 1) {
+            *p = (T)o[0];
+        } else if constexpr(sizeof(T) == 2) {
+            half8_t v;
+#pragma unroll
+            for(int j = 0; j < VN; j++)
+                v[j] = (T)o[j];
+            *(half8_t *)p = v;
+        } else {
+            float4_t v;
+#pragma unroll
+            for(int j = 0; j < VN; j++)
+                v[j] = o[j];
+            *(float4_t *)p = v;
+        }
+    }
+};
+
+__device__ __forceinline__ int64_t off4(const DView &v, int n, int c, int h, int w)
+{
+    return n * v.s[0] + c * v.s[1] + h * v.s[2] + w * v.s[3];
+}
+
+// Decodes a linear work index into (n, c0, h, w) for a tensor of dims (N, C, H, W) walked in
+// vectors of VN channels; channel vectors are fastest when VN > 1, w otherwise.
+template <int VN>
+__device__ __forceinline__ void decode(int64_t i, int C, int H, int W, int &n, int &c, int &h, int &w)
+{
+    if(VN > 1) {
+        const int cv = C / VN;
+        c = (int)(i % cv) * VN;
+        i /= cv;
+        w = (int)(i % W);
+        i /= W;
+        h = (int)(i % H);
+        n = (int)(i / H);
+    } else {
+        w = (int)(i % W);
+        i /= W;
+        h = (int)(i % H);
+        i /= H;
+        c = (int)(i % C);
+        n = (int)(i / C);
+    }
+}
+
+__device__ __forceinline__ bool better(float v, float best) { return v > best || (v != v && best == best); }
+__device__ __forceinline__ bool same(float a, float b) { return a == b || (a != a && b != b); }
+
+template <typename T, int VN, int MODE>
+__global__ void __launch_bounds__(256)
+    pool_fwd_k(DView x, DView y, DView idx, int has_idx, int k, int pad, int stride, int64_t total)
+{
+    const int C = y.d[1], P = y.d[2], Q = y.d[3], H = x.d[2], W = x.d[3];
+    const float inv = 1.0f / (float)(k * k);
+    for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        int n, c, p, q;
+        decode<VN>(i, C, P, Q, n, c, p, q);
+        float acc[VN];
+        int best[VN];
+        bool first = true; // the first in-bounds position seeds the maximum for every channel
+#pragma unroll
+        for(int j = 0; j < VN; j++) {
+            acc[j] = MODE == SAGA_POOL_MAX ? -INFINITY : 0.0f;
+            best[j] = -1;
+        }
+        for(int r = 0; r < k; r++) {
+            const int h = p * stride - pad + r;
+            if(h < 0 || h >= H)
+                continue;
+            for(int s = 0; s < k; s++) {
+                const int w = q * stride - pad + s;
+                if(w < 0 || w >= W)
+                    continue;
+                float v[VN];
+                PV<T, VN>::load((const T *)x.ptr + off4(x, n, c, h, w), v);
+                const int pos = h * W + w;
+#pragma unroll
+                for(int j = 0; j < VN; j++) {
+                    if(MODE == SAGA_POOL_MAX) {
+                        const bool take = first | better(v[j], acc[j]);
+                        acc[j] = take ? v[j] : acc[j];
+                        best[j] = take ? pos : best[j];
+                    } else {
+                        acc[j] += v[j];
+                    }
+                }
+                first = false;
+            }
+        }
+        if(MODE == SAGA_POOL_AVG) {
+#pragma unroll
+            for(int j = 0; j < VN; j++)
+                acc[j] *= inv;
+        }
+        PV<T, VN>::store((T *)y.ptr + off4(y, n, c, p, q), acc);
+        if(MODE == SAGA_POOL_MAX && has_idx) {
+#pragma unroll
+            for(int j = 0; j < VN; j++)
+                ((int32_t *)idx.ptr)[off4(idx, n, c + j, p, q)] = best[j];
+        }
+    }
+}
+
+static __device__ __forceinline__ int cdiv_floor(int a, int b) { return a >= 0 ? a / b : -((-a + b - 1) / b); }
+
+template <typename T, int VN, int MODE>
+__global__ void __launch_bounds__(256)
+    pool_bwd_k(DView x, DView y, DView dy, DView dx, int k, int pad, int stride, float beta, int64_t total)
+{
+    const int C = dx.d[1], H = dx.d[2], W = dx.d[3], P = dy.d[2], Q = dy.d[3];
+    const float inv = 1.0f / (float)(k * k);
+    for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        int n, c, h, w;
+        decode<VN>(i, C, H, W, n, c, h, w);
+        float acc[VN], xv[VN];
+#pragma unroll
+        for(int j = 0; j < VN; j++)
+            acc[j] = 0.0f;
+        if(MODE == SAGA_POOL_MAX)
+            PV<T, VN>::load((const T *)x.ptr + off4(x, n, c, h, w), xv);
+        int p0 = cdiv_floor(h + pad - k + stride, stride), p1 = cdiv_floor(h + pad, stride);
+        int q0 = cdiv_floor(w + pad - k + stride, stride), q1 = cdiv_floor(w + pad, stride);
+        if(p0 < 0) p0 = 0;
+        if(q0 < 0) q0 = 0;
+        if(p1 > P - 1) p1 = P - 1;
+        if(q1 > Q - 1) q1 = Q - 1;
+        for(int p = p0; p <= p1; p++) {
+            for(int q = q0; q <= q1; q++) {
+                float g[VN];
+                PV<T, VN>::load((const T *)dy.ptr + off4(dy, n, c, p, q), g);
+                if(MODE == SAGA_POOL_AVG) {
+#pragma unroll
+                    for(int j = 0; j < VN; j++)
+                        acc[j] += g[j] * inv;
+                    continue;
+                }
+                float yv[VN];
+                PV<T, VN>::load((const T *)y.ptr + off4(y, n, c, p, q), yv);
+                bool hit[VN];
+                bool any = false;
+#pragma unroll
+                for(int j = 0; j < VN; j++) {
+                    hit[j] = same(xv[j], yv[j]);
+                    any |= hit[j];
+                }
+                if(!any)
+                    continue;
+                // the gradient goes to the FIRST position of the window that holds the maximum
+                const int hs = p * stride - pad, ws = q * stride - pad;
+                for(int r = 0; r < k && any; r++) {
+                    const int hh = hs + r;
+                    if(hh < 0 || hh >= H)
+                        continue;
+                    if(hh > h)
+                        break;
+                    for(int s = 0; s < k; s++) {
+                        const int ww = ws + s;
+                        if(ww < 0 || ww >= W)
+                            continue;
+                        if(hh == h && ww >= w)
+                            break;
+                        float e[VN];
+                        PV<T, VN>::load((const T *)x.ptr + off4(x, n, c, hh, ww), e);
+                        any = false;
+#pragma unroll
+                        for(int j = 0; j < VN; j++) {
+                            if(hit[j] && same(e[j], yv[j]))
+                                hit[j] = false;
+                            any |= hit[j];
+                        }
+                    }
+                }
+#pragma unroll
+                for(int j = 0; j < VN; j++)
+                    if(hit[j])
+                        acc[j] += g[j];
+            }
+        }
+        T *o = (T *)dx.ptr + off4(dx, n, c, h, w);
+        if(beta != 0.0f) {
+            float old[VN];
+            PV<T, VN>::load(o, old);
+#pragma unroll
+            for(int j = 0; j < VN; j++)
+                acc[j] += beta * old[j];
+        }
+        PV<T, VN>::store(o, acc);
+    }
+}
+
+static int vec_for(int dtype, std::initializer_list<const SagaTensorView *> vs)
+{
+    const int vn = dtype == SAGA_HALF ? 8 : 4;
+    for(auto v : vs) {
+        if(!v)
+            continue;
+        if(v->dims[1] % vn || (v->dims[1] > 1 && v->strides[1] != 1) || !aligned16(v->ptr))
+            return 1;
+        for(int i : {0, 2, 3})
+            if(v->dims[i] > 1 && v->strides[i] % vn)
+                return 1;
+    }
+    return vn;
+}
+
+static int pool_dim(int in, int k, int pad, int stride) { return 1 + (in + 2 * pad - k) / stride; }
+
+} // namespace
+
+extern "C" {
+
+int saga_hip_pool_fwd(int mode, const SagaTensorView *x, const SagaTensorView *y, const SagaTensorView *idx,
+                      int size, int pad, int stride, saga_stream_t stream)
+{
+    if(!valid_view(x) || !valid_view(y) || size < 1 || stride < 1 || pad < 0 || (idx && !valid_view(idx)))
+        return SAGA_HIP_EINVAL;
+    if(mode != SAGA_POOL_MAX && mode != SAGA_POOL_AVG)
+        return SAGA_HIP_EINVAL;
+    if(y->dims[0] != x->dims[0] || y->dims[1] != x->dims[1] || y->dims[2] != pool_dim(x->dims[2], size, pad, stride) ||
+       y->dims[3] != pool_dim(x->dims[3], size, pad, stride) || (idx && !same_dims(idx, y)))
+        return SAGA_HIP_ESHAPE;
+    if(x->dtype != y->dtype || (x->dtype != SAGA_HALF && x->dtype != SAGA_FLOAT) || (idx && idx->dtype != SAGA_I32))
+        return SAGA_HIP_EUNSUPPORTED;
+    const int vn = vec_for(x->dtype, {x, y});
+    const int64_t total = view_elements(y) / vn;
+    const int g = grid_for(total, 256, 256 * 32);
+    hipStream_t st = as_stream(stream);
+    DView dvx = dview(x), dvy = dview(y), dvi = idx ? dview(idx) : dview(y);
+#define GO(T, VN)                                                                                        \
+    do {                                                                                                 \
+        if(mode == SAGA_POOL_MAX)                                                                        \
+            pool_fwd_k<T, VN, SAGA_POOL_MAX><<<g, 256, 0, st>>>(dvx, dvy, dvi, idx != nullptr, size, pad, \
+                                                                stride, total);                          \
+        else                                                                                             \
+            pool_fwd_k<T, VN, SAGA_POOL_AVG><<<g, 256, 0, st>>>(dvx, dvy, dvi, 0, size, pad, stride, total); \
+    } while(0)
+    if(x->dtype == SAGA_HALF) {
+        if(vn == 8) GO(half_t, 8); else GO(half_t, 1);
+    } else {
+        if(vn == 4) GO(float, 4); else GO(float, 1);
+    }
+#undef GO
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
+int saga_hip_pool_bwd(int mode, const SagaTensorView *x, const SagaTensorView *y, const SagaTensorView *dy,
+                      const SagaTensorView *dx, int size, int pad, int stride, float beta, saga_stream_t stream)
+{
+    if(!valid_view(dy) || !valid_view(dx) || size < 1 || stride < 1 || pad < 0)
+        return SAGA_HIP_EINVAL;
+    if(mode != SAGA_POOL_MAX && mode != SAGA_POOL_AVG)
+        return SAGA_HIP_EINVAL;
+    const bool mx = mode == SAGA_POOL_MAX;
+    if(mx && (!valid_view(x) || !valid_view(y)))
+        return SAGA_HIP_EINVAL;
+    if(dy->dims[0] != dx->dims[0] || dy->dims[1] != dx->dims[1] ||
+       dy->dims[2] != pool_dim(dx->dims[2], size, pad, stride) || dy->dims[3] != pool_dim(dx->dims[3], size, pad, stride) ||
+       (mx && (!same_dims(x, dx) || !same_dims(y, dy))))
+        return SAGA_HIP_ESHAPE;
+    const int dt = dx->dtype;
+    if((dt != SAGA_HALF && dt != SAGA_FLOAT) || dy->dtype != dt || (mx && (x->dtype != dt || y->dtype != dt)))
+        return SAGA_HIP_EUNSUPPORTED;
+    const int vn = vec_for(dt, {dx, dy, mx ? x : nullptr, mx ? y : nullptr});
+    const int64_t total = view_elements(dx) / vn;
+    const int g = grid_for(total, 256, 256 * 32);
+    hipStream_t st = as_stream(stream);
+    DView dvx = mx ? dview(x) : dview(dx), dvy = mx ? dview(y) : dview(dy), dvdy = dview(dy), dvdx = dview(dx);
+#define GO(T, VN)                                                                                              \
+    do {                                                                                                       \
+        if(mx)                                                                                                 \
+            pool_bwd_k<T, VN, SAGA_POOL_MAX><<<g, 256, 0, st>>>(dvx, dvy, dvdy, dvdx, size, pad, stride, beta, total); \
+        else                                                                                                   \
+            pool_bwd_k<T, VN, SAGA_POOL_AVG><<<g, 256, 0, st>>>(dvx, dvy, dvdy, dvdx, size, pad, stride, beta, total); \
+    } while(0)
+    if(dt == SAGA_HALF) {
+        if(vn == 8) GO(half_t, 8); else GO(half_t, 1);
+    } else {
+        if(vn == 4) GO(float, 4); else GO(float, 1);
+    }
+#undef GO
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
+} // extern "C"

@@ -1,0 +1,488 @@
+"""GPU parity: every entry point of the C ABI (include/saga_hip.h) against the CPU oracle on the
+same seeded inputs.  fp32 within 1e-4 and fp16 within 2e-2 of the per-tensor max-abs value;
+labels, pooling indices and flags bit-exact."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import ref
+from saga_amd import kernels as K
+from tests.gpu_util import assert_close, dev, host, rnd
+
+pytestmark = pytest.mark.gpu
+
+DT = [torch.float32, torch.float16]
+LAYOUTS = [("nchw", 0), ("nhwc", 0), ("nhwc", 8)]
+
+
+def S():
+    return K.stream_ptr()
+
+
+def T(g, name):
+    t = g[name]
+    return np.array(t["data"][: int(np.prod(t["dims"]))], np.float32).reshape(t["dims"])
+
+
+def w_dev(w, dtype, layout):
+    return dev(w, dtype, "nhwc" if layout == "nhwc" else "nchw")
+
+
+CONV_CASES = [
+    # N, C, H, W, K, R, pad, stride, group
+    (2, 16, 9, 9, 8, 3, 1, 1, 1),
+    (2, 8, 11, 10, 16, 3, 1, 2, 1),
+    (1, 3, 15, 15, 8, 7, 3, 2, 1),
+    (2, 16, 8, 8, 32, 1, 0, 1, 1),
+    (2, 32, 8, 8, 16, 1, 0, 2, 1),
+    (2, 8, 7, 7, 4, 3, 0, 1, 2),
+    (3, 64, 14, 14, 64, 3, 1, 1, 1),
+]
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("layout,padc", LAYOUTS)
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv_fwd_bwd(case, layout, padc, dtype):
+    N, Cc, H, W, Kk, R, pad, stride, group = case
+    rng = np.random.default_rng(hash(case) % 1000)
+    x = rnd(rng, N, Cc, H, W, dtype=dtype)
+    w = rnd(rng, Kk, Cc // group, R, R, dtype=dtype, scale=(2.0 / (Cc // group * R * R)) ** 0.5)
+    y_ref = ref.conv2d_fwd(x, w, pad, stride, 1, group)
+    dy = rnd(rng, *y_ref.shape, dtype=dtype)
+    dx_ref = ref.conv2d_bwd_data(dy, w, x.shape, pad, stride, 1, group)
+    dw_ref = ref.conv2d_bwd_filter(x, dy, w.shape, pad, stride, 1, group)
+
+    xd, wd = dev(x, dtype, layout, padc), w_dev(w, dtype, layout)
+    yd = dev(np.zeros_like(y_ref), dtype, layout, padc)
+    K.conv2d(K.CONV_FWD, xd, wd, yd, pad, stride, 1, group)
+    assert_close(host(yd), y_ref, dtype, "y")
+    # beta = 1 accumulates into the existing output (residual sum folded into the conv)
+    K.conv2d(K.CONV_FWD, xd, wd, yd, pad, stride, 1, group, 1.0, 1.0)
+    assert_close(host(yd), 2 * y_ref, dtype, "y beta=1")
+
+    dyd = dev(dy, dtype, layout, padc)
+    dxd = dev(np.zeros_like(x), dtype, layout, padc)
+    K.conv2d(K.CONV_BWD_DATA, dyd, wd, dxd, pad, stride, 1, group)
+    assert_close(host(dxd), dx_ref, dtype, "dx")
+    dwd = w_dev(np.zeros_like(w), dtype, layout)
+    K.conv2d(K.CONV_BWD_FILTER, xd, dyd, dwd, pad, stride, 1, group)
+    assert_close(host(dwd), dw_ref, dtype, "dw")
+    K.conv2d(K.CONV_BWD_FILTER, xd, dyd, dwd, pad, stride, 1, group, 1.0, 1.0)
+    assert_close(host(dwd), 2 * dw_ref, dtype, "dw beta=1")
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_conv_golden(golden, dtype):
+    g = golden["ops"]
+    for layout in ("nchw", "nhwc"):
+        x, w = dev(T(g, "conv_input_x"), dtype, layout), w_dev(T(g, "conv_input_w"), dtype, layout)
+        y = dev(np.zeros((1, 2, 8, 8), np.float32), dtype, layout)
+        K.conv2d(K.CONV_FWD, x, w, y, pad=1)
+        b = dev(T(g, "conv_input_b").reshape(-1), dtype)
+        K.check(K.lib().saga_hip_bias_add(C.byref(K.view(y)), C.byref(K.view(b.view(1, 2, 1, 1))), S()))
+        sse = float(((host(y).astype(np.float64) - T(g, "conv_output")) ** 2).sum())
+        assert sse <= (1e-4 if dtype == torch.float32 else 1e-3), sse
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_transposed_conv(dtype):
+    # forward of a transposed conv is bwd_data with x in the dy role (src/cuda/cuda_dnn.cpp:545-548)
+    rng = np.random.default_rng(3)
+    x, w = rnd(rng, 2, 16, 5, 5, dtype=dtype), rnd(rng, 16, 8, 2, 2, dtype=dtype, scale=0.2)
+    Ho = ref.tconv_out(5, 2, 0, 2)
+    y_ref = ref.conv2d_bwd_data(x, w, (2, 8, Ho, Ho), 0, 2)
+    for layout in ("nchw", "nhwc"):
+        yd = dev(np.zeros_like(y_ref), dtype, layout)
+        K.conv2d(K.CONV_BWD_DATA, dev(x, dtype, layout), w_dev(w, dtype, layout), yd, 0, 2)
+        assert_close(host(yd), y_ref, dtype, "tconv y")
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("layout,padc", LAYOUTS)
+def test_bias(layout, padc, dtype):
+    rng = np.random.default_rng(5)
+    y, b = rnd(rng, 3, 16, 5, 5, dtype=dtype), rnd(rng, 16, dtype=dtype)
+    yd = dev(y, dtype, layout, padc)
+    bd = dev(b, torch.float32)
+    K.check(K.lib().saga_hip_bias_add(C.byref(K.view(yd)), C.byref(K.view(bd.view(1, 16, 1, 1))), S()))
+    assert_close(host(yd), ref.bias_add(y, b), dtype, "bias add")
+    db = dev(np.ones(16, np.float32), torch.float32)
+    dyd = dev(y, dtype, layout, padc)
+    K.check(K.lib().saga_hip_bias_bwd(C.byref(K.view(dyd)), C.byref(K.view(db.view(1, 16, 1, 1))), 1.0, S()))
+    assert_close(host(db), ref.bias_bwd(y) + 1, dtype, "bias bwd")
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("tA,tB", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_gemm(tA, tB, dtype):
+    rng = np.random.default_rng(11)
+    M, N, Kd = 37, 70, 129
+    A, B = rnd(rng, M, Kd, dtype=dtype, scale=0.3), rnd(rng, Kd, N, dtype=dtype, scale=0.3)
+    Cref = A.astype(np.float64) @ B.astype(np.float64)
+    Ad = dev(A.T if tA else A, dtype)
+    Bd = dev(B.T if tB else B, dtype)
+    Cd = dev(np.ones((M, N), np.float32), dtype)
+    code = K.HALF if dtype == torch.float16 else K.FLOAT
+    K.check(K.lib().saga_hip_gemm(tA, tB, M, N, Kd, 1.0, K.ptr(Ad), Ad.shape[1], K.ptr(Bd), Bd.shape[1], 1.0, K.ptr(Cd),
+                                  N, code, S()))
+    assert_close(host(Cd), Cref + 1, dtype, "gemm")
+
+
+def test_fc_golden(golden):
+    g = golden["ops"]
+    x, w = T(g, "fc2_input_x"), T(g, "fc2_input_w")  # transW: w is [out, in]
+    xd, wd = dev(x), dev(w)
+    yd = dev(np.zeros((2, 8), np.float32))
+    K.check(K.lib().saga_hip_gemm(0, 1, 2, 8, 32, 1.0, K.ptr(xd), 32, K.ptr(wd), 32, 0.0, K.ptr(yd), 8, K.FLOAT, S()))
+    assert float(((host(yd) - T(g, "fc2_output_no_bias")) ** 2).sum()) <= 1e-4
+    x, w = T(g, "fc1_input_x"), T(g, "fc1_input_w")
+    xd, wd, yd = dev(x), dev(w), dev(np.zeros((2, 3), np.float32))
+    K.check(K.lib().saga_hip_gemm(0, 0, 2, 3, 2, 1.0, K.ptr(xd), 2, K.ptr(wd), 3, 0.0, K.ptr(yd), 3, K.FLOAT, S()))
+    assert float(((host(yd) - T(g, "fc1_output_no_bias")) ** 2).sum()) <= 1e-4
+
+
+def _bn_params(rng, Cc):
+    s = (rng.standard_normal(Cc) * 0.5 + 1).astype(np.float32)
+    b = rng.standard_normal(Cc).astype(np.float32)
+    m = (rng.standard_normal(Cc) * 0.1).astype(np.float32)
+    v = rng.uniform(0.5, 1.5, Cc).astype(np.float32)
+    return s, b, m, v
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("layout,padc", LAYOUTS)
+@pytest.mark.parametrize("flags", [0, K.BN_RELU, K.BN_RELU | K.BN_ADD])
+@pytest.mark.parametrize("shape", [(4, 16, 6, 6), (3, 10, 5, 7), (2, 64, 9, 9)])
+def test_batchnorm(shape, flags, layout, padc, dtype):
+    rng = np.random.default_rng(sum(shape) + flags)
+    Cc = shape[1]
+    x = rnd(rng, *shape, dtype=dtype) * 2 + 3  # mean far from zero: exercises the shifted statistics
+    if dtype == torch.float16:
+        x = x.astype(np.float16).astype(np.float32)
+    z = rnd(rng, *shape, dtype=dtype)
+    s, b, m, v = _bn_params(rng, Cc)
+    L = K.lib()
+    xd, zd = dev(x, dtype, layout, padc), dev(z, dtype, layout, padc)
+    sd, bd, md, vd = (dev(t) for t in (s, b, m, v))
+    zarg = C.byref(K.view(zd)) if flags & K.BN_ADD else None
+
+    def post(y):
+        if flags & K.BN_ADD:
+            y = y + z
+        if flags & K.BN_RELU:
+            y = ref.act_fwd(y)
+        return y
+
+    # inference
+    yd = dev(np.zeros(shape, np.float32), dtype, layout, padc)
+    K.check(L.saga_hip_bn_infer(C.byref(K.view(xd)), zarg, C.byref(K.view(yd)), K.ptr(sd), K.ptr(bd), K.ptr(md),
+                                K.ptr(vd), 1e-5, flags, S()))
+    assert_close(host(yd), post(ref.bn_infer(x, s, b, m, v)), dtype, "bn infer")
+
+    # training forward
+    ws = K.bn_workspace(xd)
+    sm, sv = dev(np.zeros(Cc, np.float32)), dev(np.zeros(Cc, np.float32))
+    K.check(L.saga_hip_bn_train_fwd(C.byref(K.view(xd)), zarg, C.byref(K.view(yd)), K.ptr(sd), K.ptr(bd), K.ptr(md),
+                                    K.ptr(vd), K.ptr(sm), K.ptr(sv), 1e-5, 0.1, flags, K.ptr(ws), ws.numel(), S()))
+    y_bn, rsm, rsv, rm, rv = ref.bn_train_fwd(x, s, b, m, v, 1e-5, 0.1)
+    y_ref = post(y_bn)
+    assert_close(host(yd), y_ref, dtype, "bn train y")
+    assert_close(host(sm), rsm, torch.float32, "saved mean", 1e-4 if dtype == torch.float32 else 1e-3)
+    assert_close(host(sv), rsv, torch.float32, "saved invstd", 1e-4 if dtype == torch.float32 else 1e-3)
+    assert_close(host(md), rm, torch.float32, "running mean", 1e-4 if dtype == torch.float32 else 1e-3)
+    assert_close(host(vd), rv, torch.float32, "running var", 1e-4 if dtype == torch.float32 else 1e-3)
+
+    # backward (uses the oracle's saved statistics so both sides see identical inputs)
+    dy = rnd(rng, *shape, dtype=dtype)
+    y_h = ref.round_half(y_ref) if dtype == torch.float16 else y_ref
+    dyp = dy * (y_h > 0) if flags & K.BN_RELU else dy
+    dx_ref, ds_ref, db_ref = ref.bn_bwd(x, dyp, s, rsm, rsv)
+    dxd = dev(np.ones(shape, np.float32), dtype, layout, padc)
+    dzd = dev(np.zeros(shape, np.float32), dtype, layout, padc)
+    dsd, dbd = dev(np.zeros(Cc, np.float32)), dev(np.zeros(Cc, np.float32))
+    y_in = dev(y_h, dtype, layout, padc)
+    dyd, rsmd, rsvd = dev(dy, dtype, layout, padc), dev(rsm), dev(rsv)  # named: the kernel reads them after this line
+    K.check(L.saga_hip_bn_bwd(C.byref(K.view(xd)), C.byref(K.view(y_in)) if flags & K.BN_RELU else None,
+                              C.byref(K.view(dyd)), C.byref(K.view(dxd)),
+                              C.byref(K.view(dzd)) if flags & K.BN_ADD else None, K.ptr(sd), K.ptr(rsmd),
+                              K.ptr(rsvd), K.ptr(dsd), K.ptr(dbd), 1.0, 0.0, 0.0, flags, K.ptr(ws), ws.numel(), S()))
+    assert_close(host(dxd), dx_ref + 1, dtype, "bn dx (beta=1)")
+    assert_close(host(dsd), ds_ref, torch.float32, "bn ds", 1e-4 if dtype == torch.float32 else 5e-3)
+    assert_close(host(dbd), db_ref, torch.float32, "bn db", 1e-4 if dtype == torch.float32 else 5e-3)
+    if flags & K.BN_ADD:
+        assert_close(host(dzd), dyp, dtype, "bn dz")
+
+
+def test_batchnorm_golden(golden):
+    g = golden["ops"]
+    x = T(g, "batchnorm_input_x")
+    for layout in ("nchw", "nhwc"):
+        xd = dev(x, torch.float32, layout)
+        yd = dev(np.zeros_like(x), torch.float32, layout)
+        p = [dev(T(g, "batchnorm_input_" + n)) for n in "sbmv"]
+        K.check(K.lib().saga_hip_bn_infer(C.byref(K.view(xd)), None, C.byref(K.view(yd)), K.ptr(p[0]), K.ptr(p[1]),
+                                          K.ptr(p[2]), K.ptr(p[3]), 1e-5, 0, S()))
+        assert float(((host(yd) - T(g, "batchnorm_output")) ** 2).sum()) <= 1e-4
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("layout,padc", LAYOUTS)
+@pytest.mark.parametrize("mode", ["relu", "sigmoid", "tanh", "swish", "leakyrelu"])
+def test_activation(mode, layout, padc, dtype):
+    rng = np.random.default_rng(2)
+    shape = (2, 16, 5, 5)
+    x, dy = rnd(rng, *shape, dtype=dtype), rnd(rng, *shape, dtype=dtype)
+    alpha = 0.01 if mode == "leakyrelu" else 0.0
+    code = ["relu", "sigmoid", "tanh", "swish", "leakyrelu"].index(mode)
+    xd = dev(x, dtype, layout, padc)
+    yd = dev(np.zeros(shape, np.float32), dtype, layout, padc)
+    K.check(K.lib().saga_hip_act_fwd(code, alpha, C.byref(K.view(xd)), C.byref(K.view(yd)), 0.0, S()))
+    y_ref = ref.act_fwd(x, mode, alpha)
+    assert_close(host(yd), y_ref, dtype, "act fwd")
+    dxd = dev(np.ones(shape, np.float32), dtype, layout, padc)
+    dyd = dev(dy, dtype, layout, padc)
+    K.check(K.lib().saga_hip_act_bwd(code, alpha, C.byref(K.view(xd)), C.byref(K.view(yd)), C.byref(K.view(dyd)),
+                                     C.byref(K.view(dxd)), 1.0, S()))
+    assert_close(host(dxd), ref.act_bwd(x, host(yd), dy, mode, alpha) + 1, dtype, "act bwd")
+
+
+def test_relu_golden_and_nan(golden):
+    g = golden["ops"]
+    x = T(g, "relu_input")
+    xd, yd = dev(x), dev(np.zeros_like(x))
+    K.check(K.lib().saga_hip_act_fwd(0, 0.0, C.byref(K.view(xd)), C.byref(K.view(yd)), 0.0, S()))
+    np.testing.assert_array_equal(host(yd), T(g, "relu_output"))
+    xd = dev(np.array([[np.nan, -1.0, 2.0]], np.float32))
+    yd = dev(np.zeros((1, 3), np.float32))
+    K.check(K.lib().saga_hip_act_fwd(0, 0.0, C.byref(K.view(xd)), C.byref(K.view(yd)), 0.0, S()))
+    r = host(yd)
+    assert np.isnan(r[0, 0]) and r[0, 1] == 0 and r[0, 2] == 2
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("layout,padc", LAYOUTS)
+@pytest.mark.parametrize("k,pad,stride,H", [(2, 0, 2, 8), (3, 1, 2, 9), (3, 1, 1, 6), (7, 0, 1, 7)])
+def test_pooling(k, pad, stride, H, layout, padc, dtype):
+    rng = np.random.default_rng(k * 10 + H)
+    shape = (2, 16, H, H)
+    x = rnd(rng, *shape, dtype=dtype)
+    x = np.maximum(x, 0)  # post-relu data: many exact ties at 0 stress the first-index rule
+    P = ref.pool_out(H, k, pad, stride)
+    oshape = (2, 16, P, P)
+    dy = rnd(rng, *oshape, dtype=dtype)
+    L = K.lib()
+    xd = dev(x, dtype, layout, padc)
+    for mode, code in (("max", K.POOL_MAX), ("avg", K.POOL_AVG)):
+        yd = dev(np.zeros(oshape, np.float32), dtype, layout, padc)
+        idx = torch.zeros(oshape, dtype=torch.int32, device="cuda")
+        K.check(L.saga_hip_pool_fwd(code, C.byref(K.view(xd)), C.byref(K.view(yd)),
+                                    C.byref(K.view(idx)) if mode == "max" else None, k, pad, stride, S()))
+        if mode == "max":
+            y_ref, idx_ref = ref.maxpool_fwd(x, k, pad, stride, with_idx=True)
+            np.testing.assert_array_equal(host(yd), y_ref)  # max is exact in any precision
+            np.testing.assert_array_equal(idx.cpu().numpy(), idx_ref)  # pooling indices bit-exact
+            dx_ref = ref.maxpool_bwd(x, dy, k, pad, stride)
+        else:
+            assert_close(host(yd), ref.avgpool_fwd(x, k, pad, stride), dtype, "avgpool")
+            dx_ref = ref.avgpool_bwd(dy, shape, k, pad, stride)
+        dxd = dev(np.ones(shape, np.float32), dtype, layout, padc)
+        dyd = dev(dy, dtype, layout, padc)
+        K.check(L.saga_hip_pool_bwd(code, C.byref(K.view(xd)), C.byref(K.view(yd)), C.byref(K.view(dyd)),
+                                    C.byref(K.view(dxd)), k, pad, stride, 1.0, S()))
+        assert_close(host(dxd), dx_ref + 1, dtype, mode + "pool bwd")
+
+
+def test_pooling_golden(golden):
+    g = golden["ops"]
+    x = T(g, "pooling_input")
+    for layout in ("nchw", "nhwc"):
+        xd = dev(x, torch.float32, layout)
+        for code, k, st, name in ((K.POOL_MAX, 2, 2, "maxpool_output"), (K.POOL_MAX, 8, 1, "maxpool_output_global"),
+                                  (K.POOL_AVG, 2, 2, "avgpool_output"), (K.POOL_AVG, 8, 1, "avgpool_output_global")):
+            want = T(g, name)
+            yd = dev(np.zeros_like(want), torch.float32, layout)
+            K.check(K.lib().saga_hip_pool_fwd(code, C.byref(K.view(xd)), C.byref(K.view(yd)), None, k, 0, st, S()))
+            assert float(((host(yd) - want) ** 2).sum()) <= 1e-4, name
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_add_axpby_convert_concat(dtype, golden):
+    rng = np.random.default_rng(9)
+    shape = (2, 8, 4, 4)
+    a, b = rnd(rng, *shape, dtype=dtype), rnd(rng, *shape, dtype=dtype)
+    L = K.lib()
+    for la, lb, lo in (("nchw", "nchw", "nchw"), ("nhwc", "nhwc", "nhwc"), ("nhwc", "nchw", "nhwc")):
+        ad, bd, od = dev(a, dtype, la), dev(b, dtype, lb, 8 if lb == "nhwc" else 0), dev(np.zeros(shape), dtype, lo)
+        K.check(L.saga_hip_add(C.byref(K.view(ad)), C.byref(K.view(bd)), C.byref(K.view(od)), S()))
+        assert_close(host(od), a + b, dtype, "add")
+        K.check(L.saga_hip_axpby(C.byref(K.view(ad)), C.byref(K.view(od)), 1.0, 1.0, S()))
+        assert_close(host(od), 2 * a + b, dtype, "axpby")
+    # concat realised as strided outputs: two producers write channel slices of one NHWC buffer
+    g = golden["ops"]
+    x0, x1 = T(g, "concat_input_x0"), T(g, "concat_input_x1")
+    wide = torch.zeros((2, 4, 4, 4), dtype=dtype, device="cuda")  # N,H,W,C
+    for i, src in enumerate((x0, x1)):
+        sl = wide[..., 2 * i:2 * i + 2].permute(0, 3, 1, 2)
+        srcd = dev(src, dtype, "nhwc")
+        K.check(L.saga_hip_axpby(C.byref(K.view(srcd)), C.byref(K.view(sl)), 1.0, 0.0, S()))
+        torch.cuda.synchronize()
+    got = host(wide.permute(0, 3, 1, 2))
+    assert float(((got - T(g, "concat_output")) ** 2).sum()) <= (1e-4 if dtype == torch.float32 else 1e-3)
+    # u8 -> float/half with scale
+    u = rng.integers(0, 256, shape).astype(np.uint8)
+    ud = torch.from_numpy(u).cuda()
+    od = dev(np.zeros(shape), dtype, "nhwc")
+    K.check(L.saga_hip_convert(C.byref(K.view(ud)), C.byref(K.view(od)), 1 / 255.0, S()))
+    assert_close(host(od), u.astype(np.float32) / 255.0, dtype, "convert")
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_softmax(dtype):
+    rng = np.random.default_rng(4)
+    x = rnd(rng, 2, 8, 5, 5, dtype=dtype, scale=3)
+    for layout in ("nchw", "nhwc"):
+        xd, yd = dev(x, dtype, layout), dev(np.zeros_like(x), dtype, layout)
+        K.check(K.lib().saga_hip_softmax(C.byref(K.view(xd)), C.byref(K.view(yd)), S()))
+        assert_close(host(yd), ref.softmax(x), dtype, "softmax")
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("N,Cc", [(7, 10), (64, 1000), (5, 65)])
+def test_catclassifier(N, Cc, dtype):
+    rng = np.random.default_rng(N + Cc)
+    x = rnd(rng, N, Cc, dtype=dtype, scale=3)
+    x[1, 3] = x[1, Cc - 2] = x[1].max() + 1  # tie -> first index
+    if N > 2:
+        x[2, :] = 0.5  # all equal -> label 0
+    labels = rng.integers(0, Cc, N).astype(np.int32)
+    xd = dev(x, dtype)
+    pred = torch.zeros(N, dtype=torch.int32, device="cuda")
+    L = K.lib()
+    K.check(L.saga_hip_catclassifier_fwd(C.byref(K.view(xd)), K.ptr(pred), S()))
+    pred_ref = ref.catclassifier_fwd(x)
+    np.testing.assert_array_equal(pred.cpu().numpy(), pred_ref)  # labels bit-exact
+    scale = 1.0 / N if dtype == torch.float32 else 1024.0 / N
+    dxd = dev(np.zeros_like(x), dtype)
+    loss = torch.zeros(N, dtype=torch.float32, device="cuda")
+    labd = torch.from_numpy(labels).cuda()
+    K.check(L.saga_hip_catclassifier_bwd(C.byref(K.view(xd)), C.byref(K.view(dxd)), K.ptr(pred), K.ptr(labd),
+                                         K.ptr(loss), scale, S()))
+    dx_ref, loss_ref = ref.catclassifier_bwd(x, pred_ref, labels, scale)
+    assert_close(host(dxd), dx_ref, dtype, "catclassifier dx")
+    assert_close(host(loss), loss_ref, torch.float32, "loss", 1e-5)
+
+
+def test_adam_f32_100_steps():
+    rng = np.random.default_rng(1)
+    n = 10007
+    w = rng.standard_normal(n).astype(np.float32)
+    m, v = np.zeros(n, np.float32), np.zeros(n, np.float32)
+    wd, md, vd = dev(w), dev(m), dev(v)
+    aux = torch.zeros(4, dtype=torch.int32, device="cuda")
+    L = K.lib()
+    for t in range(1, 101):
+        g = (rng.standard_normal(n) * 0.1).astype(np.float32)
+        b1t, b2t = ref.adam_bias_terms(t)
+        gd = dev(g)
+        K.check(L.saga_hip_adam_f32(n, K.ptr(wd), K.ptr(gd), K.ptr(md), K.ptr(vd), float(b1t), float(b2t), 1e-3, 1e-4,
+                                    K.ptr(aux), S()))
+        torch.cuda.synchronize()
+        ref.adam_f32(w, g, m, v, t, 1e-3, 1e-4)
+    assert_close(host(wd), w, torch.float32, "adam weights after 100 steps", 1e-5)
+    assert aux.cpu().tolist() == [0, 0, 0, 0]
+    g = np.zeros(n, np.float32)
+    g[5], g[n - 1] = np.inf, np.nan  # vector body and scalar tail
+    before = host(wd).copy()
+    gd = dev(g)
+    K.check(L.saga_hip_adam_f32(n, K.ptr(wd), K.ptr(gd), K.ptr(md), K.ptr(vd), 1.0, 1.0, 1e-3, 0.0, K.ptr(aux), S()))
+    assert aux.cpu().tolist() == [0, 1, 1, 0]
+    after = host(wd)
+    assert after[5] == before[5] and after[n - 1] == before[n - 1]
+
+
+def test_adam_mixed_100_steps():
+    rng = np.random.default_rng(2)
+    n = 4099
+    scale = 256.0
+    w16 = rng.standard_normal(n).astype(np.float16)
+    c = w16.astype(np.float32)
+    m, v = np.zeros(n, np.float32), np.zeros(n, np.float32)
+    wbits = w16.view(np.uint16).copy()
+    wd = torch.from_numpy(w16.copy()).cuda()
+    cd, md, vd = dev(c), dev(m), dev(v)
+    aux = torch.zeros(4, dtype=torch.int32, device="cuda")
+    L = K.lib()
+    for t in range(1, 101):
+        g16 = (rng.standard_normal(n) * 0.1 * scale).astype(np.float16)
+        b1t, b2t = ref.adam_bias_terms(t)
+        gd = torch.from_numpy(g16).cuda()
+        K.check(L.saga_hip_adam_mixed(n, float(np.float32(1.0) / np.float32(scale)), K.ptr(wd), K.ptr(gd), K.ptr(md),
+                                      K.ptr(vd), K.ptr(cd), float(b1t), float(b2t), 1e-3, 1e-4, K.ptr(aux), S()))
+        torch.cuda.synchronize()
+        ref.adam_mixed(wbits, g16.view(np.uint16), m, v, c, t, 1e-3, scale, 1e-4)
+    assert_close(host(cd), c, torch.float32, "adam master weights after 100 steps", 1e-5)
+    got16 = wd.cpu().numpy().view(np.uint16).astype(np.int32)
+    assert np.abs(got16 - wbits.astype(np.int32)).max() <= 1  # fp16 copies agree to one ulp
+    assert aux.cpu().tolist() == [0, 0, 0, 0]
+    gbad = np.zeros(n, np.uint16)
+    gbad[0], gbad[1], gbad[n - 1] = 0x7800, 0x7c00, 0x7e00
+    gd = torch.from_numpy(gbad.view(np.float16)).cuda()
+    K.check(L.saga_hip_adam_mixed(n, 1.0, K.ptr(wd), K.ptr(gd), K.ptr(md), K.ptr(vd), K.ptr(cd), 1.0, 1.0, 1e-3, 0.0,
+                                  K.ptr(aux), S()))
+    assert aux.cpu().tolist() == [1, 1, 1, 0]
+
+
+def test_fill():
+    t = torch.zeros(1000003, dtype=torch.uint8, device="cuda")
+    K.check(K.lib().saga_hip_fill(C.c_void_p(t.data_ptr() + 3), 0xAB, 1000000 - 3, S()))
+    h = t.cpu().numpy()
+    assert (h[3:1000000] == 0xAB).all() and (h[:3] == 0).all() and (h[1000000:] == 0).all()
+
+
+def test_rejects_bad_arguments():
+    x = dev(np.zeros((1, 4, 4, 4), np.float32))
+    y = dev(np.zeros((1, 4, 3, 3), np.float32))
+    w = dev(np.zeros((4, 4, 3, 3), np.float32))
+    with pytest.raises(K.SagaHipError):
+        K.conv2d(K.CONV_FWD, x, w, y, pad=0)  # y should be 2x2
+    assert K.lib().saga_hip_act_fwd(99, 0.0, C.byref(K.view(x)), C.byref(K.view(x)), 0.0, S()) == -1
+
+
+RESNET_SHAPES = [
+    # C, H, K, R, stride, pad   (rows of the ResNet-50 v1.5 shape list, batch reduced to 2)
+    (64, 56, 64, 3, 1, 1),
+    (64, 56, 256, 1, 1, 0),
+    (256, 56, 64, 1, 1, 0),
+    (128, 56, 128, 3, 2, 1),
+    (256, 56, 512, 1, 2, 0),
+    (512, 7, 512, 3, 1, 1),
+    (1024, 14, 2048, 1, 2, 0),
+    (16, 32, 16, 3, 1, 1),
+    (24, 9, 40, 3, 1, 1),
+]
+
+
+@pytest.mark.parametrize("shape", RESNET_SHAPES)
+def test_conv_fp16_nhwc_network_shapes(shape):
+    """fp16 NHWC at the real spatial sizes of the target networks: the MFMA implicit-GEMM path."""
+    Cc, H, Kk, R, stride, pad = shape
+    N, dtype = 2, torch.float16
+    rng = np.random.default_rng(Cc + Kk + R)
+    x = rnd(rng, N, Cc, H, H, dtype=dtype)
+    w = rnd(rng, Kk, Cc, R, R, dtype=dtype, scale=(2.0 / (Cc * R * R)) ** 0.5)
+    y_ref = ref.conv2d_fwd(x, w, pad, stride)
+    dy = rnd(rng, *y_ref.shape, dtype=dtype)
+    xd, wd = dev(x, dtype, "nhwc"), dev(w, dtype, "nhwc")
+    yd = dev(np.zeros_like(y_ref), dtype, "nhwc")
+    K.conv2d(K.CONV_FWD, xd, wd, yd, pad, stride)
+    assert_close(host(yd), y_ref, dtype, "y")
+    dyd = dev(dy, dtype, "nhwc")
+    dxd = dev(np.zeros_like(x), dtype, "nhwc")
+    K.conv2d(K.CONV_BWD_DATA, dyd, wd, dxd, pad, stride)
+    assert_close(host(dxd), ref.conv2d_bwd_data(dy, w, x.shape, pad, stride), dtype, "dx")
+    dwd = dev(np.zeros_like(w), dtype, "nhwc")
+    K.conv2d(K.CONV_BWD_FILTER, xd, dyd, dwd, pad, stride)
+    assert_close(host(dwd), ref.conv2d_bwd_filter(x, dy, w.shape, pad, stride), dtype, "dw")
