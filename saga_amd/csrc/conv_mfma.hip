@@ -241,6 +241,244 @@ __global__ void __launch_bounds__(256) transpose_filter(const half_t *__restrict
     }
 }
 
+
+// ---------------------------------------------------------------- backward filter
+//
+// dw[k, tap, c] = sum_m dy[m, k] * x[pix(m, tap), c].  Both operands arrive with the
+// reduction index m as the SLOW axis (rows of channels), while the MFMA wants, per lane,
+// eight consecutive reduction elements of one row.  The tiles are therefore transposed on
+// their way into LDS: each thread loads 16 bytes = 8 channels of one pixel and scatters
+// them with eight 2-byte LDS writes into [channel][pixel] rows.  Channel ch of a tile
+// is placed in LDS row (ch % 8) * NV + ch / 8 (NV = channel vectors per tile): with that
+// permutation the 64 lanes of one write hit 64 different banks, and the epilogue simply
+// undoes it when it writes the result.
+// The reduction is split over `splits` blocks per output tile; every block writes an fp32
+// partial tile to the workspace and a second kernel adds the partials in a fixed order
+// (deterministic, no atomics) and applies alpha/beta.
+
+struct FilterArgs {
+    const half_t *x;
+    const half_t *dy;
+    float *partial;    // [splits][K][RSC]
+    int M;             // N * P * Q
+    int K, C, RSC;
+    int H, W, P, Q, S;
+    int pad, stride, dil;
+    int ldx, ldy;
+    int tiles_k, tiles_c;
+    int splits, m_per_split; // m_per_split is a multiple of BK
+};
+
+template <int BM, int BN>
+__global__ void __launch_bounds__(256) conv_bwd_filter_mfma(FilterArgs g)
+{
+    constexpr int NVA = BM / 8, NVB = BN / 8;           // channel vectors per tile
+    constexpr int PA = 256 / NVA, PB = 256 / NVB;       // pixels covered per round
+    constexpr int RA = BK / PA, RB = BK / PB;           // rounds per slice
+    constexpr int WGM = BM >= 128 ? 2 : 1, WGN = 4 / WGM;
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    static_assert(RA >= 1 && RB >= 1 && TM >= 1 && TN >= 1, "tile");
+
+    __shared__ __attribute__((aligned(16))) half_t As[2][BM * LDK];
+    __shared__ __attribute__((aligned(16))) half_t Bs[2][BN * LDK];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int b = blockIdx.x;
+    const int split = b % g.splits;
+    b /= g.splits;
+    const int tc = b % g.tiles_c, tk = b / g.tiles_c;
+    const int k0 = tk * BM, j0 = tc * BN;
+    const int m_begin = split * g.m_per_split;
+    int m_end = m_begin + g.m_per_split;
+    if(m_end > g.M)
+        m_end = g.M;
+
+    // A operand (dy): channel vector cva, pixel slots pa(j) = 2*ga + j  (RA == 2) or ga (RA == 1)
+    const int cva = tid % NVA, ga = tid / NVA;
+    const bool ka_ok = k0 + cva * 8 < g.K;
+    // B operand (x): column vector -> fixed (tap, c) for this thread
+    const int cvb = tid % NVB, gb = tid / NVB;
+    const int col = j0 + cvb * 8;
+    const bool cb_ok = col < g.RSC;
+    const int tap = cb_ok ? col / g.C : 0;
+    const int cc = cb_ok ? col - tap * g.C : 0;
+    const int fr = tap / g.S, fs = tap - fr * g.S;
+    const int offy = fr * g.dil - g.pad, offx = fs * g.dil - g.pad;
+
+    // pixel coordinates of this thread's B rows, advanced incrementally by BK per slice
+    int bn_[RB], by_[RB], bx_[RB];
+#pragma unroll
+    for(int j = 0; j < RB; j++) {
+        const int pm = RB == 1 ? gb : gb * RB + j;
+        const int m = m_begin + pm;
+        const int mm = m < g.M ? m : 0;
+        bx_[j] = mm % g.Q;
+        const int t = mm / g.Q;
+        by_[j] = t % g.P;
+        bn_[j] = t / g.P;
+    }
+
+    half8_t ra[RA], rb[RB];
+    const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    auto load_slice = [&](int ms) {
+#pragma unroll
+        for(int j = 0; j < RA; j++) {
+            const int pm = RA == 1 ? ga : ga * RA + j;
+            const int m = ms + pm;
+            ra[j] = zero;
+            if(ka_ok && m < m_end)
+                ra[j] = *(const half8_t *)(g.dy + (int64_t)m * g.ldy + k0 + cva * 8);
+        }
+#pragma unroll
+        for(int j = 0; j < RB; j++) {
+            const int pm = RB == 1 ? gb : gb * RB + j;
+            const int m = ms + pm;
+            const int iy = by_[j] * g.stride + offy, ix = bx_[j] * g.stride + offx;
+            rb[j] = zero;
+            if(cb_ok && m < m_end && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W)
+                rb[j] = *(const half8_t *)(g.x + (int64_t)((bn_[j] * g.H + iy) * g.W + ix) * g.ldx + cc);
+        }
+    };
+    auto advance = [&]() {
+#pragma unroll
+        for(int j = 0; j < RB; j++) {
+            bx_[j] += BK;
+            while(bx_[j] >= g.Q) {
+                bx_[j] -= g.Q;
+                by_[j]++;
+            }
+            while(by_[j] >= g.P) {
+                by_[j] -= g.P;
+                bn_[j]++;
+            }
+        }
+    };
+    auto store_slice = [&](int st) {
+#pragma unroll
+        for(int j = 0; j < RA; j++) {
+            const int pm = RA == 1 ? ga : ga * RA + j;
+#pragma unroll
+            for(int e = 0; e < 8; e++)
+                As[st][(e * NVA + cva) * LDK + pm] = ra[j][e];
+        }
+#pragma unroll
+        for(int j = 0; j < RB; j++) {
+            const int pm = RB == 1 ? gb : gb * RB + j;
+#pragma unroll
+            for(int e = 0; e < 8; e++)
+                Bs[st][(e * NVB + cvb) * LDK + pm] = rb[j][e];
+        }
+    };
+
+    float16_t acc[TM][TN];
+#pragma unroll
+    for(int i = 0; i < TM; i++)
+#pragma unroll
+        for(int j = 0; j < TN; j++)
+#pragma unroll
+            for(int v = 0; v < 16; v++)
+                acc[i][j][v] = 0.0f;
+
+    const int wm = (wave / WGN) * WTM, wn = (wave % WGN) * WTN;
+    const int frow = lane & 31, fk = (lane >> 5) * 8;
+    const int KT = (m_end - m_begin + BK - 1) / BK;
+
+    if(KT > 0) {
+        load_slice(m_begin);
+        store_slice(0);
+    }
+    __syncthreads();
+    for(int kt = 0; kt < KT; kt++) {
+        const int cur = kt & 1;
+        if(kt + 1 < KT) {
+            advance();
+            load_slice(m_begin + (kt + 1) * BK);
+        }
+#pragma unroll
+        for(int kk = 0; kk < BK; kk += 16) {
+            half8_t fa[TM], fb[TN];
+#pragma unroll
+            for(int i = 0; i < TM; i++)
+                fa[i] = *(const half8_t *)(&As[cur][(wm + i * 32 + frow) * LDK + kk + fk]);
+#pragma unroll
+            for(int j = 0; j < TN; j++)
+                fb[j] = *(const half8_t *)(&Bs[cur][(wn + j * 32 + frow) * LDK + kk + fk]);
+#pragma unroll
+            for(int i = 0; i < TM; i++)
+#pragma unroll
+                for(int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+        if(kt + 1 < KT)
+            store_slice(cur ^ 1);
+        __syncthreads();
+    }
+
+    // epilogue: undo the row permutations, write the fp32 partial tile
+    float *out = g.partial + (int64_t)split * g.K * g.RSC;
+    const int ecol = lane & 31, erow = (lane >> 5) * 4;
+#pragma unroll
+    for(int i = 0; i < TM; i++) {
+#pragma unroll
+        for(int j = 0; j < TN; j++) {
+            const int pb = wn + j * 32 + ecol;                 // permuted column
+            const int cj = j0 + (pb % NVB) * 8 + pb / NVB;     // flat (tap, c) column
+            if(cj >= g.RSC)
+                continue;
+#pragma unroll
+            for(int v = 0; v < 16; v++) {
+                const int pa = wm + i * 32 + (v >> 2) * 8 + erow + (v & 3);
+                const int k = k0 + (pa % NVA) * 8 + pa / NVA;
+                if(k < g.K)
+                    out[(int64_t)k * g.RSC + cj] = acc[i][j][v];
+            }
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256)
+    filter_reduce(const float *__restrict__ partial, half_t *__restrict__ dw, int64_t n, int splits, float alpha, float beta)
+{
+    for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        float s = 0;
+        for(int p = 0; p < splits; p++)
+            s += partial[(int64_t)p * n + i];
+        s *= alpha;
+        if(beta != 0.0f)
+            s += beta * (float)dw[i];
+        dw[i] = (half_t)s;
+    }
+}
+
+struct FilterPlan {
+    int bm, bn, tiles_k, tiles_c, splits, m_per_split;
+};
+
+static FilterPlan plan_filter(const ConvGeom &g)
+{
+    FilterPlan p;
+    const int RSC = g.R * g.S * g.C;
+    const int64_t M = (int64_t)g.N * g.P * g.Q;
+    p.bm = g.K > 64 ? 128 : 64;
+    p.bn = 128;
+    p.tiles_k = (g.K + p.bm - 1) / p.bm;
+    p.tiles_c = (RSC + p.bn - 1) / p.bn;
+    const int tiles = p.tiles_k * p.tiles_c;
+    int64_t want = (1024 + tiles - 1) / tiles;
+    const int64_t maxs = (M + 255) / 256; // at least 256 pixels per split
+    if(want > maxs)
+        want = maxs;
+    if(want < 1)
+        want = 1;
+    int64_t per = (M + want - 1) / want;
+    per = (per + BK - 1) / BK * BK;
+    p.m_per_split = (int)per;
+    p.splits = (int)((M + per - 1) / per);
+    return p;
+}
+
 static bool krsc_dense(const SagaTensorView *w)
 {
     const int C = w->dims[1], R = w->dims[2], S = w->dims[3];
@@ -307,6 +545,10 @@ size_t conv_mfma_workspace(int kind, const SagaTensorView *x, const SagaTensorVi
         return 0;
     if(kind == SAGA_CONV_BWD_DATA)
         return (size_t)g.K * g.C * g.R * g.S * sizeof(half_t) + 256;
+    if(kind == SAGA_CONV_BWD_FILTER) {
+        const FilterPlan p = plan_filter(g);
+        return (size_t)p.splits * g.K * g.R * g.S * g.C * sizeof(float) + 256;
+    }
     return 0;
 }
 
@@ -363,8 +605,37 @@ int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const 
     return launch_gather<true>(a, st);
 }
 
-int conv_mfma_bwd_filter(const SagaTensorView *, const SagaTensorView *, const SagaTensorView *, const ConvGeom &,
-                         float, float, void *, size_t, hipStream_t)
+int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, const SagaTensorView *dw,
+                         const ConvGeom &g, float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st)
 {
-    return SAGA_HIP_EUNSUPPORTED;
+    CLInfo lx, ldy;
+    if(!common_ok(x, dw, dy, g, &lx, &ldy))
+        return SAGA_HIP_EUNSUPPORTED;
+    if(g.K % 8 || ldy.pitch % 8 || !aligned16(dy->ptr))
+        return SAGA_HIP_EUNSUPPORTED;
+    const FilterPlan p = plan_filter(g);
+    const int64_t n = (int64_t)g.K * g.R * g.S * g.C;
+    const size_t need = (size_t)p.splits * n * sizeof(float);
+    if(!ws || ws_bytes < need || !aligned16(ws))
+        return SAGA_HIP_EWORKSPACE;
+    FilterArgs a;
+    a.x = (const half_t *)x->ptr;
+    a.dy = (const half_t *)dy->ptr;
+    a.partial = (float *)ws;
+    a.M = (int)ldy.rows;
+    a.K = g.K; a.C = g.C; a.RSC = g.R * g.S * g.C;
+    a.H = g.H; a.W = g.W; a.P = g.P; a.Q = g.Q; a.S = g.S;
+    a.pad = g.pad; a.stride = g.stride; a.dil = g.dil;
+    a.ldx = (int)lx.pitch; a.ldy = (int)ldy.pitch;
+    a.tiles_k = p.tiles_k; a.tiles_c = p.tiles_c;
+    a.splits = p.splits; a.m_per_split = p.m_per_split;
+    const int blocks = p.tiles_k * p.tiles_c * p.splits;
+    if(p.bm == 128)
+        conv_bwd_filter_mfma<128, 128><<<blocks, 256, 0, st>>>(a);
+    else
+        conv_bwd_filter_mfma<64, 128><<<blocks, 256, 0, st>>>(a);
+    SAGA_CHECK_LAUNCH();
+    filter_reduce<<<grid_for(n, 256, 256 * 8), 256, 0, st>>>((const float *)ws, (half_t *)dw->ptr, n, p.splits, alpha, beta);
+    SAGA_CHECK_LAUNCH();
+    return 0;
 }
