@@ -1,0 +1,968 @@
+// Node lowerings and graph transforms of the hip engine: every node type of the front end
+// becomes a short list of kernel-library calls (saga_hip.h), forward and backward.
+// Role of the reference's src/cuda/cuda_dnn.cpp; cited per lowering.
+#include <math.h>
+
+#include "hip_common.hpp"
+
+namespace saga {
+
+namespace {
+
+using T = std::shared_ptr<HipTensor>;
+
+saga_stream_t S(HipProgram &p) { return (saga_stream_t)p.m_ctx->m_stream; }
+
+T alias_of(const T &base, const Dims &dims, const std::vector<int64_t> &strides, int64_t offset,
+           const std::optional<const std::string> &name)
+{
+    return std::make_shared<HipTensor>(base->m_storage, dims, strides, offset, name);
+}
+
+// ---------------------------------------------------------------- convolution
+// reference: src/cuda/cuda_dnn.cpp:323-577
+
+struct ConvDesc {
+    SagaConvParams params;
+};
+
+struct ConvFwd : public HipOperation {
+    const T x_, w_, y_;
+    const SagaConvParams cp_;
+    float beta_ = 0;
+    ConvFwd(HipProgram &p, T x, T w, T y, SagaConvParams cp) : HipOperation("convfwd"), x_(x), w_(w), y_(y), cp_(cp)
+    {
+        const SagaTensorView vx = x->view(), vw = w->view(), vy = y->view();
+        p.m_ctx->m_workspace.request(saga_hip_conv2d_workspace_size(SAGA_CONV_FWD, &vx, &vw, &vy, &cp_));
+    }
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vx = x_->view(), vw = w_->view(), vy = y_->view();
+        chkSaga(saga_hip_conv2d_fwd(&vx, &vw, &vy, &cp_, 1.0f, beta_, p.m_ctx->m_workspace.ptr(),
+                                    p.m_ctx->m_workspace.size(), S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"x", x_}, {"w", w_}}; }
+    HipOpArgs listOutputs() const override { return {{"y", y_}}; }
+    float *getBeta(const T &t) override { return t == y_ ? &beta_ : nullptr; }
+};
+
+struct ConvBwdData : public HipOperation {
+    const T w_, dy_, dx_;
+    const SagaConvParams cp_;
+    float beta_ = 0;
+    ConvBwdData(HipProgram &p, T w, T dy, T dx, SagaConvParams cp)
+      : HipOperation("convbwddata"), w_(w), dy_(dy), dx_(dx), cp_(cp)
+    {
+        const SagaTensorView vx = dx->view(), vw = w->view(), vy = dy->view();
+        p.m_ctx->m_workspace.request(saga_hip_conv2d_workspace_size(SAGA_CONV_BWD_DATA, &vx, &vw, &vy, &cp_));
+    }
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vdy = dy_->view(), vw = w_->view(), vdx = dx_->view();
+        chkSaga(saga_hip_conv2d_bwd_data(&vdy, &vw, &vdx, &cp_, 1.0f, beta_, p.m_ctx->m_workspace.ptr(),
+                                         p.m_ctx->m_workspace.size(), S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"w", w_}, {"dy", dy_}}; }
+    HipOpArgs listOutputs() const override { return {{"dx", dx_}}; }
+    float *getBeta(const T &t) override { return t == dx_ ? &beta_ : nullptr; }
+};
+
+struct ConvBwdFilter : public HipOperation {
+    const T x_, dy_, dw_;
+    const SagaConvParams cp_;
+    float beta_ = 0;
+    ConvBwdFilter(HipProgram &p, T x, T dy, T dw, SagaConvParams cp)
+      : HipOperation("convbwdfilter"), x_(x), dy_(dy), dw_(dw), cp_(cp)
+    {
+        const SagaTensorView vx = x->view(), vw = dw->view(), vy = dy->view();
+        p.m_ctx->m_workspace.request(saga_hip_conv2d_workspace_size(SAGA_CONV_BWD_FILTER, &vx, &vw, &vy, &cp_));
+    }
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vx = x_->view(), vdy = dy_->view(), vdw = dw_->view();
+        chkSaga(saga_hip_conv2d_bwd_filter(&vx, &vdy, &vdw, &cp_, 1.0f, beta_, p.m_ctx->m_workspace.ptr(),
+                                           p.m_ctx->m_workspace.size(), S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"x", x_}, {"dy", dy_}}; }
+    HipOpArgs listOutputs() const override { return {{"dw", dw_}}; }
+    float *getBeta(const T &t) override { return t == dw_ ? &beta_ : nullptr; }
+};
+
+// y += b, b broadcast over the channel axis (reference: CudnnAddTensor, :39-68)
+struct BiasAdd : public HipOperation {
+    const T b_, y_;
+    BiasAdd(T b, T y) : HipOperation("biasadd"), b_(b), y_(y) {}
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vy = y_->view(), vb = b_->view();
+        chkSaga(saga_hip_bias_add(&vy, &vb, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"b", b_}, {"y", y_}}; }
+    HipOpArgs listOutputs() const override { return {{"y", y_}}; }
+    // the output is read as well as written; report it as accumulating so that liveness sees the read
+    float one_ = 1.0f;
+    float *getBeta(const T &t) override { return t == y_ ? &one_ : nullptr; }
+};
+
+struct BiasBwd : public HipOperation {
+    const T dy_, db_;
+    float beta_ = 0;
+    BiasBwd(T dy, T db) : HipOperation("biasbwd"), dy_(dy), db_(db) {}
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vdy = dy_->view(), vdb = db_->view();
+        chkSaga(saga_hip_bias_bwd(&vdy, &vdb, beta_, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"dy", dy_}}; }
+    HipOpArgs listOutputs() const override { return {{"db", db_}}; }
+    float *getBeta(const T &t) override { return t == db_ ? &beta_ : nullptr; }
+};
+
+void conv_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
+{
+    auto x = p.lower(pu, n.m_inputs["x"]);
+    auto y = p.lower(pu, n.m_outputs["y"]);
+    auto w = p.lower(pu, n.m_inputs["w"]);
+    auto b = n.m_inputs.has("b") ? p.lower(pu, n.m_inputs["b"], y->m_dims.size()) : nullptr;
+
+    SagaConvParams cp;
+    cp.pad = n.m_attributes.get("pad", 0);
+    cp.stride = n.m_attributes.get("stride", 1);
+    cp.dilation = 1; // like the reference backend, which ignores the attribute (:227-231)
+    cp.group = n.m_attributes.get("group", 1);
+    const bool transpose = n.m_attributes.get("transpose", false);
+    const bool training = p.m_pt == ProgramType::TRAINING;
+
+    if(!transpose) {
+        pu.fwd(std::make_shared<ConvFwd>(p, x, w, y, cp));
+        if(b)
+            pu.fwd(std::make_shared<BiasAdd>(b, y));
+        if(!training)
+            return;
+        auto dy = p.lowerGrad(pu, n.m_outputs["y"]);
+        if(b) {
+            auto db = p.lowerGrad(pu, n.m_inputs["b"], y->m_dims.size());
+            pu.bwd(std::make_shared<BiasBwd>(dy, db));
+            p.upd(n.m_inputs["b"], b, db);
+        }
+        auto dw = p.lowerGrad(pu, n.m_inputs["w"]);
+        pu.bwd(std::make_shared<ConvBwdFilter>(p, x, dy, dw, cp));
+        p.upd(n.m_inputs["w"], w, dw);
+        if(auto dx = p.lowerGrad(pu, n.m_inputs["x"]))
+            pu.bwd(std::make_shared<ConvBwdData>(p, w, dy, dx, cp));
+    } else {
+        // transposed convolution: the three kernels with x and y exchanged (:542-574)
+        pu.fwd(std::make_shared<ConvBwdData>(p, w, x, y, cp));
+        if(b)
+            pu.fwd(std::make_shared<BiasAdd>(b, y));
+        if(!training)
+            return;
+        auto dy = p.lowerGrad(pu, n.m_outputs["y"]);
+        if(b) {
+            auto db = p.lowerGrad(pu, n.m_inputs["b"], y->m_dims.size());
+            pu.bwd(std::make_shared<BiasBwd>(dy, db));
+            p.upd(n.m_inputs["b"], b, db);
+        }
+        auto dw = p.lowerGrad(pu, n.m_inputs["w"]);
+        pu.bwd(std::make_shared<ConvBwdFilter>(p, dy, x, dw, cp));
+        p.upd(n.m_inputs["w"], w, dw);
+        if(auto dx = p.lowerGrad(pu, n.m_inputs["x"]))
+            pu.bwd(std::make_shared<ConvFwd>(p, dy, w, dx, cp));
+    }
+}
+REGISTER_HIP_OP("conv", conv_setup);
+
+// ---------------------------------------------------------------- activations
+// reference: src/cuda/cuda_dnn.cpp:610-806
+
+struct ActFwd : public HipOperation {
+    const T x_, y_;
+    const int mode_;
+    const float alpha_;
+    float beta_ = 0;
+    ActFwd(T x, T y, int mode, float alpha) : HipOperation("actfwd"), x_(x), y_(y), mode_(mode), alpha_(alpha) {}
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vx = x_->view(), vy = y_->view();
+        chkSaga(saga_hip_act_fwd(mode_, alpha_, &vx, &vy, beta_, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"x", x_}}; }
+    HipOpArgs listOutputs() const override { return {{"y", y_}}; }
+    float *getBeta(const T &t) override { return t == y_ ? &beta_ : nullptr; }
+    std::string info() const override
+    {
+        static const char *names[] = {"relu", "sigmoid", "tanh", "swish", "leakyrelu"};
+        return names[mode_];
+    }
+};
+
+struct ActBwd : public HipOperation {
+    const T x_, y_, dx_, dy_;
+    const int mode_;
+    const float alpha_;
+    float beta_ = 0;
+    ActBwd(T x, T y, T dx, T dy, int mode, float alpha)
+      : HipOperation("actbwd"), x_(x), y_(y), dx_(dx), dy_(dy), mode_(mode), alpha_(alpha)
+    {
+    }
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vx = x_->view(), vy = y_->view(), vdy = dy_->view(), vdx = dx_->view();
+        chkSaga(saga_hip_act_bwd(mode_, alpha_, &vx, &vy, &vdy, &vdx, beta_, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"x", x_}, {"y", y_}, {"dy", dy_}}; }
+    HipOpArgs listOutputs() const override { return {{"dx", dx_}}; }
+    float *getBeta(const T &t) override { return t == dx_ ? &beta_ : nullptr; }
+};
+
+void activation_setup(HipProgram &p, HipProgramUnit &pu, const Node &n, int mode, float alpha)
+{
+    auto x = p.lower(pu, n.m_inputs["x"]);
+    auto y = p.lowerLike(pu, n.m_outputs["y"], *x);
+    pu.fwd(std::make_shared<ActFwd>(x, y, mode, alpha));
+    if(p.m_pt == ProgramType::INFERENCE)
+        return;
+    auto dx = p.lowerGrad(pu, n.m_inputs["x"]);
+    auto dy = p.lowerGrad(pu, n.m_outputs["y"]);
+    pu.bwd(std::make_shared<ActBwd>(x, y, dx, dy, mode, alpha));
+}
+
+void relu_setup(HipProgram &p, HipProgramUnit &pu, const Node &n) { activation_setup(p, pu, n, SAGA_ACT_RELU, 0); }
+void sigmoid_setup(HipProgram &p, HipProgramUnit &pu, const Node &n) { activation_setup(p, pu, n, SAGA_ACT_SIGMOID, 0); }
+void tanh_setup(HipProgram &p, HipProgramUnit &pu, const Node &n) { activation_setup(p, pu, n, SAGA_ACT_TANH, 0); }
+void swish_setup(HipProgram &p, HipProgramUnit &pu, const Node &n) { activation_setup(p, pu, n, SAGA_ACT_SWISH, 0); }
+void leakyrelu_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
+{
+    activation_setup(p, pu, n, SAGA_ACT_LEAKYRELU, n.m_attributes.get("alpha", 0.01f));
+}
+REGISTER_HIP_OP("relu", relu_setup);
+REGISTER_HIP_OP("elu", relu_setup); // the reference registers relu for "elu" as well (:732)
+REGISTER_HIP_OP("sigmoid", sigmoid_setup);
+REGISTER_HIP_OP("tanh", tanh_setup);
+REGISTER_HIP_OP("swish", swish_setup);
+REGISTER_HIP_OP("leakyrelu", leakyrelu_setup);
+
+// ---------------------------------------------------------------- pooling
+// reference: src/cuda/cuda_dnn.cpp:810-926
+
+struct PoolFwd : public HipOperation {
+    const T x_, y_;
+    const int mode_, size_, pad_, stride_;
+    PoolFwd(T x, T y, int mode, int size, int pad, int stride)
+      : HipOperation("poolfwd"), x_(x), y_(y), mode_(mode), size_(size), pad_(pad), stride_(stride)
+    {
+    }
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vx = x_->view(), vy = y_->view();
+        chkSaga(saga_hip_pool_fwd(mode_, &vx, &vy, nullptr, size_, pad_, stride_, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"x", x_}}; }
+    HipOpArgs listOutputs() const override { return {{"y", y_}}; }
+    std::string info() const override { return mode_ == SAGA_POOL_MAX ? "max" : "avg"; }
+};
+
+struct PoolBwd : public HipOperation {
+    const T x_, y_, dx_, dy_;
+    const int mode_, size_, pad_, stride_;
+    float beta_ = 0;
+    PoolBwd(T x, T y, T dx, T dy, int mode, int size, int pad, int stride)
+      : HipOperation("poolbwd"), x_(x), y_(y), dx_(dx), dy_(dy), mode_(mode), size_(size), pad_(pad), stride_(stride)
+    {
+    }
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vx = x_->view(), vy = y_->view(), vdy = dy_->view(), vdx = dx_->view();
+        chkSaga(saga_hip_pool_bwd(mode_, &vx, &vy, &vdy, &vdx, size_, pad_, stride_, beta_, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"x", x_}, {"y", y_}, {"dy", dy_}}; }
+    HipOpArgs listOutputs() const override { return {{"dx", dx_}}; }
+    float *getBeta(const T &t) override { return t == dx_ ? &beta_ : nullptr; }
+};
+
+void pooling_setup(HipProgram &p, HipProgramUnit &pu, const Node &n, int mode)
+{
+    auto x = p.lower(pu, n.m_inputs["x"]);
+    auto y = p.lowerLike(pu, n.m_outputs["y"], *x);
+    const int size = n.m_attributes.get("global", false) ? (int)x->m_dims[2] : n.m_attributes.get("size", 1);
+    const int pad = n.m_attributes.get("pad", 0);
+    const int stride = n.m_attributes.get("stride", 1);
+    pu.fwd(std::make_shared<PoolFwd>(x, y, mode, size, pad, stride));
+    if(p.m_pt == ProgramType::INFERENCE)
+        return;
+    auto dx = p.lowerGrad(pu, n.m_inputs["x"]);
+    auto dy = p.lowerGrad(pu, n.m_outputs["y"]);
+    pu.bwd(std::make_shared<PoolBwd>(x, y, dx, dy, mode, size, pad, stride));
+}
+void maxpool_setup(HipProgram &p, HipProgramUnit &pu, const Node &n) { pooling_setup(p, pu, n, SAGA_POOL_MAX); }
+void avgpool_setup(HipProgram &p, HipProgramUnit &pu, const Node &n) { pooling_setup(p, pu, n, SAGA_POOL_AVG); }
+REGISTER_HIP_OP("maxpool", maxpool_setup);
+REGISTER_HIP_OP("avgpool", avgpool_setup);
+
+// ---------------------------------------------------------------- fully connected
+// reference: src/cuda/cuda_dnn.cpp:968-1130 (column-major cuBLAS calls restated row-major)
+
+struct Gemm : public HipOperation {
+    const int ta_, tb_, m_, n_, k_;
+    const T a_, b_, c_;
+    const int lda_, ldb_, ldc_;
+    float beta_ = 0;
+    Gemm(int ta, int tb, int m, int n, int k, T a, int lda, T b, int ldb, T c, int ldc, const char *name)
+      : HipOperation(name), ta_(ta), tb_(tb), m_(m), n_(n), k_(k), a_(a), b_(b), c_(c), lda_(lda), ldb_(ldb), ldc_(ldc)
+    {
+        if(a->m_data_type != b->m_data_type || a->m_data_type != c->m_data_type)
+            throw std::runtime_error("fc: operand data types differ");
+        if(!a->rowMajor() || !b->rowMajor() || !c->rowMajor())
+            throw std::runtime_error("fc: operands must be row-major matrices");
+    }
+    void exec(HipProgram &p) override
+    {
+        chkSaga(saga_hip_gemm(ta_, tb_, m_, n_, k_, 1.0f, a_->deviceMem(), lda_, b_->deviceMem(), ldb_, beta_,
+                              c_->deviceMem(), ldc_, (int)a_->m_data_type, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"a", a_}, {"b", b_}}; }
+    HipOpArgs listOutputs() const override { return {{"c", c_}}; }
+    float *getBeta(const T &t) override { return t == c_ ? &beta_ : nullptr; }
+};
+
+void fc_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
+{
+    auto x = p.lower(pu, n.m_inputs["x"]);
+    auto y = p.lower(pu, n.m_outputs["y"]);
+    auto w = p.lower(pu, n.m_inputs["w"]);
+    auto b = n.m_inputs.has("b") ? p.lower(pu, n.m_inputs["b"], 2) : nullptr;
+    const bool transW = n.m_attributes.get("transW", false);
+    const int in = x->m_dims[1], out = y->m_dims[1], batch = x->m_dims[0];
+
+    // y[batch,out] = x[batch,in] * W ; W stored [in,out], or [out,in] when transW
+    pu.fwd(std::make_shared<Gemm>(0, transW ? 1 : 0, batch, out, in, x, in, w, transW ? in : out, y, out,
+                                  transW ? "fc.fwd.t" : "fc.fwd.n"));
+    if(b)
+        pu.fwd(std::make_shared<BiasAdd>(b, y));
+    if(p.m_pt == ProgramType::INFERENCE)
+        return;
+
+    auto dx = p.lowerGrad(pu, n.m_inputs["x"]);
+    auto dy = p.lowerGrad(pu, n.m_outputs["y"]);
+    auto dw = p.lowerGrad(pu, n.m_inputs["w"]);
+    if(transW) // dW[out,in] = dy^T x
+        pu.bwd(std::make_shared<Gemm>(1, 0, out, in, batch, dy, out, x, in, dw, in, "fc.bwd.weights.t"));
+    else // dW[in,out] = x^T dy
+        pu.bwd(std::make_shared<Gemm>(1, 0, in, out, batch, x, in, dy, out, dw, out, "fc.bwd.weights.n"));
+    p.upd(n.m_inputs["w"], w, dw);
+    if(b) {
+        auto db = p.lowerGrad(pu, n.m_inputs["b"], 2);
+        pu.bwd(std::make_shared<BiasBwd>(dy, db)); // column sums of dy
+        p.upd(n.m_inputs["b"], b, db);
+    }
+    if(dx) // dx[batch,in] = dy * W^T
+        pu.bwd(std::make_shared<Gemm>(0, transW ? 0 : 1, batch, in, out, dy, out, w, transW ? in : out, dx, in,
+                                      transW ? "fc.bwd.data.t" : "fc.bwd.data.n"));
+}
+REGISTER_HIP_OP("fc", fc_setup);
+
+// ---------------------------------------------------------------- convert
+// reference: src/cuda/cuda_dnn.cpp:1134-1241
+
+struct Convert : public HipOperation {
+    const T x_, y_;
+    const float scale_;
+    Convert(T x, T y, float scale) : HipOperation("convert"), x_(x), y_(y), scale_(scale) {}
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vx = x_->view(), vy = y_->view();
+        chkSaga(saga_hip_convert(&vx, &vy, scale_, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"x", x_}}; }
+    HipOpArgs listOutputs() const override { return {{"y", y_}}; }
+};
+
+void convert_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
+{
+    const float scale = n.m_attributes.get("scale", 1.0f);
+    auto xh = n.m_inputs["x"], yh = n.m_outputs["y"];
+    auto x = p.lower(pu, xh);
+    if(xh->m_data_type == yh->m_data_type && scale == 1.0f) {
+        p.m_ctx->m_tensors[yh] = alias_of(x, x->m_dims, x->m_strides, x->m_offset, xh->namePostfix("nop-convert"));
+        return;
+    }
+    // the output takes the layout the program would give its type (fp16 -> channels-last)
+    auto y = p.lower(pu, yh);
+    pu.fwd(std::make_shared<Convert>(x, y, scale));
+}
+REGISTER_HIP_OP("convert", convert_setup);
+
+Nodes convert_transform(HipProgram &, HipProgramUnit &, const Nodes &input)
+{
+    Nodes nodes = input;
+    bool again = true;
+    while(again) {
+        again = false;
+        for(auto &n : nodes) {
+            if(n->m_type != "convert")
+                continue;
+            auto it = nodes.findSingleDownStreamNode(n->y(), "convert");
+            if(it == nodes.end())
+                continue;
+            auto b = *it;
+            auto fused = std::make_shared<Node>("convert");
+            fused->m_inputs["x"] = n->m_inputs["x"];
+            fused->m_outputs["y"] = b->m_outputs["y"];
+            fused->m_attributes["scale"] = n->m_attributes.get("scale", 1.0f) * b->m_attributes.get("scale", 1.0f);
+            fused->m_attributes["datatype"] = b->m_attributes.get("datatype", (int)b->y()->m_data_type);
+            n = fused;
+            nodes.erase(it);
+            again = true;
+            break;
+        }
+    }
+    return nodes;
+}
+REGISTER_HIP_TRANSFORM(200, ProgramType::INFERENCE | ProgramType::TRAINING, convert_transform);
+
+// ---------------------------------------------------------------- classifier head
+// reference: src/cuda/cuda_dnn.cpp:1244-1355
+
+struct CatClassifierFwd : public HipOperation {
+    const T x_, y_;
+    CatClassifierFwd(T x, T y) : HipOperation("catclassifierfwd"), x_(x), y_(y) {}
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vx = x_->view();
+        chkSaga(saga_hip_catclassifier_fwd(&vx, (int32_t *)y_->deviceMem(), S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"x", x_}}; }
+    HipOpArgs listOutputs() const override { return {{"y", y_}}; }
+};
+
+struct CatClassifierBwd : public HipOperation {
+    const T x_, y_, dx_, dy_;
+    T loss_;
+    CatClassifierBwd(T x, T y, T dx, T dy, T loss)
+      : HipOperation("catclassifierbwd"), x_(x), y_(y), dx_(dx), dy_(dy), loss_(loss)
+    {
+    }
+    void exec(HipProgram &p) override
+    {
+        const int n = x_->m_dims[0];
+        float scale = 1.0f / n;
+        if(x_->m_data_type == Tensor::DataType::HALF)
+            scale *= p.m_mp_scaling; // loss scaling enters the backward pass here (:1315)
+        const SagaTensorView vx = x_->view(), vdx = dx_->view();
+        chkSaga(saga_hip_catclassifier_bwd(&vx, &vdx, (const int32_t *)y_->deviceMem(),
+                                           (const int32_t *)dy_->deviceMem(),
+                                           loss_ ? (float *)loss_->deviceMem() : nullptr, scale, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"x", x_}, {"y", y_}, {"dy", dy_}}; }
+    HipOpArgs listOutputs() const override
+    {
+        HipOpArgs r{{"dx", dx_}};
+        if(loss_)
+            r.push_back({"loss", loss_});
+        return r;
+    }
+    bool killOutput(const std::shared_ptr<HipStorage> &s) override
+    {
+        if(loss_ && loss_->m_storage == s) {
+            loss_.reset();
+            return true;
+        }
+        return false;
+    }
+};
+
+void catclassifier_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
+{
+    auto x = p.lower(pu, n.m_inputs["x"]);
+    auto y = p.lower(pu, n.m_outputs["y"]);
+    pu.fwd(std::make_shared<CatClassifierFwd>(x, y));
+    if(p.m_pt == ProgramType::INFERENCE)
+        return;
+    auto dx = p.lowerGrad(pu, n.m_inputs["x"]);
+    auto dy = p.lowerGrad(pu, n.m_outputs["y"]);
+    // one loss value per sample; a front end that declares fewer elements gets a batch-sized tensor
+    auto lh = n.m_outputs["loss"];
+    T loss;
+    auto it = p.m_ctx->m_tensors.find(lh);
+    if(it != p.m_ctx->m_tensors.end()) {
+        loss = it->second;
+    } else {
+        Dims ld = lh->m_dims.batch(pu.m_batch_size);
+        if((int)ld.elements() < (int)x->m_dims[0])
+            ld = Dims{(int64_t)(int)x->m_dims[0]};
+        loss = std::make_shared<HipTensor>(Tensor::DataType::FLOAT, ld, HipLayout::NCHW, p.m_ctx.get(), lh->m_name);
+        p.m_ctx->m_tensors[lh] = loss;
+    }
+    if((int)loss->m_dims.elements() < (int)x->m_dims[0])
+        throw std::runtime_error("catclassifier: loss tensor smaller than the batch");
+    pu.bwd(std::make_shared<CatClassifierBwd>(x, y, dx, dy, loss));
+}
+REGISTER_HIP_OP("catclassifier", catclassifier_setup);
+
+// ---------------------------------------------------------------- batch normalisation
+// reference: src/cuda/cuda_dnn.cpp:1620-1826 (plain) and :1983-2369 (fused with relu / add)
+
+struct BnInference : public HipOperation {
+    const T x_, z_, s_, b_, m_, v_, y_;
+    const float eps_;
+    const int flags_;
+    BnInference(T x, T z, T s, T b, T m, T v, T y, float eps, int flags)
+      : HipOperation(flags ? "bninf.fused" : "bninf"), x_(x), z_(z), s_(s), b_(b), m_(m), v_(v), y_(y), eps_(eps), flags_(flags)
+    {
+    }
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vx = x_->view(), vy = y_->view();
+        SagaTensorView vz;
+        if(z_)
+            vz = z_->view();
+        chkSaga(saga_hip_bn_infer(&vx, z_ ? &vz : nullptr, &vy, (const float *)s_->deviceMem(),
+                                  (const float *)b_->deviceMem(), (const float *)m_->deviceMem(),
+                                  (const float *)v_->deviceMem(), eps_, flags_, S(p)));
+    }
+    HipOpArgs listInputs() const override
+    {
+        HipOpArgs r{{"x", x_}, {"s", s_}, {"b", b_}, {"m", m_}, {"v", v_}};
+        if(z_)
+            r.push_back({"z", z_});
+        return r;
+    }
+    HipOpArgs listOutputs() const override { return {{"y", y_}}; }
+};
+
+struct BnTrain : public HipOperation {
+    const T x_, z_, s_, b_, m_, v_, y_, sm_, sv_;
+    const float eps_;
+    const int flags_;
+    float expavg_ = NAN;
+    float m_beta_ = 1.0f, v_beta_ = 1.0f; // running statistics are read-modify-write
+    BnTrain(HipProgram &p, T x, T z, T s, T b, T m, T v, T y, T sm, T sv, float eps, int flags)
+      : HipOperation(flags ? "bntrain.fused" : "bntrain")
+      , x_(x), z_(z), s_(s), b_(b), m_(m), v_(v), y_(y), sm_(sm), sv_(sv), eps_(eps), flags_(flags)
+    {
+        const SagaTensorView vx = x->view();
+        p.m_ctx->m_workspace.request(saga_hip_bn_workspace_size(&vx));
+    }
+    void exec(HipProgram &p) override
+    {
+        // first step of auto-initialised statistics adopts the batch statistics outright (:1694-1708)
+        if(!std::isfinite(expavg_))
+            expavg_ = m_->m_auto_initialized ? 1.0f : p.m_pc.bn_expavg;
+        const SagaTensorView vx = x_->view(), vy = y_->view();
+        SagaTensorView vz;
+        if(z_)
+            vz = z_->view();
+        chkSaga(saga_hip_bn_train_fwd(&vx, z_ ? &vz : nullptr, &vy, (const float *)s_->deviceMem(),
+                                      (const float *)b_->deviceMem(), (float *)m_->deviceMem(),
+                                      (float *)v_->deviceMem(), (float *)sm_->deviceMem(), (float *)sv_->deviceMem(),
+                                      eps_, expavg_, flags_, p.m_ctx->m_workspace.ptr(), p.m_ctx->m_workspace.size(),
+                                      S(p)));
+        expavg_ = p.m_pc.bn_expavg;
+    }
+    HipOpArgs listInputs() const override
+    {
+        HipOpArgs r{{"x", x_}, {"s", s_}, {"b", b_}};
+        if(z_)
+            r.push_back({"z", z_});
+        return r;
+    }
+    HipOpArgs listOutputs() const override { return {{"y", y_}, {"m", m_}, {"v", v_}, {"sm", sm_}, {"sv", sv_}}; }
+    float *getBeta(const T &t) override
+    {
+        if(t == m_)
+            return &m_beta_;
+        if(t == v_)
+            return &v_beta_;
+        return nullptr;
+    }
+};
+
+struct BnBwd : public HipOperation {
+    const std::shared_ptr<BnTrain> fwd_;
+    const T dy_, dx_;
+    T dz_;
+    const T ds_, db_;
+    int flags_;
+    float dx_beta_ = 0, dz_beta_ = 0, ds_beta_ = 0, db_beta_ = 0;
+    BnBwd(std::shared_ptr<BnTrain> fwd, T dy, T dx, T dz, T ds, T db, int flags)
+      : HipOperation(flags ? "bnbwd.fused" : "bnbwd"), fwd_(fwd), dy_(dy), dx_(dx), dz_(dz), ds_(ds), db_(db), flags_(flags)
+    {
+    }
+    void exec(HipProgram &p) override
+    {
+        const bool relu = flags_ & SAGA_BN_RELU;
+        const SagaTensorView vx = fwd_->x_->view(), vy = fwd_->y_->view(), vdy = dy_->view(), vdx = dx_->view();
+        SagaTensorView vdz;
+        if(dz_)
+            vdz = dz_->view();
+        chkSaga(saga_hip_bn_bwd(&vx, relu ? &vy : nullptr, &vdy, &vdx, dz_ ? &vdz : nullptr,
+                                (const float *)fwd_->s_->deviceMem(), (const float *)fwd_->sm_->deviceMem(),
+                                (const float *)fwd_->sv_->deviceMem(), (float *)ds_->deviceMem(),
+                                (float *)db_->deviceMem(), dx_beta_, dz_beta_, ds_beta_, flags_,
+                                p.m_ctx->m_workspace.ptr(), p.m_ctx->m_workspace.size(), S(p)));
+    }
+    HipOpArgs listInputs() const override
+    {
+        HipOpArgs r{{"x", fwd_->x_}, {"dy", dy_}, {"s", fwd_->s_}, {"sm", fwd_->sm_}, {"sv", fwd_->sv_}};
+        if(flags_ & SAGA_BN_RELU)
+            r.push_back({"y", fwd_->y_});
+        return r;
+    }
+    HipOpArgs listOutputs() const override
+    {
+        HipOpArgs r{{"dx", dx_}, {"ds", ds_}, {"db", db_}};
+        if(dz_)
+            r.push_back({"dz", dz_});
+        return r;
+    }
+    bool killOutput(const std::shared_ptr<HipStorage> &s) override
+    {
+        if(dz_ && dz_->m_storage == s) {
+            dz_.reset();
+            return true;
+        }
+        return false;
+    }
+    float *getBeta(const T &t) override
+    {
+        if(t == dx_)
+            return &dx_beta_;
+        if(dz_ && t == dz_)
+            return &dz_beta_;
+        if(t == ds_)
+            return &ds_beta_;
+        if(t == db_)
+            return &db_beta_;
+        return nullptr;
+    }
+};
+
+// x0 = normalised input, x1 = residual (optional); flags from the "relu" attribute
+void batchnorm_lower(HipProgram &p, HipProgramUnit &pu, const Node &n, std::shared_ptr<Tensor> xh,
+                     std::shared_ptr<Tensor> zh, int flags)
+{
+    auto x = p.lower(pu, xh);
+    auto z = zh ? p.lower(pu, zh) : nullptr;
+    auto y = p.lowerLike(pu, n.m_outputs["y"], *x);
+    auto s = p.lower(pu, n.m_inputs["s"], 2);
+    auto b = p.lower(pu, n.m_inputs["b"], 2);
+    auto m = p.lower(pu, n.m_inputs["m"], 2);
+    auto v = p.lower(pu, n.m_inputs["v"], 2);
+    for(const auto &t : {s, b, m, v})
+        if(t->m_data_type != Tensor::DataType::FLOAT || (int)t->m_dims.elements() != (int)x->m_dims[1])
+            throw std::runtime_error("batchnorm parameters must be fp32 vectors of C elements");
+    const float eps = n.m_attributes.get("epsilon", 1e-5f);
+
+    if(p.m_pt == ProgramType::INFERENCE) {
+        pu.fwd(std::make_shared<BnInference>(x, z, s, b, m, v, y, eps, flags));
+        return;
+    }
+    auto sm = std::make_shared<HipTensor>(Tensor::DataType::FLOAT, *m, m->namePostfix("smean"));
+    auto sv = std::make_shared<HipTensor>(Tensor::DataType::FLOAT, *v, v->namePostfix("svar"));
+    auto f = std::make_shared<BnTrain>(p, x, z, s, b, m, v, y, sm, sv, eps, flags);
+    pu.fwd(f);
+
+    auto dx = p.lowerGrad(pu, xh);
+    auto dz = zh ? p.lowerGrad(pu, zh) : nullptr;
+    auto dy = p.lowerGrad(pu, n.m_outputs["y"]);
+    auto ds = p.lowerGrad(pu, n.m_inputs["s"], 2);
+    auto db = p.lowerGrad(pu, n.m_inputs["b"], 2);
+    pu.bwd(std::make_shared<BnBwd>(f, dy, dx, dz, ds, db, flags));
+    p.upd(n.m_inputs["s"], s, ds);
+    p.upd(n.m_inputs["b"], b, db);
+}
+
+void batchnorm_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
+{
+    batchnorm_lower(p, pu, n, n.m_inputs["x"], nullptr, 0);
+}
+REGISTER_HIP_OP("batchnorm", batchnorm_setup);
+
+void batchnorm_fused_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
+{
+    int flags = 0;
+    std::shared_ptr<Tensor> z;
+    if(n.m_attributes.get("relu", false))
+        flags |= SAGA_BN_RELU;
+    if(n.m_inputs.has("x1")) {
+        z = n.m_inputs["x1"];
+        flags |= SAGA_BN_ADD;
+    }
+    batchnorm_lower(p, pu, n, n.m_inputs["x0"], z, flags);
+}
+REGISTER_HIP_OP("batchnorm.persistent", batchnorm_fused_setup);
+
+bool single_consumer(const Nodes &nodes, const std::shared_ptr<Tensor> &t)
+{
+    int uses = 0;
+    for(const auto &n : nodes)
+        for(const auto &in : n->m_inputs)
+            if(in.second == t)
+                uses++;
+    return uses == 1;
+}
+
+std::shared_ptr<Node> fuse_bn(std::shared_ptr<Node> bn, std::shared_ptr<Node> sum, std::shared_ptr<Node> relu)
+{
+    auto nn = std::make_shared<Node>("batchnorm.persistent", bn->m_name);
+    nn->m_inputs["x0"] = bn->m_inputs["x"];
+    if(sum) {
+        const bool bn_is_x0 = sum->m_inputs["x0"] == bn->m_outputs["y"];
+        nn->m_inputs["x1"] = sum->m_inputs[bn_is_x0 ? "x1" : "x0"];
+    }
+    for(const char *k : {"s", "b", "m", "v"})
+        nn->m_inputs[k] = bn->m_inputs[k];
+    if(bn->m_attributes.find("epsilon") != bn->m_attributes.end())
+        nn->m_attributes["epsilon"] = bn->m_attributes["epsilon"];
+    if(relu)
+        nn->m_attributes["relu"] = true;
+    nn->m_outputs["y"] = relu ? relu->m_outputs["y"] : bn->m_outputs["y"];
+    return nn;
+}
+
+// bn,relu / bn,sum,relu runs of ADJACENT nodes become one fused node
+// (reference: batchnorm_relu_transform, :2326-2369; that one is limited to fp16 channels-last
+// training programs, the kernels here take any type and layout and fuse in inference too).
+Nodes batchnorm_relu_transform(HipProgram &p, HipProgramUnit &, const Nodes &nodes)
+{
+    if(p.m_pc.disable_op_fusing)
+        return nodes;
+    Nodes r;
+    const ssize_t count = nodes.size();
+    for(ssize_t i = 0; i < count; i++) {
+        std::shared_ptr<Node> n = nodes[i];
+        if(n->m_type == "batchnorm") {
+            const auto bn_y = n->m_outputs["y"];
+            if(i + 1 < count && nodes[i + 1]->m_type == "relu" && nodes[i + 1]->m_inputs["x"] == bn_y &&
+               single_consumer(nodes, bn_y)) {
+                n = fuse_bn(nodes[i], nullptr, nodes[i + 1]);
+                i += 1;
+            } else if(i + 2 < count && nodes[i + 1]->m_type == "sum" && nodes[i + 2]->m_type == "relu" &&
+                      (nodes[i + 1]->m_inputs["x0"] == bn_y || nodes[i + 1]->m_inputs["x1"] == bn_y) &&
+                      nodes[i + 1]->m_inputs["x0"] != nodes[i + 1]->m_inputs["x1"] &&
+                      nodes[i + 2]->m_inputs["x"] == nodes[i + 1]->m_outputs["y"] && single_consumer(nodes, bn_y) &&
+                      single_consumer(nodes, nodes[i + 1]->m_outputs["y"])) {
+                n = fuse_bn(nodes[i], nodes[i + 1], nodes[i + 2]);
+                i += 2;
+            }
+        }
+        r.push_back(n);
+    }
+    return r;
+}
+REGISTER_HIP_TRANSFORM(500, ProgramType::INFERENCE | ProgramType::TRAINING, batchnorm_relu_transform);
+
+// ---------------------------------------------------------------- sum / add / softmax
+// reference: src/cuda/cuda_dnn.cpp:1830-1964
+
+struct AddOp : public HipOperation {
+    const T a_, b_, c_;
+    AddOp(T a, T b, T c) : HipOperation("add"), a_(a), b_(b), c_(c) {}
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView va = a_->view(), vb = b_->view(), vc = c_->view();
+        chkSaga(saga_hip_add(&va, &vb, &vc, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"a", a_}, {"b", b_}}; }
+    HipOpArgs listOutputs() const override { return {{"c", c_}}; }
+};
+
+// dst = src + beta*dst (reference: CudnnTransform, :72-99); also converts between layouts
+struct Transform : public HipOperation {
+    const T a_, b_;
+    float beta_ = 0;
+    Transform(T a, T b, const char *name = "transform") : HipOperation(name), a_(a), b_(b) {}
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView va = a_->view(), vb = b_->view();
+        chkSaga(saga_hip_axpby(&va, &vb, 1.0f, beta_, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"a", a_}}; }
+    HipOpArgs listOutputs() const override { return {{"b", b_}}; }
+    float *getBeta(const T &t) override { return t == b_ ? &beta_ : nullptr; }
+};
+
+void sum_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
+{
+    auto x0 = p.lower(pu, n.m_inputs["x0"]);
+    auto x1 = p.lower(pu, n.m_inputs["x1"]);
+    auto y = p.lowerLike(pu, n.m_outputs["y"], *x0);
+    pu.fwd(std::make_shared<AddOp>(x0, x1, y));
+    if(p.m_pt == ProgramType::INFERENCE)
+        return;
+    auto dy = p.lowerGrad(pu, n.m_outputs["y"]);
+    pu.bwd(std::make_shared<Transform>(dy, p.lowerGrad(pu, n.m_inputs["x0"])));
+    pu.bwd(std::make_shared<Transform>(dy, p.lowerGrad(pu, n.m_inputs["x1"])));
+}
+REGISTER_HIP_OP("sum", sum_setup);
+
+// y = x + b with b either of x's shape or one value per channel (ONNX Add of a bias); inference only
+struct AddBias : public HipOperation {
+    const T x_, b_, y_;
+    AddBias(T x, T b, T y) : HipOperation("add.bias"), x_(x), b_(b), y_(y) {}
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vx = x_->view(), vy = y_->view(), vb = b_->view();
+        chkSaga(saga_hip_axpby(&vx, &vy, 1.0f, 0.0f, S(p)));
+        chkSaga(saga_hip_bias_add(&vy, &vb, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"x", x_}, {"b", b_}}; }
+    HipOpArgs listOutputs() const override { return {{"y", y_}}; }
+};
+
+void add_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
+{
+    if(p.m_pt != ProgramType::INFERENCE)
+        throw std::runtime_error{"Add not supported for backprop"};
+    auto x = p.lower(pu, n.m_inputs["x"]);
+    auto y = p.lowerLike(pu, n.m_outputs["y"], *x);
+    auto bh = n.m_inputs["b"];
+    if(bh->m_dims.elements() == x->m_dims.elements()) {
+        auto b = p.lower(pu, bh);
+        pu.fwd(std::make_shared<AddOp>(x, b, y));
+    } else {
+        auto b = p.lower(pu, bh);
+        if((int)b->m_dims.elements() != (int)x->m_dims[1])
+            throw std::runtime_error("add: b must match x or hold one value per channel");
+        pu.fwd(std::make_shared<AddBias>(x, b, y));
+    }
+}
+REGISTER_HIP_OP("add", add_setup);
+
+struct Softmax : public HipOperation {
+    const T x_, y_;
+    Softmax(T x, T y) : HipOperation("softmaxfwd"), x_(x), y_(y) {}
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vx = x_->view(), vy = y_->view();
+        chkSaga(saga_hip_softmax(&vx, &vy, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"x", x_}}; }
+    HipOpArgs listOutputs() const override { return {{"y", y_}}; }
+};
+
+void softmax_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
+{
+    if(p.m_pt != ProgramType::INFERENCE)
+        throw std::runtime_error{"not supported for training"};
+    auto x = p.lower(pu, n.m_inputs["x"]);
+    auto y = p.lowerLike(pu, n.m_outputs["y"], *x);
+    pu.fwd(std::make_shared<Softmax>(x, y));
+}
+REGISTER_HIP_OP("softmax", softmax_setup);
+
+// ---------------------------------------------------------------- dropout
+// Inference: identity (the reference aliases it away, :1576-1616).  Training needs a random
+// stream bit-compatible with nothing in particular; it is not offered by this engine.
+
+void dropout_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
+{
+    if(p.m_pt != ProgramType::INFERENCE)
+        throw std::runtime_error{"dropout is not supported for training by the hip engine"};
+    auto x = p.lower(pu, n.m_inputs["x"]);
+    p.m_ctx->m_tensors[n.m_outputs["y"]] =
+        alias_of(x, x->m_dims, x->m_strides, x->m_offset, n.m_outputs["y"]->namePostfix("nop-dropout"));
+}
+REGISTER_HIP_OP("dropout", dropout_setup);
+
+// ---------------------------------------------------------------- reshape / window / concat
+// No arithmetic: outputs alias their inputs (reference: :2504-2634).
+
+// A reshape keeps the LOGICAL (N,C,H,W) element order.  Row-major tensors are re-viewed in
+// place; a channels-last tensor with H*W > 1 is first copied into row-major order, so that
+// both layouts feed the same values to a following fc (the reference aliases the physical
+// order instead, which makes its two layouts disagree for such networks).
+void reshape_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
+{
+    auto xh = n.m_inputs["x"], yh = n.m_outputs["y"];
+    auto x = p.lower(pu, xh);
+    const Dims ydims = yh->m_dims.batch(pu.m_batch_size);
+    const bool training = p.m_pt == ProgramType::TRAINING;
+    T flat = x;
+    if(!x->rowMajor()) {
+        flat = std::make_shared<HipTensor>(x->m_data_type, x->m_dims, HipLayout::NCHW, p.m_ctx.get(),
+                                           xh->namePostfix("rowmajor"));
+        pu.fwd(std::make_shared<Transform>(x, flat, "reshape.copy"));
+    }
+    p.m_ctx->m_tensors[yh] =
+        alias_of(flat, ydims, hip_strides(ydims, HipLayout::NCHW), flat->m_offset, xh->namePostfix("reshape"));
+    if(!training)
+        return;
+    auto dx = p.lowerGrad(pu, xh);
+    if(!dx)
+        return;
+    T dflat = dx;
+    if(!dx->rowMajor()) {
+        dflat = std::make_shared<HipTensor>(dx->m_data_type, dx->m_dims, HipLayout::NCHW, p.m_ctx.get(),
+                                            xh->namePostfix("rowmajor.grad"));
+        pu.bwd(std::make_shared<Transform>(dflat, dx, "reshape.copy"));
+    }
+    p.m_ctx->m_tensors[yh->grad()] =
+        alias_of(dflat, ydims, hip_strides(ydims, HipLayout::NCHW), dflat->m_offset, xh->namePostfix("reshape.grad"));
+}
+REGISTER_HIP_OP("reshape", reshape_setup);
+
+Nodes window_transform(HipProgram &p, HipProgramUnit &pu, const Nodes &nodes)
+{
+    Nodes r;
+    for(const auto &n : nodes) {
+        if(n->m_type != "window") {
+            r.push_back(n);
+            continue;
+        }
+        auto x = p.lower(pu, n->m_inputs["x"]);
+        auto yh = n->m_outputs["y"];
+        const std::vector<int> off = n->m_attributes.get("offset", std::vector<int>{});
+        int64_t o = x->m_offset;
+        for(size_t i = 0; i < off.size() && i < x->m_strides.size(); i++)
+            o += (int64_t)off[i] * x->m_strides[i];
+        const Dims yd = yh->m_dims.batch(pu.m_batch_size);
+        p.m_ctx->m_tensors[yh] = alias_of(x, yd, x->m_strides, o, yh->namePostfix("alias"));
+        if(p.m_pt == ProgramType::TRAINING) {
+            if(auto dx = p.lowerGrad(pu, n->m_inputs["x"])) {
+                int64_t go = dx->m_offset;
+                for(size_t i = 0; i < off.size() && i < dx->m_strides.size(); i++)
+                    go += (int64_t)off[i] * dx->m_strides[i];
+                p.m_ctx->m_tensors[yh->grad()] = alias_of(dx, yd, dx->m_strides, go, yh->namePostfix("alias.grad"));
+            }
+        }
+    }
+    return r;
+}
+REGISTER_HIP_TRANSFORM(100, ProgramType::INFERENCE | ProgramType::TRAINING, window_transform);
+
+// Every input becomes a strided view into the output at its offset along `axis`, so the
+// producers write straight into the concatenated tensor.  Walks the nodes back to front so
+// that nested concats resolve outermost first.
+Nodes concat_transform(HipProgram &p, HipProgramUnit &pu, const Nodes &nodes)
+{
+    Nodes r;
+    for(ssize_t i = (ssize_t)nodes.size() - 1; i >= 0; i--) {
+        const auto &n = nodes[i];
+        if(n->m_type != "concat") {
+            r.insert(r.begin(), n);
+            continue;
+        }
+        const int axis = n->m_attributes.get("axis", 1);
+        auto y = p.lower(pu, n->m_outputs["y"]);
+        T dy = p.m_pt == ProgramType::TRAINING ? p.lowerGrad(pu, n->m_outputs["y"]) : nullptr;
+        int64_t along = 0;
+        for(const auto &xh : n->m_inputs.getv("x")) {
+            const Dims xd = xh->m_dims.batch(pu.m_batch_size);
+            auto x = alias_of(y, xd, y->m_strides, y->m_offset + along * y->m_strides[axis], xh->namePostfix("alias"));
+            x->copyFromHost(*xh); // inputs that carry values (graph inputs) are placed right away
+            p.m_ctx->m_tensors[xh] = x;
+            if(dy)
+                p.m_ctx->m_tensors[xh->grad()] = alias_of(dy, xd, dy->m_strides,
+                                                          dy->m_offset + along * dy->m_strides[axis],
+                                                          xh->namePostfix("alias.grad"));
+            along += (int)xh->m_dims[axis];
+        }
+    }
+    return r;
+}
+REGISTER_HIP_TRANSFORM(100, ProgramType::INFERENCE | ProgramType::TRAINING, concat_transform);
+
+}  // namespace
+
+}  // namespace saga

@@ -1,0 +1,640 @@
+// Engine, context and program of the hip backend: node lowering driver, op-list assembly
+// (forward ops, then backward ops in reverse creation order, then the optimizers), the
+// accumulate-on-second-writer rule, dead-operation elimination and the run loop with
+// double-buffered batched tensors and the loss-scale controller.
+// Role of the reference's src/cuda/cuda_common.cpp and src/cuda/cuda_program.cpp.
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <algorithm>
+#include <cmath>
+#include <sstream>
+
+#include "engine.hpp"
+#include "hip_common.hpp"
+
+namespace saga {
+
+// ---------------------------------------------------------------- registries
+
+static std::map<std::string, HipOpSetup> &op_table()
+{
+    static std::map<std::string, HipOpSetup> t;
+    return t;
+}
+
+struct TransformEntry {
+    int prio;
+    ProgramType types;
+    HipTransform fn;
+};
+
+static std::vector<TransformEntry> &transform_table()
+{
+    static std::vector<TransformEntry> t;
+    return t;
+}
+
+void hipRegisterOp(const char *name, HipOpSetup setup) { op_table()[name] = setup; }
+
+void hipRegisterTransform(int prio, ProgramType types, HipTransform fn)
+{
+    auto &t = transform_table();
+    t.push_back({prio, types, fn});
+    std::stable_sort(t.begin(), t.end(), [](const TransformEntry &a, const TransformEntry &b) { return a.prio < b.prio; });
+}
+
+HipOpSetup hipFindOp(const std::string &type)
+{
+    auto it = op_table().find(type);
+    return it == op_table().end() ? nullptr : it->second;
+}
+
+Nodes hipApplyTransforms(HipProgram &p, HipProgramUnit &pu, const Nodes &nodes)
+{
+    Nodes cur = nodes;
+    for(const auto &t : transform_table())
+        if(!!(p.m_pt & t.types))
+            cur = t.fn(p, pu, cur);
+    return cur;
+}
+
+// ---------------------------------------------------------------- operations (generic part)
+
+HipOpArgs HipOperation::getInputs()
+{
+    HipOpArgs r = listInputs();
+    for(auto &o : listOutputs()) {
+        float *beta = getBeta(o.second);
+        if(beta && *beta != 0.0f)
+            r.push_back(o);
+    }
+    return r;
+}
+
+std::string HipOperation::str()
+{
+    std::stringstream ss;
+    const char *sep = "";
+    for(const auto &o : getOutputs()) {
+        float *beta = getBeta(o.second);
+        ss << sep << (beta && *beta != 0.0f ? "+" : "") << o.first << ":" << o.second->shortname();
+        sep = ", ";
+    }
+    ss << " = " << name() << "(";
+    sep = "";
+    for(const auto &i : listInputs()) {
+        ss << sep << i.first << ":" << i.second->shortname();
+        sep = ", ";
+    }
+    const std::string inf = info();
+    if(!inf.empty())
+        ss << ", " << inf;
+    ss << ")";
+    return ss.str();
+}
+
+void HipOperation::dump(FILE *out, bool full)
+{
+    if(!full) {
+        fprintf(out, "%s\n", str().c_str());
+        return;
+    }
+    fprintf(out, "OP: %s %s\n", name().c_str(), info().c_str());
+    for(const auto &t : getInputs())
+        fprintf(out, "\tI: %3s: %s\n", t.first, t.second->info().c_str());
+    for(const auto &t : getOutputs())
+        fprintf(out, "\tO: %3s: %s\n", t.first, t.second->info().c_str());
+}
+
+// ---------------------------------------------------------------- engine / context
+
+class HipEngine : public Engine {
+public:
+    explicit HipEngine(const std::shared_ptr<UI> &ui) : m_ui(ui) {}
+    // One context per process: this backend drives a single GPU
+    // (the reference creates one per device, src/cuda/cuda_common.cpp:89-129).
+    std::vector<std::shared_ptr<Context>> createContexts(bool) override
+    {
+        int count = 0;
+        if(hipGetDeviceCount(&count) != hipSuccess || count < 1)
+            throw std::runtime_error("hip engine: no GPU visible");
+        return {std::make_shared<HipContext>(m_ui, 0)};
+    }
+    const std::shared_ptr<UI> m_ui;
+};
+
+static std::shared_ptr<Engine> createHipEngine(const std::shared_ptr<UI> &ui) { return std::make_shared<HipEngine>(ui); }
+
+static void __attribute__((constructor)) registerHipEngine(void)
+{
+    if(getenv("SAGA_DISABLE_HIP"))
+        return;
+    registerEngineFactory("hip", &createHipEngine);
+}
+
+HipContext::HipContext(const std::shared_ptr<UI> &ui, int device) : m_ui(ui), m_device(device)
+{
+    chkHip(hipSetDevice(device));
+    chkSaga(saga_hip_init(device, &m_num_cu));
+    chkHip(hipStreamCreateWithFlags(&m_stream, hipStreamDefault));
+    hipDeviceProp_t prop;
+    chkHip(hipGetDeviceProperties(&prop, device));
+    m_ui->updateCell(getUiPage(), 0, 0, UI::Align::LEFT, "%s", prop.name);
+    m_ui->updateCell(getUiPage(), 0, 1, UI::Align::LEFT, "Dev #%d", device);
+    m_workspace.request(4096);
+}
+
+HipContext::~HipContext()
+{
+    if(m_stream) {
+        (void)hipStreamSynchronize(m_stream);
+        (void)hipStreamDestroy(m_stream);
+    }
+}
+
+void HipContext::reset()
+{
+    sync();
+    m_exported.clear();
+    m_tensors.clear();
+    m_deferred_copy.clear();
+    m_storage_id_gen = 0;
+    m_program_index_gen = 0;
+}
+
+// reference: src/cuda/cuda_common.cpp:145-158
+std::shared_ptr<Tensor> HipContext::resolveTensor(std::shared_ptr<Tensor> src)
+{
+    if(!src)
+        return nullptr;
+    auto it = m_tensors.find(src);
+    if(it == m_tensors.end())
+        return nullptr;
+    m_exported.push_back(it->second->m_storage);
+    return it->second;
+}
+
+// reference: src/cuda/cuda_common.cpp:322-399
+std::shared_ptr<Program> HipContext::createMultiProgram(const std::vector<ProgramSource> &sources, ProgramType pt,
+                                                        const ProgramConfig &pc)
+{
+    chkHip(hipSetDevice(m_device));
+    auto p = std::make_shared<HipProgram>(shared_from_this(), pt, pc);
+    p->m_name = pt == ProgramType::INFERENCE ? "Inference" : "Training";
+    m_ui->updateCell(getUiPage(), p->getUiRow(), 0, UI::Align::LEFT, "%s", p->m_name.c_str());
+
+    float batch_sum = 0;
+    for(const auto &s : sources) {
+        p->addBatchedTensors(s);
+        p->m_units.emplace_back();
+        auto &pu = p->m_units.back();
+        pu.m_batch_size = s.batch_size;
+        batch_sum += s.batch_size;
+        pu.m_transformed = hipApplyTransforms(*p, pu, s.graph.m_nodes);
+    }
+    // initial loss scale: sum of the batch sizes (src/cuda/cuda_common.cpp:339-353) unless configured
+    p->m_mp_scaling = batch_sum;
+#ifdef SAGA_HAS_INITIAL_LOSS_SCALE
+    if(pc.initial_loss_scale > 0)
+        p->m_mp_scaling = pc.initial_loss_scale;
+#endif
+
+    size_t index = 0;
+    for(auto &pu : p->m_units) {
+        for(const auto &n : pu.m_transformed) {
+            HipOpSetup setup = hipFindOp(n->m_type);
+            try {
+                // the reference silently skips node types it has no operation for; here that is an error
+                if(!setup)
+                    throw std::runtime_error("the hip engine has no operation for this node type");
+                setup(*p, pu, *n);
+            } catch(const std::exception &e) {
+                throw std::runtime_error(
+                    fmt("Unable to create operation %s (#%zd) -- %s", n->m_type.c_str(), index, e.what()));
+            }
+            index++;
+        }
+        if(pt == ProgramType::INFERENCE && !pu.m_bwd.empty())
+            throw std::runtime_error("inference program produced backward operations");
+    }
+    if(pt == ProgramType::TRAINING) {
+        p->m_opt = p->createOptimizers();
+        p->m_updates.clear();
+    }
+    return p;
+}
+
+// ---------------------------------------------------------------- program: lowering helpers
+
+HipProgram::HipProgram(std::shared_ptr<HipContext> ctx, ProgramType pt, const ProgramConfig &pc)
+  : m_ctx(ctx), m_index(ctx->m_program_index_gen++), m_pt(pt), m_pc(pc)
+{
+    chkHip(hipHostMalloc((void **)&m_aux, 4096, hipHostMallocDefault));
+    memset(m_aux, 0, 4096);
+}
+
+HipProgram::~HipProgram()
+{
+    m_ctx->sync();
+    (void)hipHostFree(m_aux);
+}
+
+// fp16 and u8 tensors are channels-last, everything else channels-first, unless the program
+// asks for one layout (reference: tensorFormat, src/cuda/cuda_program.cpp:66-90)
+HipLayout HipProgram::layoutFor(Tensor::DataType dt) const
+{
+    switch(m_pc.tensor_layout) {
+    case TensorLayout::NHWC: return HipLayout::NHWC;
+    case TensorLayout::NCHW: return HipLayout::NCHW;
+    case TensorLayout::Auto: break;
+    }
+    return (dt == Tensor::DataType::HALF || dt == Tensor::DataType::U8) ? HipLayout::NHWC : HipLayout::NCHW;
+}
+
+// reference: lower_tensor, src/cuda/cuda_program.cpp:92-120
+std::shared_ptr<HipTensor> HipProgram::lower(const HipProgramUnit &pu, std::shared_ptr<Tensor> src,
+                                             size_t minimum_rank)
+{
+    if(!src)
+        return nullptr;
+    auto it = m_ctx->m_tensors.find(src);
+    if(it != m_ctx->m_tensors.end())
+        return it->second;
+    Dims dims = src->m_dims;
+    if(minimum_rank > 1) {
+        if(dims.size() < 2)
+            dims.insert(dims.begin(), (int64_t)1);
+        while(dims.size() < minimum_rank)
+            dims.push_back((int64_t)1);
+    }
+    dims = dims.batch(pu.m_batch_size);
+    auto t = std::make_shared<HipTensor>(src->m_data_type, dims, layoutFor(src->m_data_type), m_ctx.get(), src->m_name);
+    m_ctx->m_deferred_copy[t] = src;
+    m_ctx->m_tensors[src] = t;
+    return t;
+}
+
+std::shared_ptr<HipTensor> HipProgram::lowerLike(const HipProgramUnit &pu, std::shared_ptr<Tensor> src,
+                                                 const HipTensor &blueprint)
+{
+    auto it = m_ctx->m_tensors.find(src);
+    if(it != m_ctx->m_tensors.end())
+        return it->second;
+    const Dims dims = src->m_dims.batch(pu.m_batch_size);
+    HipLayout layout = layoutFor(src->m_data_type);
+    if(dims.size() == 4 && blueprint.m_dims.size() == 4)
+        layout = blueprint.cpacked() ? HipLayout::NHWC : HipLayout::NCHW;
+    auto t = std::make_shared<HipTensor>(src->m_data_type, dims, layout, m_ctx.get(), src->m_name);
+    m_ctx->m_deferred_copy[t] = src;
+    m_ctx->m_tensors[src] = t;
+    return t;
+}
+
+std::shared_ptr<HipTensor> HipProgram::lowerGrad(const HipProgramUnit &pu, std::shared_ptr<Tensor> src,
+                                                 size_t minimum_rank)
+{
+    if(!src)
+        return nullptr;
+    auto g = src->grad();
+    if(!g)
+        return nullptr; // tensors of foreign classes may have no gradient twin
+    // a gradient shares the layout of its value when that is already lowered (aliases!)
+    auto vit = m_ctx->m_tensors.find(src);
+    auto git = m_ctx->m_tensors.find(g);
+    if(git != m_ctx->m_tensors.end())
+        return git->second;
+    if(vit != m_ctx->m_tensors.end() && vit->second->m_dims.size() == 4) {
+        auto t = std::make_shared<HipTensor>(g->m_data_type, *vit->second, g->m_name);
+        m_ctx->m_deferred_copy[t] = g;
+        m_ctx->m_tensors[g] = t;
+        return t;
+    }
+    return lower(pu, g, minimum_rank);
+}
+
+void HipProgram::upd(const std::shared_ptr<Tensor> &key, const std::shared_ptr<HipTensor> &w,
+                     const std::shared_ptr<HipTensor> &g)
+{
+    m_updates[key] = std::make_pair(w, g);
+}
+
+// reference: addBatchedTensors, src/cuda/cuda_program.cpp:378-404
+void HipProgram::addBatchedTensors(const ProgramSource &ps)
+{
+    for(const auto &bt : ps.batched_tensors) {
+        auto src = bt.first;
+        auto &slot = m_batched[src];
+        if(!slot.first) {
+            auto existing = m_ctx->m_tensors.find(src);
+            if(existing != m_ctx->m_tensors.end() && existing->second->m_storage->doubleBuffered()) {
+                slot.first = std::static_pointer_cast<HipDoubleBuffer>(existing->second->m_storage);
+                m_batched_tensors[src] = existing->second;
+            } else {
+                const Dims dims = src->m_dims.batch(ps.batch_size);
+                auto st = std::make_shared<HipDoubleBuffer>(src->m_data_type, dims.elements(), m_ctx.get());
+                auto t = std::make_shared<HipTensor>(st, dims, hip_strides(dims, layoutFor(src->m_data_type)), 0,
+                                                     src->m_name);
+                t->copyFromHost(*src);
+                m_ctx->m_tensors[src] = t;
+                m_batched_tensors[src] = t;
+                slot.first = st;
+            }
+            slot.second = (Phase)0;
+        }
+        if(!(slot.second & Phase::POST) && !!(bt.second & Phase::POST))
+            m_ctx->m_exported.push_back(slot.first);
+        slot.second = slot.second | bt.second;
+    }
+}
+
+// ---------------------------------------------------------------- finalize
+
+// Backward liveness over the op list, treated as one iteration of a loop: a storage is needed
+// at the end of the step if the host can see it or if the next step reads it before writing
+// it (weights, running statistics, optimizer state).  Operations none of whose outputs are
+// needed are dropped; single unneeded outputs are offered to killOutput()
+// (reference: reduceLiveranges, src/cuda/cuda_analysis.cpp:328-374).
+void HipProgram::eliminateDeadOps()
+{
+    std::set<HipStorage *> live;
+    for(const auto &s : m_ctx->m_exported)
+        live.insert(s.get());
+    {
+        std::set<HipStorage *> written;
+        for(const auto &op : m_ops) {
+            for(const auto &i : op->getInputs())
+                if(!written.count(i.second->m_storage.get()))
+                    live.insert(i.second->m_storage.get()); // read before written: carried across steps
+            for(const auto &o : op->getOutputs())
+                written.insert(o.second->m_storage.get());
+        }
+    }
+    HipOps kept;
+    for(auto it = m_ops.rbegin(); it != m_ops.rend(); ++it) {
+        auto &op = *it;
+        bool needed = false;
+        for(const auto &o : op->getOutputs())
+            if(live.count(o.second->m_storage.get()))
+                needed = true;
+        if(!needed)
+            continue;
+        for(const auto &o : op->getOutputs()) {
+            HipStorage *s = o.second->m_storage.get();
+            if(!live.count(s)) {
+                op->killOutput(o.second->m_storage);
+                continue;
+            }
+            float *beta = op->getBeta(o.second);
+            const bool overwrites = !(beta && *beta != 0.0f) && o.second->m_dims.elements() == s->m_elements;
+            const bool pinned =
+                std::any_of(m_ctx->m_exported.begin(), m_ctx->m_exported.end(), [&](auto &e) { return e.get() == s; });
+            if(overwrites && !pinned)
+                live.erase(s);
+        }
+        for(const auto &i : op->getInputs())
+            live.insert(i.second->m_storage.get());
+        kept.push_back(op);
+    }
+    std::reverse(kept.begin(), kept.end());
+    m_ops = kept;
+}
+
+// reference: finalize, src/cuda/cuda_program.cpp:406-475
+void HipProgram::finalize()
+{
+    if(m_finalized)
+        return;
+    m_finalized = true;
+
+    for(const auto &kv : m_ctx->m_deferred_copy)
+        kv.first->copyFromHost(*kv.second);
+    m_ctx->m_deferred_copy.clear();
+
+    for(auto &pu : m_units) {
+        m_ops.insert(m_ops.end(), pu.m_fwd.begin(), pu.m_fwd.end());
+        m_ops.insert(m_ops.end(), pu.m_bwd.begin(), pu.m_bwd.end());
+        m_ops.insert(m_ops.end(), pu.m_tail.begin(), pu.m_tail.end());
+        pu.m_fwd.clear();
+        pu.m_bwd.clear();
+        pu.m_tail.clear();
+    }
+
+    // When several operations write the same tensor the results are summed: every writer after
+    // the first accumulates (beta = 1).  This is how gradients that fan in (skip connections)
+    // are added inside the convolution / GEMM epilogue (reference: src/cuda/cuda_program.cpp:429-453).
+    // An accumulating writer reads its output, so the dead-op pass below keeps the first writer
+    // whenever it keeps a later one.
+    std::set<HipTensor *> written;
+    for(auto &op : m_ops) {
+        for(auto &o : op->listOutputs()) {
+            if(written.insert(o.second.get()).second)
+                continue;
+            float *beta = op->getBeta(o.second);
+            if(!beta)
+                throw std::runtime_error(fmt("Operation ''%s'' does not support beta for %s", op->str().c_str(), o.first));
+            if(*beta == 0.0f)
+                *beta = 1.0f;
+        }
+    }
+
+    // optimizers read every gradient, so they keep the weight-gradient ops alive
+    m_ops.insert(m_ops.end(), m_opt.begin(), m_opt.end());
+    m_opt.clear();
+
+    eliminateDeadOps();
+
+    m_ctx->m_workspace.alloc();
+}
+
+// ---------------------------------------------------------------- run loop
+
+void HipProgram::runCallbacks(const TensorBatchCallback &cb, long batch, Phase phase)
+{
+    if(!cb)
+        return;
+    std::unordered_map<std::shared_ptr<Tensor>, TensorAccess *> amap;
+    std::vector<std::unique_ptr<TensorAccess>> keep;
+    for(const auto &bt : m_batched) {
+        if(!(bt.second.second & phase))
+            continue;
+        auto ta = m_batched_tensors[bt.first]->access();
+        amap[bt.first] = ta.get();
+        keep.push_back(std::move(ta));
+    }
+    cb(batch, *this, amap);
+}
+
+// Upload what the host wrote into the back buffers, then swap front and back.
+void HipProgram::flip(Phase upload_phase)
+{
+    for(auto &bt : m_batched) {
+        if(!!(bt.second.second & upload_phase))
+            bt.second.first->uploadBack(m_ctx->m_stream);
+        bt.second.first->flip();
+    }
+}
+
+void HipProgram::checkAnomaly(HipOperation &op, const HipOpArgs &tensors, const char *what)
+{
+    for(const auto &t : tensors) {
+        if(t.second->m_data_type != Tensor::DataType::HALF && t.second->m_data_type != Tensor::DataType::FLOAT)
+            continue;
+        if(t.second->m_storage->m_nonfinite_is_valid)
+            continue;
+        auto ta = t.second->access();
+        bool bad = false;
+        Dims c(t.second->m_dims.size(), (int64_t)0);
+        const std::vector<int64_t> ext = t.second->m_dims.i64();
+        std::vector<int64_t> cur(ext.size(), 0);
+        const size_t n = t.second->m_dims.elements();
+        for(size_t i = 0; i < n && !bad; i++) {
+            if(!std::isfinite((double)ta->get(c)))
+                bad = true;
+            for(ssize_t j = (ssize_t)ext.size() - 1; j >= 0; j--) {
+                if(++cur[j] == ext[j]) {
+                    cur[j] = 0;
+                    c[j] = (int64_t)0;
+                } else {
+                    c[j] = cur[j];
+                    break;
+                }
+            }
+        }
+        if(bad) {
+            fprintf(stderr, "\n\n *** Anomaly in tensor %s (%s)\n", t.second->info().c_str(), what);
+            op.dump(stderr, true);
+            abort();
+        }
+    }
+}
+
+void HipProgram::runOps(const HipOps &ops)
+{
+    for(const auto &op : ops) {
+        if(m_pc.anomaly_detect)
+            checkAnomaly(*op, op->getInputs(), "input");
+        try {
+            op->exec(*this);
+        } catch(const std::exception &e) {
+            throw std::runtime_error(fmt("Op %s failed -- %s", op->name().c_str(), e.what()));
+        }
+        if(m_pc.anomaly_detect)
+            checkAnomaly(*op, op->getOutputs(), "output");
+    }
+}
+
+void HipProgram::prep(long, long batch_offset)
+{
+    finalize();
+    runCallbacks(m_pc.pre_ops, 0 + batch_offset, Phase::PRE);
+    flip(Phase::PRE);
+    m_ctx->sync();
+    m_total_samples = 0;
+    m_epoch_start = now();
+}
+
+// reference: step, src/cuda/cuda_program.cpp:261-320
+void HipProgram::step(long batch, long batches, long batch_offset)
+{
+    runOps(m_ops);
+    for(auto &bt : m_batched)
+        if(!!(bt.second.second & Phase::POST))
+            bt.second.first->downloadFront(m_ctx->m_stream);
+
+    // host work for the neighbouring batches overlaps the GPU work enqueued above
+    if(batch > 0)
+        runCallbacks(m_pc.post_ops, batch - 1 + batch_offset, Phase::POST);
+    if(batch < batches - 1)
+        runCallbacks(m_pc.pre_ops, batch + 1 + batch_offset, Phase::PRE);
+    flip(Phase::PRE);
+
+    for(const auto &u : m_units)
+        m_total_samples += u.m_batch_size;
+
+    m_ctx->sync(); // the only synchronisation per step
+
+    if(m_mp_enabled) {
+        // loss-scale controller (reference: src/cuda/cuda_program.cpp:295-307)
+        if(m_aux->inf || m_aux->nan)
+            m_mp_scaling *= 0.5;
+        else if(m_aux->range > 1)
+            m_mp_scaling *= 0.9;
+        else
+            m_mp_scaling *= 1.02;
+        m_aux->range = 0;
+        m_aux->inf = 0;
+        m_aux->nan = 0;
+    }
+    const float sps = m_total_samples / (1e-6 * (now() - m_epoch_start));
+    m_ctx->m_ui->updateCell(m_ctx->getUiPage(), getUiRow(), 7, UI::Align::LEFT, "%ld (%.1f/s)", (long)m_total_samples, sps);
+    if(m_mp_enabled)
+        m_ctx->m_ui->updateCell(m_ctx->getUiPage(), getUiRow(), 9, UI::Align::LEFT, "%.1e", m_mp_scaling);
+}
+
+void HipProgram::post(long batches, long batch_offset)
+{
+    runCallbacks(m_pc.post_ops, batches - 1 + batch_offset, Phase::POST);
+}
+
+ExecResult HipProgram::run(long batches, StopCheck stop_check, long batch_offset)
+{
+    if(batches == 0)
+        return ExecResult::OK;
+    if(stop_check && stop_check())
+        return ExecResult::STOPPED;
+    chkHip(hipSetDevice(m_ctx->m_device));
+    prep(batches, batch_offset);
+    for(long i = 0; i < batches; i++) {
+        step(i, batches, batch_offset);
+        if(stop_check && stop_check())
+            return ExecResult::STOPPED;
+    }
+    post(batches, batch_offset);
+    return ExecResult::OK;
+}
+
+void HipProgram::dump(FILE *output, bool detailed)
+{
+    finalize();
+    fprintf(output, "\n%zd ops\n", m_ops.size());
+    int index = 0;
+    for(const auto &op : m_ops) {
+        fprintf(output, "#%3d: ", index++);
+        op->dump(output, detailed);
+    }
+}
+
+bool HipProgram::dumpGraph(const char *path)
+{
+    finalize();
+    FILE *fp = fopen(path, "w");
+    if(!fp)
+        return false;
+    fprintf(fp, "digraph HipOps {\n");
+    std::set<std::string> storages;
+    int i = 0;
+    for(auto &op : m_ops) {
+        fprintf(fp, "node [shape=circle,label=\"%s\"]; O%d;\n", op->name().c_str(), i++);
+        for(const auto &t : op->getInputs())
+            storages.insert(fmt("T%d", t.second->m_storage->m_id));
+        for(const auto &t : op->getOutputs())
+            storages.insert(fmt("T%d", t.second->m_storage->m_id));
+    }
+    for(const auto &s : storages)
+        fprintf(fp, "node [shape=box,label=\"%s\"]; %s;\n", s.c_str(), s.c_str());
+    i = 0;
+    for(auto &op : m_ops) {
+        for(const auto &t : op->getInputs())
+            fprintf(fp, "T%d->O%d;\n", t.second->m_storage->m_id, i);
+        for(const auto &t : op->getOutputs())
+            fprintf(fp, "O%d->T%d;\n", i, t.second->m_storage->m_id);
+        i++;
+    }
+    fprintf(fp, "overlap=false\n}\n");
+    fclose(fp);
+    return true;
+}
+
+}  // namespace saga
