@@ -1,0 +1,165 @@
+#!/usr/bin/env python3
+"""Headline benchmark: images/sec of fp16 NHWC ResNet-50 v1.5 at batch 256 on one MI355X,
+one training step (forward + backward + mixed-precision Adam) and inference, through the
+Saga Graph/Context/Program boundary on the hip engine.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+Prints ONE JSON line.  `value` is training images/sec over exactly K timed steps with the
+input batch already resident in HBM; `infer_images_per_sec` is the inference program on the
+same weights.  `roofline` describes the operation kind that takes the most GPU time in the
+training step (HIP-event timing of every operation on the engine's stream, taken in a second
+pass of K steps so that the events do not sit inside the timed region); `kernels` lists every
+operation kind the same way.  `cpu_baseline` is the CPU oracle (oracle/) running the same
+training step on a small batch on the host cores - a reported baseline, not a target.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 matrix
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+MATRIX_KINDS = ("convfwd", "convbwddata", "convbwdfilter", "fc.")
+
+
+def profile_rows(rows):
+    out = []
+    for r in rows:
+        if r["launches"] == 0 or r["ms"] <= 0:
+            continue
+        matrix = r["kind"].startswith(MATRIX_KINDS)
+        sec = r["ms"] * 1e-3
+        row = {"kind": r["kind"], "launches": r["launches"], "ms_total": round(r["ms"], 3),
+               "avg_us": round(r["ms"] * 1e3 / r["launches"], 2)}
+        if matrix:
+            a = r["flops"] / sec / 1e12
+            row.update(bound="mfma", achieved=round(a, 2), peak=PEAK_FP16_TFLOPS, unit="TFLOP/s",
+                       frac=round(a / PEAK_FP16_TFLOPS, 4))
+        else:
+            a = r["bytes"] / sec / 1e9
+            row.update(bound="hbm", achieved=round(a, 1), peak=PEAK_HBM_GBS, unit="GB/s",
+                       frac=round(a / PEAK_HBM_GBS, 4))
+        out.append(row)
+    out.sort(key=lambda r: -r["ms_total"])
+    return out
+
+
+def cpu_baseline(batch, image):
+    """The CPU oracle's training step on a bounded sample (small batch, same network)."""
+    from oracle.net import OracleNet
+    from saga_amd import networks as N
+
+    net = N.resnet50(batch, image=image)
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((batch, 3, image, image)).astype(np.float16).astype(np.float32)
+    labels = rng.integers(0, 1000, (batch, 1)).astype(np.int32)
+    o = OracleNet(net, lr=1e-4, loss_scale=1024.0)
+    t0 = time.perf_counter()
+    o.train_step(x, labels)
+    dt = time.perf_counter() - t0
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return {"value": round(batch / dt, 4), "unit": "images/sec", "cores": cores, "kind": "port",
+            "sample": f"one ResNet-50 training step (fwd+bwd+Adam) at batch {batch}, {image}x{image}, "
+                      f"{dt:.1f} s of CPU work"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--batch", type=int, default=256)
+    ap.add_argument("--image", type=int, default=224)
+    ap.add_argument("--cpu-batch", type=int, default=2)
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-profile", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build drives exactly one GPU (no collectives, no sharding); run with --gpus 1")
+
+    from saga_amd import api as S
+    from saga_amd import networks as N
+
+    net = N.resnet50(args.batch, image=args.image)
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((args.batch, 3, args.image, args.image)).astype(np.float16)
+    labels = rng.integers(0, 1000, (args.batch, 1)).astype(np.int32)
+
+    ctx = S.Context()
+    graph, t = N.build_graph(net, x)
+    train = ctx.create_program(graph, args.batch, training=True, learning_rate=1e-4, initial_loss_scale=1024.0)
+    infer = ctx.create_program(graph, args.batch, training=False)
+    ctx.resolve(t["labels"]).write(labels)
+    loss = ctx.resolve(t["loss"])
+    pred = ctx.resolve(t["pred"])
+    train.finalize()
+    infer.finalize()
+
+    # ---- training: W warm-up steps, then exactly K timed steps (each step ends in a stream sync)
+    train.run(args.warmup)
+    t0 = time.perf_counter()
+    train.run(args.steps)
+    t_train = time.perf_counter() - t0
+    mean_loss = float(loss.read().mean())
+
+    # ---- inference on the same weights
+    infer.run(args.warmup)
+    t0 = time.perf_counter()
+    infer.run(args.steps)
+    t_infer = time.perf_counter() - t0
+    pred.read()
+
+    kernels, roof = [], None
+    if not args.no_profile:
+        train.set_profiling(True)
+        train.run(args.steps)
+        kernels = profile_rows(train.profile())
+        train.set_profiling(False)
+        if kernels:
+            d = kernels[0]
+            roof = {"kernel": d["kind"], "bound": d["bound"], "achieved": d["achieved"], "peak": d["peak"],
+                    "unit": d["unit"], "frac": d["frac"], "traffic": None,
+                    "avg_launch_us": d["avg_us"], "launches": d["launches"]}
+
+    flops_step = 3 * net.flops_fwd * args.batch  # fwd + bwd-data + bwd-filter (the stem has no bwd-data)
+    ips = args.batch * args.steps / t_train
+    out = {
+        "metric": "images/sec fp16 NHWC ResNet-50 b256 infer+train step; conv MFMA util %",
+        "value": round(ips, 1),
+        "unit": "images/sec",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(t_train / args.steps * 1e3, 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": f"ResNet-50 v1.5 training step (fwd+bwd+Adam), fp16 NHWC, batch {args.batch}, "
+                               f"{args.image}x{args.image}, 1000 classes", "global_batch": args.batch},
+        "train_images_per_sec": round(ips, 1),
+        "infer_images_per_sec": round(args.batch * args.steps / t_infer, 1),
+        "infer_ms_per_batch": round(t_infer / args.steps * 1e3, 3),
+        "train_tflops": round(flops_step / (t_train / args.steps) / 1e12, 1),
+        "infer_tflops": round(net.flops_fwd * args.batch / (t_infer / args.steps) / 1e12, 1),
+        "loss_scale": train.loss_scale(),
+        "mean_loss": round(mean_loss, 4),
+        "roofline": roof,
+        "kernels": kernels,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(args.cpu_batch, args.image)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -95,6 +95,19 @@ int saga_program_run(saga_program_t p, long batches);
 double saga_program_loss_scale(saga_program_t p);
 int saga_program_dump(saga_program_t p, const char *path, int detailed);
 
+/* Per-operation-kind timing (HIP events on the program's stream around every operation) with the
+ * algorithmic flops / bytes of the timed launches.  No counterpart in the reference, whose only
+ * timing is samples per second (src/cuda/cuda_program.cpp:309-312). */
+typedef struct saga_profile_row {
+    char kind[48];
+    long launches;
+    double ms;
+    double flops;
+    double bytes;
+} saga_profile_row_t;
+int saga_program_set_profiling(saga_program_t p, int on);
+int saga_program_profile(saga_program_t p, saga_profile_row_t *rows, int capacity);
+
 #ifdef __cplusplus
 }
 #endif

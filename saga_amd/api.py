@@ -31,6 +31,11 @@ class _Attr(C.Structure):
                 ("ints", C.POINTER(C.c_int)), ("n_ints", C.c_int)]
 
 
+class _ProfileRow(C.Structure):
+    _fields_ = [("kind", C.c_char * 48), ("launches", C.c_long), ("ms", C.c_double), ("flops", C.c_double),
+                ("bytes", C.c_double)]
+
+
 class _Config(C.Structure):
     _fields_ = [("learning_rate", C.c_float), ("l2_lambda", C.c_float), ("bn_expavg", C.c_float),
                 ("tensor_layout", C.c_int), ("anomaly_detect", C.c_int), ("disable_op_fusing", C.c_int),
@@ -76,6 +81,8 @@ SIGNATURES = {
     "saga_program_run": (C.c_int, [_VP, C.c_long]),
     "saga_program_loss_scale": (C.c_double, [_VP]),
     "saga_program_dump": (C.c_int, [_VP, C.c_char_p, C.c_int]),
+    "saga_program_set_profiling": (C.c_int, [_VP, C.c_int]),
+    "saga_program_profile": (C.c_int, [_VP, C.POINTER(_ProfileRow), C.c_int]),
 }
 
 
@@ -333,6 +340,20 @@ class Program:
 
     def loss_scale(self):
         return lib().saga_program_loss_scale(self._h)
+
+    def set_profiling(self, on=True):
+        """Time every operation with HIP events on the program's stream (cleared when switched on)."""
+        if lib().saga_program_set_profiling(self._h, int(on)):
+            raise _err("set_profiling")
+
+    def profile(self):
+        """[{kind, launches, ms, flops, bytes}] accumulated since set_profiling(True)."""
+        rows = (_ProfileRow * 64)()
+        n = lib().saga_program_profile(self._h, rows, 64)
+        if n < 0:
+            raise _err("profile")
+        return [{"kind": rows[i].kind.decode(), "launches": rows[i].launches, "ms": rows[i].ms,
+                 "flops": rows[i].flops, "bytes": rows[i].bytes} for i in range(n)]
 
     def dump(self, path=None, detailed=False):
         if lib().saga_program_dump(self._h, _name(path), int(detailed)):

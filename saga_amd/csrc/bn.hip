@@ -167,21 +167,35 @@ __global__ void __launch_bounds__(256)
     }
 }
 
+__device__ __forceinline__ double wave_sum_f64(double v)
+{
+#pragma unroll
+    for(int o = 32; o > 0; o >>= 1)
+        v += __shfl_xor(v, o, 64);
+    return v;
+}
+
 // Finalize: mean, biased variance, invstd, running statistics, fused scale/shift.
+// One wavefront per channel adds the per-block partials (lanes stride over the blocks).
 template <typename T>
 __global__ void __launch_bounds__(256)
     bn_stats_finalize(const float *__restrict__ partial, int gx, const T *__restrict__ xrow0, int64_t kstride,
                       const float *__restrict__ s, const float *__restrict__ b, float *run_m, float *run_v,
                       float *save_mean, float *save_invstd, float *ss, double M, int C, float eps, float expavg)
 {
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
     if(c >= C)
         return;
     double s0 = 0, s1 = 0;
-    for(int g = 0; g < gx; g++) {
+    for(int g = lane; g < gx; g += 64) {
         s0 += partial[((int64_t)g * C + c) * 2];
         s1 += partial[((int64_t)g * C + c) * 2 + 1];
     }
+    s0 = wave_sum_f64(s0);
+    s1 = wave_sum_f64(s1);
+    if(lane != 0)
+        return;
     const double k = (double)(float)xrow0[c * kstride];
     const double dm = s0 / M;
     double var = s1 / M - dm * dm;
@@ -263,19 +277,25 @@ __global__ void __launch_bounds__(256)
 }
 
 // coef[0..C) = s*invstd ; coef[C..2C) = db/M ; coef[2C..3C) = ds*invstd/M ; writes ds, db.
+// One wavefront per channel, as above.
 __global__ void __launch_bounds__(256)
     bn_bwd_finalize(const float *__restrict__ partial, int gx, const float *__restrict__ s,
                     const float *__restrict__ save_invstd, float *ds, float *db, float *coef, double M, int C,
                     float beta_p)
 {
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
     if(c >= C)
         return;
     double s0 = 0, s1 = 0;
-    for(int g = 0; g < gx; g++) {
+    for(int g = lane; g < gx; g += 64) {
         s0 += partial[((int64_t)g * C + c) * 2];
         s1 += partial[((int64_t)g * C + c) * 2 + 1];
     }
+    s0 = wave_sum_f64(s0);
+    s1 = wave_sum_f64(s1);
+    if(lane != 0)
+        return;
     const double inv = save_invstd[c];
     const double dsv = s1 * inv;
     ds[c] = (float)(beta_p != 0.0f ? dsv + (double)beta_p * ds[c] : dsv);
@@ -601,7 +621,7 @@ int saga_hip_bn_train_fwd(const SagaTensorView *x, const SagaTensorView *z, cons
 #define GO(T, VN)                                                                                                   \
     do {                                                                                                            \
         bn_stats_cl<T, VN><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, partial, lx.rows, C, sh.cvb);           \
-        bn_stats_finalize<T><<<(C + 255) / 256, 256, 0, st>>>(partial, sh.gx, (const T *)x->ptr, 1, s, b, run_m,      \
+        bn_stats_finalize<T><<<(C + 3) / 4, 256, 0, st>>>(partial, sh.gx, (const T *)x->ptr, 1, s, b, run_m,      \
                                                               run_v, save_mean, save_invstd, ss, (double)lx.rows, C, \
                                                               eps, expavg);                                         \
         bn_apply_cl<T, VN, 1><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, add ? (const T *)z->ptr : nullptr,   \
@@ -673,7 +693,7 @@ int saga_hip_bn_bwd(const SagaTensorView *x, const SagaTensorView *y, const Saga
         bn_bwd_stats_cl<T, VN><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, relu ? (const T *)y->ptr : nullptr,  \
                                                      ly.pitch, (const T *)dy->ptr, ldy.pitch, save_mean, partial,    \
                                                      lx.rows, C, sh.cvb, flags);                                     \
-        bn_bwd_finalize<<<(C + 255) / 256, 256, 0, st>>>(partial, sh.gx, s, save_invstd, ds, db, coef,                \
+        bn_bwd_finalize<<<(C + 3) / 4, 256, 0, st>>>(partial, sh.gx, s, save_invstd, ds, db, coef,                \
                                                          (double)lx.rows, C, beta_p);                                \
         bn_bwd_apply_cl<T, VN><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, relu ? (const T *)y->ptr : nullptr,  \
                                                      ly.pitch, (const T *)dy->ptr, ldy.pitch, (T *)dx->ptr,          \

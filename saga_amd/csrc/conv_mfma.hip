@@ -438,17 +438,41 @@ __global__ void __launch_bounds__(256) conv_bwd_filter_mfma(FilterArgs g)
     }
 }
 
+// dw[row, c] = alpha * sum_p partial[p][row, c] + beta * dw ; rows = K*R*S, the partial rows are
+// Cp wide (Cp >= C when the input channels were padded)
 __global__ void __launch_bounds__(256)
-    filter_reduce(const float *__restrict__ partial, half_t *__restrict__ dw, int64_t n, int splits, float alpha, float beta)
+    filter_reduce(const float *__restrict__ partial, half_t *__restrict__ dw, int64_t n, int C, int Cp, int splits,
+                  float alpha, float beta)
 {
+    const int64_t np = n / C * Cp;
     for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t row = i / C;
+        const int64_t j = row * Cp + (i - row * C);
         float s = 0;
         for(int p = 0; p < splits; p++)
-            s += partial[(int64_t)p * n + i];
+            s += partial[(int64_t)p * np + j];
         s *= alpha;
         if(beta != 0.0f)
             s += beta * (float)dw[i];
         dw[i] = (half_t)s;
+    }
+}
+
+// Copies rows of C channels (pitch `sp`) into rows of Cp = multiple-of-8 channels, zero filled:
+// gives odd channel counts (the 3-channel network input) the 16-byte vectors the MFMA kernels load.
+__global__ void __launch_bounds__(256)
+    pad_channels(const half_t *__restrict__ src, int64_t sp, int C, half_t *__restrict__ dst, int Cp, int64_t rows)
+{
+    const int groups = Cp / 8;
+    const int64_t total = rows * groups;
+    for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t r = i / groups;
+        const int c0 = (int)(i - r * groups) * 8;
+        half8_t v;
+#pragma unroll
+        for(int e = 0; e < 8; e++)
+            v[e] = (c0 + e < C) ? src[r * sp + c0 + e] : (half_t)0;
+        *(half8_t *)(dst + r * Cp + c0) = v;
     }
 }
 
@@ -519,17 +543,25 @@ template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
     return 0;
 }
 
+static int round8(int v) { return (v + 7) & ~7; }
+
+// *pad is set when the gathered tensor cannot be loaded in 16-byte channel vectors as it is
+// (channel count, pitch or base address) and has to go through pad_channels first
 static bool common_ok(const SagaTensorView *act_in, const SagaTensorView *w, const SagaTensorView *act_out,
-                      const ConvGeom &g, CLInfo *li, CLInfo *lo)
+                      const ConvGeom &g, CLInfo *li, CLInfo *lo, bool *pad = nullptr)
 {
     if(act_in->dtype != SAGA_HALF || g.group != 1)
         return false;
     if(!as_channels_last(act_in, li) || !as_channels_last(act_out, lo) || !krsc_dense(w))
         return false;
-    if(li->C % 8 || li->pitch % 8 || !aligned16(act_in->ptr) || !aligned16(w->ptr))
+    const bool odd = li->C % 8 || li->pitch % 8 || !aligned16(act_in->ptr) || !aligned16(w->ptr);
+    if(odd && !pad)
         return false;
+    if(pad)
+        *pad = odd;
     // 32-bit element offsets inside the kernels
-    if(li->rows * li->pitch >= (int64_t)1 << 31 || lo->rows * lo->pitch >= (int64_t)1 << 31)
+    const int64_t in_pitch = odd ? round8(li->C) : li->pitch;
+    if(li->rows * in_pitch >= (int64_t)1 << 31 || lo->rows * lo->pitch >= (int64_t)1 << 31)
         return false;
     if((int64_t)g.K * g.R * g.S * g.C >= (int64_t)1 << 31)
         return false;
@@ -543,11 +575,20 @@ size_t conv_mfma_workspace(int kind, const SagaTensorView *x, const SagaTensorVi
 {
     if(x->dtype != SAGA_HALF)
         return 0;
+    // room for channel-padded copies of x and w (taken whenever C is not a multiple of 8; a
+    // misaligned pitch or base needs it too, so it is always reserved - it is small next to x)
+    const size_t Cp = round8(g.C);
+    const size_t xpad = ((size_t)g.N * g.H * g.W * Cp * sizeof(half_t) + 255) & ~(size_t)255;
+    const size_t wpad = ((size_t)g.K * g.R * g.S * Cp * sizeof(half_t) + 255) & ~(size_t)255;
+    if(kind == SAGA_CONV_FWD)
+        return xpad + wpad + 256;
     if(kind == SAGA_CONV_BWD_DATA)
         return (size_t)g.K * g.C * g.R * g.S * sizeof(half_t) + 256;
     if(kind == SAGA_CONV_BWD_FILTER) {
-        const FilterPlan p = plan_filter(g);
-        return (size_t)p.splits * g.K * g.R * g.S * g.C * sizeof(float) + 256;
+        ConvGeom gp = g;
+        gp.C = (int)Cp;
+        const FilterPlan p = plan_filter(gp);
+        return xpad + (size_t)p.splits * g.K * g.R * g.S * Cp * sizeof(float) + 256;
     }
     return 0;
 }
@@ -556,19 +597,36 @@ int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTe
                   float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st)
 {
     CLInfo lx, ly;
-    if(!common_ok(x, w, y, g, &lx, &ly))
+    bool pad = false;
+    if(!common_ok(x, w, y, g, &lx, &ly, &pad))
         return SAGA_HIP_EUNSUPPORTED;
     GatherArgs a;
     a.a = (const half_t *)x->ptr;
     a.b = (const half_t *)w->ptr;
+    a.Cred = g.C;
+    a.lda = (int)lx.pitch;
+    if(pad) {
+        const int Cp = round8(g.C);
+        const size_t xpad = ((size_t)lx.rows * Cp * sizeof(half_t) + 255) & ~(size_t)255;
+        const size_t wpad = (size_t)g.K * g.R * g.S * Cp * sizeof(half_t);
+        if(!ws || ws_bytes < xpad + wpad || !aligned16(ws))
+            return SAGA_HIP_EWORKSPACE;
+        half_t *xp = (half_t *)ws, *wp = (half_t *)((char *)ws + xpad);
+        pad_channels<<<grid_for(lx.rows * (Cp / 8), 256, 256 * 16), 256, 0, st>>>((const half_t *)x->ptr, lx.pitch, g.C,
+                                                                                 xp, Cp, lx.rows);
+        pad_channels<<<grid_for((int64_t)g.K * g.R * g.S * (Cp / 8), 256, 256 * 16), 256, 0, st>>>(
+            (const half_t *)w->ptr, g.C, g.C, wp, Cp, (int64_t)g.K * g.R * g.S);
+        a.a = xp;
+        a.b = wp;
+        a.Cred = Cp;
+        a.lda = Cp;
+    }
     a.out = (half_t *)y->ptr;
     a.M = (int)ly.rows;
     a.Ngemm = g.K;
-    a.Cred = g.C;
     a.IH = g.H; a.IW = g.W; a.OH = g.P; a.OW = g.Q;
     a.R = g.R; a.S = g.S;
     a.pad = g.pad; a.stride = g.stride; a.dil = g.dil; a.sshift = 0;
-    a.lda = (int)lx.pitch;
     a.ldo = (int)ly.pitch;
     a.alpha = alpha; a.beta = beta;
     return launch_gather<false>(a, st);
@@ -609,24 +667,37 @@ int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, cons
                          const ConvGeom &g, float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st)
 {
     CLInfo lx, ldy;
-    if(!common_ok(x, dw, dy, g, &lx, &ldy))
+    bool pad = false;
+    if(!common_ok(x, dw, dy, g, &lx, &ldy, &pad))
         return SAGA_HIP_EUNSUPPORTED;
     if(g.K % 8 || ldy.pitch % 8 || !aligned16(dy->ptr))
         return SAGA_HIP_EUNSUPPORTED;
-    const FilterPlan p = plan_filter(g);
+    const int Cp = pad ? round8(g.C) : g.C;
+    ConvGeom gp = g;
+    gp.C = Cp;
+    const FilterPlan p = plan_filter(gp);
     const int64_t n = (int64_t)g.K * g.R * g.S * g.C;
-    const size_t need = (size_t)p.splits * n * sizeof(float);
+    const size_t xpad = pad ? (((size_t)lx.rows * Cp * sizeof(half_t) + 255) & ~(size_t)255) : 0;
+    const size_t need = xpad + (size_t)p.splits * g.K * g.R * g.S * Cp * sizeof(float);
     if(!ws || ws_bytes < need || !aligned16(ws))
         return SAGA_HIP_EWORKSPACE;
     FilterArgs a;
     a.x = (const half_t *)x->ptr;
+    a.ldx = (int)lx.pitch;
+    if(pad) {
+        half_t *xp = (half_t *)ws;
+        pad_channels<<<grid_for(lx.rows * (Cp / 8), 256, 256 * 16), 256, 0, st>>>((const half_t *)x->ptr, lx.pitch, g.C,
+                                                                                 xp, Cp, lx.rows);
+        a.x = xp;
+        a.ldx = Cp;
+    }
     a.dy = (const half_t *)dy->ptr;
-    a.partial = (float *)ws;
+    a.partial = (float *)((char *)ws + xpad);
     a.M = (int)ldy.rows;
-    a.K = g.K; a.C = g.C; a.RSC = g.R * g.S * g.C;
+    a.K = g.K; a.C = Cp; a.RSC = g.R * g.S * Cp;
     a.H = g.H; a.W = g.W; a.P = g.P; a.Q = g.Q; a.S = g.S;
     a.pad = g.pad; a.stride = g.stride; a.dil = g.dil;
-    a.ldx = (int)lx.pitch; a.ldy = (int)ldy.pitch;
+    a.ldy = (int)ldy.pitch;
     a.tiles_k = p.tiles_k; a.tiles_c = p.tiles_c;
     a.splits = p.splits; a.m_per_split = p.m_per_split;
     const int blocks = p.tiles_k * p.tiles_c * p.splits;
@@ -635,7 +706,8 @@ int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, cons
     else
         conv_bwd_filter_mfma<64, 128><<<blocks, 256, 0, st>>>(a);
     SAGA_CHECK_LAUNCH();
-    filter_reduce<<<grid_for(n, 256, 256 * 8), 256, 0, st>>>((const float *)ws, (half_t *)dw->ptr, n, p.splits, alpha, beta);
+    filter_reduce<<<grid_for(n, 256, 256 * 8), 256, 0, st>>>(a.partial, (half_t *)dw->ptr, n, g.C, Cp, p.splits, alpha,
+                                                            beta);
     SAGA_CHECK_LAUNCH();
     return 0;
 }

@@ -6,6 +6,7 @@
 
 #include "saga.hpp"
 #include "saga_capi.h"
+#include "hip/hip_common.hpp"
 
 using namespace saga;
 
@@ -334,6 +335,40 @@ int saga_program_run(saga_program_t p, long batches)
 }
 
 double saga_program_loss_scale(saga_program_t p) { return ((ProgramBox *)p)->p->getMPS(); }
+
+int saga_program_set_profiling(saga_program_t p, int on)
+{
+    return guard([&] {
+        auto hp = std::dynamic_pointer_cast<HipProgram>(((ProgramBox *)p)->p);
+        if(!hp)
+            throw std::runtime_error("not a hip program");
+        hp->setProfiling(on != 0);
+    });
+}
+
+int saga_program_profile(saga_program_t p, saga_profile_row_t *rows, int capacity)
+{
+    int n = -1;
+    guard([&] {
+        auto hp = std::dynamic_pointer_cast<HipProgram>(((ProgramBox *)p)->p);
+        if(!hp)
+            throw std::runtime_error("not a hip program");
+        const auto prof = hp->profile();
+        n = 0;
+        for(const auto &r : prof) {
+            if(n >= capacity)
+                break;
+            strncpy(rows[n].kind, r.kind.c_str(), sizeof(rows[n].kind) - 1);
+            rows[n].kind[sizeof(rows[n].kind) - 1] = 0;
+            rows[n].launches = r.launches;
+            rows[n].ms = r.ms;
+            rows[n].flops = r.flops;
+            rows[n].bytes = r.bytes;
+            n++;
+        }
+    });
+    return n;
+}
 
 int saga_program_dump(saga_program_t p, const char *path, int detailed)
 {

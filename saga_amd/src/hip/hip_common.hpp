@@ -159,6 +159,10 @@ struct HipOperation {
     // drop an output nobody reads; false if the op cannot do without it
     virtual bool killOutput(const std::shared_ptr<HipStorage> &s) { return false; }
     virtual std::string info() const { return ""; }
+    // algorithmic work of one execution: floating point operations (matrix ops) and bytes that
+    // must cross HBM (memory-bound ops); used for roofline accounting only
+    virtual double flops() const { return 0; }
+    virtual double bytes() const { return 0; }
 
     // inputs plus the outputs that are accumulated into
     HipOpArgs getInputs();
@@ -268,6 +272,19 @@ public:
     std::map<std::shared_ptr<Tensor>, std::pair<std::shared_ptr<HipTensor>, std::shared_ptr<HipTensor>>> m_updates;
     std::unordered_map<std::shared_ptr<Tensor>, std::pair<std::shared_ptr<HipDoubleBuffer>, Phase>> m_batched;
     std::unordered_map<std::shared_ptr<Tensor>, std::shared_ptr<HipTensor>> m_batched_tensors;
+
+    // ---- optional per-operation timing with HIP events on the program's stream
+    struct ProfileRow {
+        std::string kind;
+        long launches = 0;
+        double ms = 0, flops = 0, bytes = 0;
+    };
+    void setProfiling(bool on);
+    std::vector<ProfileRow> profile() const;
+    bool m_profiling = false;
+    std::vector<hipEvent_t> m_events;          // one per op boundary (ops + 1)
+    std::map<std::string, ProfileRow> m_profile;
+    void collectProfile();
 
     SagaAux *m_aux = nullptr; // pinned host memory the optimizer kernels write their flags to
     float m_mp_scaling = 1.0f;

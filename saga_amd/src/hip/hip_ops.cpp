@@ -13,6 +13,14 @@ using T = std::shared_ptr<HipTensor>;
 
 saga_stream_t S(HipProgram &p) { return (saga_stream_t)p.m_ctx->m_stream; }
 
+double nbytes(const T &t) { return (double)t->m_dims.elements() * Tensor::DataTypeSize(t->m_data_type); }
+
+// 2 * N * K * P * Q * (C / group) * R * S for a convolution with input x, filter w, output y
+double conv_flops(const T &x, const T &w, const T &y, int group)
+{
+    return 2.0 * (double)y->m_dims.elements() * (double)((int)w->m_dims[1]) * (int)w->m_dims[2] * (int)w->m_dims[3];
+}
+
 T alias_of(const T &base, const Dims &dims, const std::vector<int64_t> &strides, int64_t offset,
            const std::optional<const std::string> &name)
 {
@@ -44,6 +52,8 @@ struct ConvFwd : public HipOperation {
     HipOpArgs listInputs() const override { return {{"x", x_}, {"w", w_}}; }
     HipOpArgs listOutputs() const override { return {{"y", y_}}; }
     float *getBeta(const T &t) override { return t == y_ ? &beta_ : nullptr; }
+    double flops() const override { return conv_flops(x_, w_, y_, cp_.group); }
+    double bytes() const override { return nbytes(x_) + nbytes(w_) + nbytes(y_) * (beta_ != 0 ? 2 : 1); }
 };
 
 struct ConvBwdData : public HipOperation {
@@ -65,6 +75,8 @@ struct ConvBwdData : public HipOperation {
     HipOpArgs listInputs() const override { return {{"w", w_}, {"dy", dy_}}; }
     HipOpArgs listOutputs() const override { return {{"dx", dx_}}; }
     float *getBeta(const T &t) override { return t == dx_ ? &beta_ : nullptr; }
+    double flops() const override { return conv_flops(dx_, w_, dy_, cp_.group); }
+    double bytes() const override { return nbytes(dy_) + nbytes(w_) + nbytes(dx_) * (beta_ != 0 ? 2 : 1); }
 };
 
 struct ConvBwdFilter : public HipOperation {
@@ -86,6 +98,8 @@ struct ConvBwdFilter : public HipOperation {
     HipOpArgs listInputs() const override { return {{"x", x_}, {"dy", dy_}}; }
     HipOpArgs listOutputs() const override { return {{"dw", dw_}}; }
     float *getBeta(const T &t) override { return t == dw_ ? &beta_ : nullptr; }
+    double flops() const override { return conv_flops(x_, dw_, dy_, cp_.group); }
+    double bytes() const override { return nbytes(x_) + nbytes(dy_) + nbytes(dw_); }
 };
 
 // y += b, b broadcast over the channel axis (reference: CudnnAddTensor, :39-68)
@@ -189,6 +203,7 @@ struct ActFwd : public HipOperation {
     HipOpArgs listInputs() const override { return {{"x", x_}}; }
     HipOpArgs listOutputs() const override { return {{"y", y_}}; }
     float *getBeta(const T &t) override { return t == y_ ? &beta_ : nullptr; }
+    double bytes() const override { return 2 * nbytes(x_); }
     std::string info() const override
     {
         static const char *names[] = {"relu", "sigmoid", "tanh", "swish", "leakyrelu"};
@@ -213,6 +228,7 @@ struct ActBwd : public HipOperation {
     HipOpArgs listInputs() const override { return {{"x", x_}, {"y", y_}, {"dy", dy_}}; }
     HipOpArgs listOutputs() const override { return {{"dx", dx_}}; }
     float *getBeta(const T &t) override { return t == dx_ ? &beta_ : nullptr; }
+    double bytes() const override { return (beta_ != 0 ? 4 : 3) * nbytes(dx_); }
 };
 
 void activation_setup(HipProgram &p, HipProgramUnit &pu, const Node &n, int mode, float alpha)
@@ -260,6 +276,7 @@ struct PoolFwd : public HipOperation {
     HipOpArgs listInputs() const override { return {{"x", x_}}; }
     HipOpArgs listOutputs() const override { return {{"y", y_}}; }
     std::string info() const override { return mode_ == SAGA_POOL_MAX ? "max" : "avg"; }
+    double bytes() const override { return nbytes(x_) + nbytes(y_); }
 };
 
 struct PoolBwd : public HipOperation {
@@ -278,6 +295,10 @@ struct PoolBwd : public HipOperation {
     HipOpArgs listInputs() const override { return {{"x", x_}, {"y", y_}, {"dy", dy_}}; }
     HipOpArgs listOutputs() const override { return {{"dx", dx_}}; }
     float *getBeta(const T &t) override { return t == dx_ ? &beta_ : nullptr; }
+    double bytes() const override
+    {
+        return nbytes(dx_) + nbytes(dy_) + (mode_ == SAGA_POOL_MAX ? nbytes(x_) + nbytes(y_) : 0);
+    }
 };
 
 void pooling_setup(HipProgram &p, HipProgramUnit &pu, const Node &n, int mode)
@@ -323,6 +344,8 @@ struct Gemm : public HipOperation {
     HipOpArgs listInputs() const override { return {{"a", a_}, {"b", b_}}; }
     HipOpArgs listOutputs() const override { return {{"c", c_}}; }
     float *getBeta(const T &t) override { return t == c_ ? &beta_ : nullptr; }
+    double flops() const override { return 2.0 * m_ * n_ * k_; }
+    double bytes() const override { return nbytes(a_) + nbytes(b_) + nbytes(c_); }
 };
 
 void fc_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
@@ -528,6 +551,7 @@ struct BnInference : public HipOperation {
         return r;
     }
     HipOpArgs listOutputs() const override { return {{"y", y_}}; }
+    double bytes() const override { return (z_ ? 3 : 2) * nbytes(x_); }
 };
 
 struct BnTrain : public HipOperation {
@@ -567,6 +591,8 @@ struct BnTrain : public HipOperation {
         return r;
     }
     HipOpArgs listOutputs() const override { return {{"y", y_}, {"m", m_}, {"v", v_}, {"sm", sm_}, {"sv", sv_}}; }
+    // statistics pass reads x, normalise pass reads x (+z) and writes y
+    double bytes() const override { return (z_ ? 4 : 3) * nbytes(x_); }
     float *getBeta(const T &t) override
     {
         if(t == m_)
@@ -622,6 +648,13 @@ struct BnBwd : public HipOperation {
             return true;
         }
         return false;
+    }
+    // both passes read x and dy (and y when the relu is fused); the second writes dx (and dz)
+    double bytes() const override
+    {
+        const double e = nbytes(dx_);
+        return e * (4 + ((flags_ & SAGA_BN_RELU) ? 2 : 0) + 1 + (dz_ ? 1 : 0) + (dx_beta_ != 0 ? 1 : 0) +
+                    (dz_ && dz_beta_ != 0 ? 1 : 0));
     }
     float *getBeta(const T &t) override
     {
@@ -765,6 +798,7 @@ struct AddOp : public HipOperation {
     }
     HipOpArgs listInputs() const override { return {{"a", a_}, {"b", b_}}; }
     HipOpArgs listOutputs() const override { return {{"c", c_}}; }
+    double bytes() const override { return 3 * nbytes(c_); }
 };
 
 // dst = src + beta*dst (reference: CudnnTransform, :72-99); also converts between layouts
@@ -780,6 +814,7 @@ struct Transform : public HipOperation {
     HipOpArgs listInputs() const override { return {{"a", a_}}; }
     HipOpArgs listOutputs() const override { return {{"b", b_}}; }
     float *getBeta(const T &t) override { return t == b_ ? &beta_ : nullptr; }
+    double bytes() const override { return (beta_ != 0 ? 3 : 2) * nbytes(b_); }
 };
 
 void sum_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)

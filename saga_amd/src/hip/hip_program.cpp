@@ -238,6 +238,8 @@ HipProgram::HipProgram(std::shared_ptr<HipContext> ctx, ProgramType pt, const Pr
 HipProgram::~HipProgram()
 {
     m_ctx->sync();
+    for(auto e : m_events)
+        (void)hipEventDestroy(e);
     (void)hipHostFree(m_aux);
 }
 
@@ -510,8 +512,49 @@ void HipProgram::checkAnomaly(HipOperation &op, const HipOpArgs &tensors, const 
     }
 }
 
+void HipProgram::setProfiling(bool on)
+{
+    m_profiling = on;
+    m_profile.clear();
+}
+
+std::vector<HipProgram::ProfileRow> HipProgram::profile() const
+{
+    std::vector<ProfileRow> r;
+    for(const auto &kv : m_profile)
+        r.push_back(kv.second);
+    return r;
+}
+
+// after the step's synchronisation: turn the event pairs into per-kind totals
+void HipProgram::collectProfile()
+{
+    if(!m_profiling || m_events.size() < m_ops.size() + 1)
+        return;
+    for(size_t i = 0; i < m_ops.size(); i++) {
+        float ms = 0;
+        if(hipEventElapsedTime(&ms, m_events[i], m_events[i + 1]) != hipSuccess)
+            continue;
+        auto &row = m_profile[m_ops[i]->name()];
+        row.kind = m_ops[i]->name();
+        row.launches++;
+        row.ms += ms;
+        row.flops += m_ops[i]->flops();
+        row.bytes += m_ops[i]->bytes();
+    }
+}
+
 void HipProgram::runOps(const HipOps &ops)
 {
+    if(m_profiling) {
+        while(m_events.size() < ops.size() + 1) {
+            hipEvent_t e;
+            chkHip(hipEventCreate(&e));
+            m_events.push_back(e);
+        }
+        chkHip(hipEventRecord(m_events[0], m_ctx->m_stream));
+    }
+    size_t index = 0;
     for(const auto &op : ops) {
         if(m_pc.anomaly_detect)
             checkAnomaly(*op, op->getInputs(), "input");
@@ -522,6 +565,9 @@ void HipProgram::runOps(const HipOps &ops)
         }
         if(m_pc.anomaly_detect)
             checkAnomaly(*op, op->getOutputs(), "output");
+        index++;
+        if(m_profiling)
+            chkHip(hipEventRecord(m_events[index], m_ctx->m_stream));
     }
 }
 
@@ -554,6 +600,7 @@ void HipProgram::step(long batch, long batches, long batch_offset)
         m_total_samples += u.m_batch_size;
 
     m_ctx->sync(); // the only synchronisation per step
+    collectProfile();
 
     if(m_mp_enabled) {
         // loss-scale controller (reference: src/cuda/cuda_program.cpp:295-307)
