@@ -11,8 +11,9 @@
 #include <cmath>
 #include <sstream>
 
-#include "engine.hpp"
 #include "hip_common.hpp"
+// after saga.hpp: the registry header relies on its declarations
+#include "engine.hpp"
 
 namespace saga {
 
