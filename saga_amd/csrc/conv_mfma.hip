@@ -19,6 +19,8 @@
 // Blocks are renumbered so that consecutive tiles land on the same XCD and share its L2.
 #include "conv.hpp"
 
+#include <stdlib.h>
+
 namespace {
 
 constexpr int BK = 32;        // reduction elements per LDS slice
@@ -41,6 +43,8 @@ struct GatherArgs {
     float alpha, beta;
     int nblk_n;        // number of block columns
     int nblocks;
+    unsigned a_bytes;  // extent of the gathered tensor / of b, for range-checked buffer loads
+    unsigned b_bytes;
 };
 
 __device__ __forceinline__ int xcd_remap(int b, int nblocks)
@@ -205,6 +209,197 @@ __global__ void __launch_bounds__(256) conv_gather_gemm(GatherArgs g)
 
     // ---- epilogue: accumulator element v of a 32x32 tile sits at row 8*(v/4) + 4*(lane/32) + v%4,
     // column lane%32
+    const int ecol = lane & 31, erow = (lane >> 5) * 4;
+#pragma unroll
+    for(int i = 0; i < TM; i++) {
+#pragma unroll
+        for(int j = 0; j < TN; j++) {
+            const int n = n0 + wn + j * 32 + ecol;
+            if(n >= g.Ngemm)
+                continue;
+#pragma unroll
+            for(int v = 0; v < 16; v++) {
+                const int m = m0 + wm + i * 32 + (v >> 2) * 8 + erow + (v & 3);
+                if(m >= g.M)
+                    continue;
+                half_t *o = g.out + (int64_t)m * g.ldo + n;
+                float val = g.alpha * acc[i][j][v];
+                if(g.beta != 0.0f)
+                    val += g.beta * (float)*o;
+                *o = (half_t)val;
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------- pipelined variant
+//
+// Same GEMM, different data movement: global -> LDS goes through the buffer-load-to-LDS path
+// (16 bytes per lane, no register staging), which lets STAGES-1 slices be in flight per
+// workgroup instead of one, enough to cover HBM latency at 2-3 workgroups per CU.
+//  * One such instruction fills 1 KB of LDS contiguously (lane i -> base + 16*i), i.e. 16 rows
+//    of one 64-byte slice row each.  Rows are therefore unpadded; bank conflicts of the MFMA
+//    fragment reads are avoided by an XOR swizzle of the four 16-byte slots of a row with
+//    bits 2..3 of the row number - applied on the way in by choosing WHICH 16 bytes a lane
+//    fetches, and on the way out by the fragment read address.
+//  * Lanes whose element is padding (outside the image, past M / N / C) use an offset beyond
+//    the buffer's num_records: the range check of the buffer load returns zeros for them.
+//  * Waits are explicit: loads retire in order, so "at most (STAGES-2) slices outstanding"
+//    means the oldest slice has landed.
+
+typedef __attribute__((address_space(3))) void *lds_ptr_t;
+
+template <int BM, int BN, int WGM, int WGN, int STAGES, bool BWD>
+__global__ void __launch_bounds__(256) conv_gather_gemm_dma(GatherArgs g)
+{
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    constexpr int AV = BM / 64, BV = BN / 64;
+    constexpr int ROWB = BK * 2;                       // bytes per LDS row (64)
+    constexpr int STAGE_BYTES = (BM + BN) * ROWB;
+    constexpr unsigned OOB = 0x7fffff00u;
+    static_assert(WGM * WGN == 4 && BK == 32, "layout");
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int bid = xcd_remap(blockIdx.x, g.nblocks);
+    const int bm = bid / g.nblk_n, bn = bid - bm * g.nblk_n;
+    const int m0 = bm * BM, n0 = bn * BN;
+
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void *)g.a, 0, g.a_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void *)g.b, 0, g.b_bytes, 0x00020000);
+
+    // this lane fills slot (tid & 3) of row lrow (+64 per round) and fetches the logical
+    // channel vector that the swizzle assigns to that slot
+    const int lrow = tid >> 2;
+    const int kv = (((tid & 3) ^ ((lrow >> 2) & 3))) * 8;
+    int a_base[AV], a_y[AV], a_x[AV];
+    bool a_ok[AV];
+#pragma unroll
+    for(int j = 0; j < AV; j++) {
+        const int m = m0 + lrow + 64 * j;
+        a_ok[j] = m < g.M;
+        const int mm = a_ok[j] ? m : 0;
+        const int ox = mm % g.OW;
+        const int t = mm / g.OW;
+        const int oy = t % g.OH;
+        const int n = t / g.OH;
+        a_base[j] = n * g.IH * g.IW;
+        if(BWD) {
+            a_y[j] = oy + g.pad;
+            a_x[j] = ox + g.pad;
+        } else {
+            a_y[j] = oy * g.stride - g.pad;
+            a_x[j] = ox * g.stride - g.pad;
+        }
+    }
+    const int ktot = g.R * g.S * g.Cred;
+    int b_off[BV];
+    bool b_ok[BV];
+#pragma unroll
+    for(int j = 0; j < BV; j++) {
+        const int n = n0 + lrow + 64 * j;
+        b_ok[j] = n < g.Ngemm;
+        b_off[j] = (b_ok[j] ? n : 0) * ktot;
+    }
+
+    int r = 0, s = 0, c0 = 0; // tap and channel offset of the NEXT slice to be issued
+    const int csteps = (g.Cred + BK - 1) / BK;
+    const int KT = g.R * g.S * csteps;
+
+    auto issue = [&](int stage) {
+        char *sa = smem + stage * STAGE_BYTES;
+        char *sb = sa + BM * ROWB;
+        const int c = c0 + kv;
+        const bool cok = c < g.Cred;
+#pragma unroll
+        for(int j = 0; j < AV; j++) {
+            int iy, ix;
+            bool ok = a_ok[j] && cok;
+            if(BWD) {
+                const int ty = a_y[j] - r * g.dil, tx = a_x[j] - s * g.dil;
+                ok = ok && ty >= 0 && tx >= 0 && ((ty | tx) & (g.stride - 1)) == 0;
+                iy = ty >> g.sshift;
+                ix = tx >> g.sshift;
+            } else {
+                iy = a_y[j] + r * g.dil;
+                ix = a_x[j] + s * g.dil;
+                ok = ok && iy >= 0 && ix >= 0;
+            }
+            ok = ok && iy < g.IH && ix < g.IW;
+            const unsigned off = ok ? (unsigned)(((a_base[j] + iy * g.IW + ix) * g.lda + c) * 2) : OOB;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(sa + (j * 64 + wave * 16) * ROWB), 16, off, 0, 0, 0);
+        }
+        const int kb = (r * g.S + s) * g.Cred + c;
+#pragma unroll
+        for(int j = 0; j < BV; j++) {
+            const unsigned off = (b_ok[j] && cok) ? (unsigned)((b_off[j] + kb) * 2) : OOB;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(sb + (j * 64 + wave * 16) * ROWB), 16, off, 0, 0, 0);
+        }
+        c0 += BK;
+        if(c0 >= g.Cred) {
+            c0 = 0;
+            if(++s == g.S) {
+                s = 0;
+                ++r;
+            }
+        }
+    };
+
+    float16_t acc[TM][TN];
+#pragma unroll
+    for(int i = 0; i < TM; i++)
+#pragma unroll
+        for(int j = 0; j < TN; j++)
+#pragma unroll
+            for(int v = 0; v < 16; v++)
+                acc[i][j][v] = 0.0f;
+
+    const int wm = (wave / WGN) * WTM, wn = (wave % WGN) * WTN;
+    const int frow = lane & 31;
+    const int swz = (frow >> 2) & 3;
+    // byte offsets of this lane's two fragment vectors (k 0..15 and 16..31) inside a row
+    const int fo0 = ((0 + (lane >> 5)) ^ swz) * 16, fo1 = ((2 + (lane >> 5)) ^ swz) * 16;
+
+#pragma unroll
+    for(int st = 0; st < STAGES - 1; st++)
+        if(st < KT)
+            issue(st);
+
+    for(int kt = 0; kt < KT; kt++) {
+        // oldest outstanding slice = kt; newer ones may stay in flight
+        // (a plain __syncthreads() would make the compiler drain every outstanding load)
+        if(kt + STAGES - 2 < KT)
+            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((AV + BV) * (STAGES - 2)) : "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+        if(kt + STAGES - 1 < KT)
+            issue((kt + STAGES - 1) % STAGES);
+        const char *sa = smem + (kt % STAGES) * STAGE_BYTES;
+        const char *sb = sa + BM * ROWB;
+        half8_t fa[2][TM], fb[2][TN];
+#pragma unroll
+        for(int i = 0; i < TM; i++) {
+            fa[0][i] = *(const half8_t *)(sa + (wm + i * 32 + frow) * ROWB + fo0);
+            fa[1][i] = *(const half8_t *)(sa + (wm + i * 32 + frow) * ROWB + fo1);
+        }
+#pragma unroll
+        for(int j = 0; j < TN; j++) {
+            fb[0][j] = *(const half8_t *)(sb + (wn + j * 32 + frow) * ROWB + fo0);
+            fb[1][j] = *(const half8_t *)(sb + (wn + j * 32 + frow) * ROWB + fo1);
+        }
+#pragma unroll
+        for(int kk = 0; kk < 2; kk++)
+#pragma unroll
+            for(int i = 0; i < TM; i++)
+#pragma unroll
+                for(int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kk][i], fb[kk][j], acc[i][j], 0, 0, 0);
+    }
+
     const int ecol = lane & 31, erow = (lane >> 5) * 4;
 #pragma unroll
     for(int i = 0; i < TM; i++) {
@@ -525,8 +720,44 @@ static int ilog2_exact(int v)
     return (1 << s) == v ? s : -1;
 }
 
+static int dma_stages()
+{
+    static int v = -1;
+    if(v < 0) {
+        const char *e = getenv("SAGA_HIP_CONV_STAGES");
+        v = e ? atoi(e) : 3; // 0 selects the register-staged kernel
+    }
+    return v;
+}
+
 template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
 {
+    const int stages = dma_stages();
+    if(stages >= 2 && g.a_bytes && g.b_bytes) {
+        if(g.Ngemm > 64) {
+            constexpr int BM = 128, BN = 128;
+            g.nblk_n = (g.Ngemm + BN - 1) / BN;
+            g.nblocks = ((g.M + BM - 1) / BM) * g.nblk_n;
+            if(stages == 2)
+                conv_gather_gemm_dma<BM, BN, 2, 2, 2, BWD><<<g.nblocks, 256, 2 * (BM + BN) * 64, st>>>(g);
+            else if(stages == 3)
+                conv_gather_gemm_dma<BM, BN, 2, 2, 3, BWD><<<g.nblocks, 256, 3 * (BM + BN) * 64, st>>>(g);
+            else
+                conv_gather_gemm_dma<BM, BN, 2, 2, 4, BWD><<<g.nblocks, 256, 4 * (BM + BN) * 64, st>>>(g);
+        } else {
+            constexpr int BM = 256, BN = 64;
+            g.nblk_n = (g.Ngemm + BN - 1) / BN;
+            g.nblocks = ((g.M + BM - 1) / BM) * g.nblk_n;
+            if(stages == 2)
+                conv_gather_gemm_dma<BM, BN, 4, 1, 2, BWD><<<g.nblocks, 256, 2 * (BM + BN) * 64, st>>>(g);
+            else if(stages == 3)
+                conv_gather_gemm_dma<BM, BN, 4, 1, 3, BWD><<<g.nblocks, 256, 3 * (BM + BN) * 64, st>>>(g);
+            else
+                conv_gather_gemm_dma<BM, BN, 4, 1, 4, BWD><<<g.nblocks, 256, 4 * (BM + BN) * 64, st>>>(g);
+        }
+        SAGA_CHECK_LAUNCH();
+        return 0;
+    }
     // tile choice by output-channel count; M tiles are 128 or 256 rows
     if(g.Ngemm > 64) {
         constexpr int BM = 128, BN = 128;
@@ -629,6 +860,12 @@ int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTe
     a.pad = g.pad; a.stride = g.stride; a.dil = g.dil; a.sshift = 0;
     a.ldo = (int)ly.pitch;
     a.alpha = alpha; a.beta = beta;
+    {
+        const int64_t ab = (pad ? lx.rows * (int64_t)a.lda : (lx.rows - 1) * lx.pitch + lx.C) * 2;
+        const int64_t bb = (int64_t)g.K * g.R * g.S * a.Cred * 2;
+        a.a_bytes = ab < 0x7fffff00 ? (unsigned)ab : 0;
+        a.b_bytes = bb < 0x7fffff00 ? (unsigned)bb : 0;
+    }
     return launch_gather<false>(a, st);
 }
 
@@ -660,6 +897,12 @@ int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const 
     a.lda = (int)ldy.pitch;
     a.ldo = (int)ldx.pitch;
     a.alpha = alpha; a.beta = beta;
+    {
+        const int64_t ab = ((ldy.rows - 1) * ldy.pitch + ldy.C) * 2;
+        const int64_t bb = (int64_t)g.K * g.R * g.S * g.C * 2;
+        a.a_bytes = ab < 0x7fffff00 ? (unsigned)ab : 0;
+        a.b_bytes = bb < 0x7fffff00 ? (unsigned)bb : 0;
+    }
     return launch_gather<true>(a, st);
 }
 

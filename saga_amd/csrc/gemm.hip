@@ -1,7 +1,9 @@
-// Row-major GEMM used by the fully-connected node: C = alpha*op(A)*op(B) + beta*C.
-// LDS-tiled 64x64x16 with a 4x4 register block per lane and fp32 accumulation; either
-// operand may be stored transposed.  (The fc layers of the target networks are a small
-// fraction of the step; convolutions take the MFMA path in conv_mfma.hip.)
+// Row-major GEMM used by the fully-connected node: C = alpha*op(A)*op(B) + beta*C, either
+// operand may be stored transposed.
+//  * fp16: gemm_mfma_f16, 64x64x32 block tiles on v_mfma_f32_32x32x16_f16 (one 32x32 tile per
+//    wave), operands staged through LDS with the reduction index contiguous; an operand
+//    stored with the other index contiguous is transposed on its way into LDS.
+//  * fp32: gemm_tiled, LDS-tiled 64x64x16 with a 4x4 register block per lane.
 #include "common.hpp"
 
 namespace {
@@ -72,6 +74,91 @@ __global__ void __launch_bounds__(256)
     }
 }
 
+// One operand tile (64 rows x 32 reduction steps) from global memory into LDS rows of LDK
+// halves.  kcontig: element (row, k) is at base[row*ld + k], else at base[k*ld + row].
+// Every lane moves 8 elements that are contiguous in memory, with one 16-byte load when the
+// run is in range and aligned.
+constexpr int GLDK = 40;
+
+__device__ __forceinline__ void gemm_stage(half_t (*dst)[GLDK], const half_t *__restrict__ base, int ld, bool kcontig,
+                                           int row0, int rows, int k0, int K, bool vec_ok, int tid)
+{
+    half8_t v;
+    if(kcontig) {
+        const int r = tid >> 2, kk = (tid & 3) * 8;
+        const int gr = row0 + r, gk = k0 + kk;
+        const half_t *src = base + (int64_t)gr * ld + gk;
+        if(vec_ok && gr < rows && gk + 8 <= K) {
+            v = *(const half8_t *)src;
+        } else {
+#pragma unroll
+            for(int j = 0; j < 8; j++)
+                v[j] = (gr < rows && gk + j < K) ? src[j] : (half_t)0;
+        }
+        *(half8_t *)&dst[r][kk] = v;
+    } else {
+        const int kk = tid >> 3, r = (tid & 7) * 8;
+        const int gr = row0 + r, gk = k0 + kk;
+        const half_t *src = base + (int64_t)gk * ld + gr;
+        if(vec_ok && gk < K && gr + 8 <= rows) {
+            v = *(const half8_t *)src;
+        } else {
+#pragma unroll
+            for(int j = 0; j < 8; j++)
+                v[j] = (gk < K && gr + j < rows) ? src[j] : (half_t)0;
+        }
+#pragma unroll
+        for(int j = 0; j < 8; j++)
+            dst[r + j][kk] = v[j];
+    }
+}
+
+__global__ void __launch_bounds__(256)
+    gemm_mfma_f16(int tA, int tB, int M, int N, int K, float alpha, const half_t *__restrict__ A, int lda,
+                  const half_t *__restrict__ B, int ldb, float beta, half_t *__restrict__ C, int ldc, int a_vec,
+                  int b_vec)
+{
+    __shared__ __attribute__((aligned(16))) half_t As[2][64][GLDK];
+    __shared__ __attribute__((aligned(16))) half_t Bs[2][64][GLDK];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+    const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+    float16_t acc;
+#pragma unroll
+    for(int v = 0; v < 16; v++)
+        acc[v] = 0.0f;
+    const int frow = lane & 31, fk = (lane >> 5) * 8;
+    const int KT = (K + 31) / 32;
+    gemm_stage(As[0], A, lda, !tA, m0, M, 0, K, a_vec, tid);
+    gemm_stage(Bs[0], B, ldb, tB, n0, N, 0, K, b_vec, tid);
+    for(int kt = 0; kt < KT; kt++) {
+        __syncthreads();
+        const int cur = kt & 1;
+        if(kt + 1 < KT) {
+            gemm_stage(As[cur ^ 1], A, lda, !tA, m0, M, (kt + 1) * 32, K, a_vec, tid);
+            gemm_stage(Bs[cur ^ 1], B, ldb, tB, n0, N, (kt + 1) * 32, K, b_vec, tid);
+        }
+#pragma unroll
+        for(int kk = 0; kk < 2; kk++) {
+            const half8_t fa = *(const half8_t *)&As[cur][wm + frow][kk * 16 + fk];
+            const half8_t fb = *(const half8_t *)&Bs[cur][wn + frow][kk * 16 + fk];
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fb, acc, 0, 0, 0);
+        }
+    }
+    const int n = n0 + wn + (lane & 31);
+    if(n >= N)
+        return;
+#pragma unroll
+    for(int v = 0; v < 16; v++) {
+        const int m = m0 + wm + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+        if(m >= M)
+            continue;
+        half_t *o = C + (int64_t)m * ldc + n;
+        const float r = alpha * acc[v];
+        *o = (half_t)(beta != 0.0f ? r + beta * (float)*o : r);
+    }
+}
+
 } // namespace
 
 extern "C" int saga_hip_gemm(int transA, int transB, int M, int N, int K, float alpha, const void *A, int lda,
@@ -83,10 +170,11 @@ extern "C" int saga_hip_gemm(int transA, int transB, int M, int N, int K, float 
         return SAGA_HIP_ESHAPE;
     dim3 grid((N + 63) / 64, (M + 63) / 64);
     hipStream_t st = as_stream(stream);
-    if(dtype == SAGA_HALF)
-        gemm_tiled<half_t><<<grid, 256, 0, st>>>(transA, transB, M, N, K, alpha, (const half_t *)A, lda,
-                                                 (const half_t *)B, ldb, beta, (half_t *)C, ldc);
-    else if(dtype == SAGA_FLOAT)
+    if(dtype == SAGA_HALF) {
+        const int a_vec = lda % 8 == 0 && ((uintptr_t)A & 15) == 0, b_vec = ldb % 8 == 0 && ((uintptr_t)B & 15) == 0;
+        gemm_mfma_f16<<<grid, 256, 0, st>>>(transA, transB, M, N, K, alpha, (const half_t *)A, lda, (const half_t *)B,
+                                            ldb, beta, (half_t *)C, ldc, a_vec, b_vec);
+    } else if(dtype == SAGA_FLOAT)
         gemm_tiled<float><<<grid, 256, 0, st>>>(transA, transB, M, N, K, alpha, (const float *)A, lda,
                                                 (const float *)B, ldb, beta, (float *)C, ldc);
     else

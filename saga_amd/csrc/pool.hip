@@ -217,6 +217,99 @@ __global__ void __launch_bounds__(256)
     }
 }
 
+// Max-pool backward for channels-last vectors, in two phases per block so that the tie-break
+// (the gradient goes to the FIRST position of a window equal to its maximum) is resolved once
+// per window instead of once per (input position, window):
+//  1. every window that overlaps the block's TH x TW patch of input positions scans its
+//     k*k inputs in order and leaves the code r*k+s of the first one equal to y (255: none)
+//     in LDS, one byte per channel;
+//  2. every input position sums dy over the windows that cover it and whose code names it.
+// Lanes run over CVB channel vectors first, then over positions.
+constexpr int POOL_TH = 16, POOL_TW = 16, POOL_CVB = 8;
+
+template <typename T, int VN>
+__global__ void __launch_bounds__(256) maxpool_bwd_tiled(DView x, DView y, DView dy, DView dx, int k, int pad,
+                                                         int stride, float beta, int tiles_w, int WPmax, int WQmax)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char codes[]; // [WPmax*WQmax][CVB][VN]
+    const int C = dx.d[1], H = dx.d[2], W = dx.d[3], P = dy.d[2], Q = dy.d[3];
+    const int tile = blockIdx.x, n = blockIdx.z;
+    const int h0 = (tile / tiles_w) * POOL_TH, w0 = (tile % tiles_w) * POOL_TW;
+    const int cvl = threadIdx.x % POOL_CVB, lpos = threadIdx.x / POOL_CVB;
+    const int c = (blockIdx.y * POOL_CVB + cvl) * VN;
+    const bool cok = c < C;
+    const int h1 = min(h0 + POOL_TH, H) - 1, w1 = min(w0 + POOL_TW, W) - 1;
+    const int p_lo = max(0, cdiv_floor(h0 + pad - k + stride, stride)), p_hi = min(P - 1, cdiv_floor(h1 + pad, stride));
+    const int q_lo = max(0, cdiv_floor(w0 + pad - k + stride, stride)), q_hi = min(Q - 1, cdiv_floor(w1 + pad, stride));
+    const int np = p_hi - p_lo + 1, nq = q_hi - q_lo + 1;
+
+    for(int wi = lpos; wi < np * nq; wi += 256 / POOL_CVB) {
+        if(!cok)
+            break;
+        const int p = p_lo + wi / nq, q = q_lo + wi % nq;
+        float yv[VN];
+        PV<T, VN>::load((const T *)y.ptr + off4(y, n, c, p, q), yv);
+        int code[VN];
+#pragma unroll
+        for(int j = 0; j < VN; j++)
+            code[j] = 255;
+        const int hs = p * stride - pad, ws = q * stride - pad;
+        for(int r = 0; r < k; r++) {
+            const int hh = hs + r;
+            if(hh < 0 || hh >= H)
+                continue;
+            for(int s = 0; s < k; s++) {
+                const int ww = ws + s;
+                if(ww < 0 || ww >= W)
+                    continue;
+                float e[VN];
+                PV<T, VN>::load((const T *)x.ptr + off4(x, n, c, hh, ww), e);
+#pragma unroll
+                for(int j = 0; j < VN; j++)
+                    code[j] = (code[j] == 255 && same(e[j], yv[j])) ? r * k + s : code[j];
+            }
+        }
+        unsigned char *o = codes + ((wi / nq) * WQmax + wi % nq) * (POOL_CVB * VN) + cvl * VN;
+#pragma unroll
+        for(int j = 0; j < VN; j++)
+            o[j] = (unsigned char)code[j];
+    }
+    __syncthreads();
+    if(!cok)
+        return;
+    for(int pi = lpos; pi < POOL_TH * POOL_TW; pi += 256 / POOL_CVB) {
+        const int h = h0 + pi / POOL_TW, w = w0 + pi % POOL_TW;
+        if(h >= H || w >= W)
+            continue;
+        float acc[VN];
+#pragma unroll
+        for(int j = 0; j < VN; j++)
+            acc[j] = 0.0f;
+        const int p0 = max(p_lo, cdiv_floor(h + pad - k + stride, stride)), p1 = min(p_hi, cdiv_floor(h + pad, stride));
+        const int q0 = max(q_lo, cdiv_floor(w + pad - k + stride, stride)), q1 = min(q_hi, cdiv_floor(w + pad, stride));
+        for(int p = p0; p <= p1; p++) {
+            for(int q = q0; q <= q1; q++) {
+                float g[VN];
+                PV<T, VN>::load((const T *)dy.ptr + off4(dy, n, c, p, q), g);
+                const int mine = (h - (p * stride - pad)) * k + (w - (q * stride - pad));
+                const unsigned char *o = codes + ((p - p_lo) * WQmax + (q - q_lo)) * (POOL_CVB * VN) + cvl * VN;
+#pragma unroll
+                for(int j = 0; j < VN; j++)
+                    acc[j] += o[j] == mine ? g[j] : 0.0f;
+            }
+        }
+        T *o = (T *)dx.ptr + off4(dx, n, c, h, w);
+        if(beta != 0.0f) {
+            float old[VN];
+            PV<T, VN>::load(o, old);
+#pragma unroll
+            for(int j = 0; j < VN; j++)
+                acc[j] += beta * old[j];
+        }
+        PV<T, VN>::store(o, acc);
+    }
+}
+
 static int vec_for(int dtype, std::initializer_list<const SagaTensorView *> vs)
 {
     const int vn = dtype == SAGA_HALF ? 8 : 4;
@@ -295,6 +388,21 @@ int saga_hip_pool_bwd(int mode, const SagaTensorView *x, const SagaTensorView *y
     const int g = grid_for(total, 256, 256 * 32);
     hipStream_t st = as_stream(stream);
     DView dvx = mx ? dview(x) : dview(dx), dvy = mx ? dview(y) : dview(dy), dvdy = dview(dy), dvdx = dview(dx);
+    if(mx && vn > 1 && size * size < 255) {
+        const int H = dx->dims[2], W = dx->dims[3];
+        const int WP = (POOL_TH + size - 2) / stride + 2, WQ = (POOL_TW + size - 2) / stride + 2;
+        const size_t lds = (size_t)WP * WQ * POOL_CVB * vn;
+        if(lds <= 64 * 1024 && dx->dims[0] <= 65535) {
+            const int tw = (W + POOL_TW - 1) / POOL_TW, th = (H + POOL_TH - 1) / POOL_TH;
+            const dim3 grid(tw * th, (dx->dims[1] / vn + POOL_CVB - 1) / POOL_CVB, dx->dims[0]);
+            if(dt == SAGA_HALF)
+                maxpool_bwd_tiled<half_t, 8><<<grid, 256, lds, st>>>(dvx, dvy, dvdy, dvdx, size, pad, stride, beta, tw, WP, WQ);
+            else
+                maxpool_bwd_tiled<float, 4><<<grid, 256, lds, st>>>(dvx, dvy, dvdy, dvdx, size, pad, stride, beta, tw, WP, WQ);
+            SAGA_CHECK_LAUNCH();
+            return 0;
+        }
+    }
 #define GO(T, VN)                                                                                              \
     do {                                                                                                       \
         if(mx)                                                                                                 \
