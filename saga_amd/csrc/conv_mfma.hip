@@ -633,6 +633,225 @@ __global__ void __launch_bounds__(256) conv_bwd_filter_mfma(FilterArgs g)
     }
 }
 
+// ---------------------------------------------------------------- pipelined backward-filter
+//
+// Same GEMM as conv_bwd_filter_mfma (rows = output channels of dy, columns = flat (tap, c),
+// reduction over pixels), but the tiles stay in their memory order in LDS - one row per pixel,
+// channels contiguous - so they can be filled by buffer-load-to-LDS with STAGES-1 slices in
+// flight, and the MFMA operands (8 consecutive PIXELS of one channel per lane) are produced
+// by the transposing LDS read: within a group of 16 lanes, lane i element j of
+// ds_read_b64_tr_b16 is element i%4 of the 8 bytes addressed by lane 4*j + i/4.  Pointing
+// lane s at (pixel s/4, channels 4*(s%4)..+3) therefore hands lane i (channel i, pixels 0..3).
+// The 16-byte granules of a row are XOR-swizzled with the pixel number so that the four
+// pixel rows one such read touches fall into different banks.
+
+typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef short short8_t __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) short4_t *lds_short4_ptr;
+
+__device__ __forceinline__ half8_t tr_read8(const char *lo, const char *hi)
+{
+    const short4_t a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)lo);
+    const short4_t b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)hi);
+    const short8_t v = __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(half8_t, v);
+}
+
+template <int BM, int BN, int STAGES>
+__global__ void __launch_bounds__(256) conv_bwd_filter_dma(FilterArgs g, unsigned x_bytes, unsigned dy_bytes)
+{
+    constexpr int GA = BM / 8, GB = BN / 8;             // 16-byte granules per LDS row
+    constexpr int RPA = 64 / GA, RPB = 64 / GB;         // pixel rows one wave instruction fills
+    constexpr int RA = BK / (4 * RPA), RB = BK / (4 * RPB);
+    constexpr int ROWA = BM * 2, ROWB = BN * 2;
+    constexpr int STAGE_BYTES = BK * (ROWA + ROWB);
+    constexpr int WGM = BM >= 128 ? 2 : 1, WGN = 4 / WGM;
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    constexpr unsigned OOB = 0x7fffff00u;
+    static_assert(RA >= 1 && RB >= 1 && (GA == 8 || GA == 16) && (GB == 8 || GB == 16), "tile");
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int b = blockIdx.x;
+    const int split = b % g.splits;
+    b /= g.splits;
+    const int tc = b % g.tiles_c, tk = b / g.tiles_c;
+    const int k0 = tk * BM, j0 = tc * BN;
+    const int m_begin = split * g.m_per_split;
+    int m_end = m_begin + g.m_per_split;
+    if(m_end > g.M)
+        m_end = g.M;
+
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)g.x, 0, x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc((void *)g.dy, 0, dy_bytes, 0x00020000);
+
+    // A (dy): this lane fills physical granule lane % GA of pixel row pa0 (+ 4*RPA per round)
+    const int pa0 = wave * RPA + lane / GA;
+    const int swa = GA == 16 ? (pa0 & 3) << 2 : ((pa0 >> 1) & 1) << 2;
+    const int ka = k0 + (((lane % GA) ^ swa) << 3);
+    const bool ka_ok = ka < g.K;
+    // B (x): likewise; the logical granule fixes this lane's (tap, c)
+    const int pb0 = wave * RPB + lane / GB;
+    const int swb = GB == 16 ? (pb0 & 3) << 2 : ((pb0 >> 1) & 1) << 2;
+    const int col = j0 + (((lane % GB) ^ swb) << 3);
+    const bool cb_ok = col < g.RSC;
+    const int tap = cb_ok ? col / g.C : 0;
+    const int cc = cb_ok ? col - tap * g.C : 0;
+    const int fr = tap / g.S, fs = tap - fr * g.S;
+    const int offy = fr * g.dil - g.pad, offx = fs * g.dil - g.pad;
+
+    int bn_[RB], by_[RB], bx_[RB];
+#pragma unroll
+    for(int j = 0; j < RB; j++) {
+        const int m = m_begin + pb0 + j * 4 * RPB;
+        const int mm = m < g.M ? m : 0;
+        bx_[j] = mm % g.Q;
+        const int t = mm / g.Q;
+        by_[j] = t % g.P;
+        bn_[j] = t / g.P;
+    }
+    int ms = m_begin; // first pixel of the next slice to be issued
+
+    auto issue = [&](int stage) {
+        char *sa = smem + stage * STAGE_BYTES;
+        char *sb = sa + BK * ROWA;
+#pragma unroll
+        for(int j = 0; j < RA; j++) {
+            const int m = ms + pa0 + j * 4 * RPA;
+            const unsigned off = (ka_ok && m < m_end) ? (unsigned)((m * g.ldy + ka) * 2) : OOB;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ry, (lds_ptr_t)(sa + (wave + 4 * j) * 1024), 16, off, 0, 0, 0);
+        }
+#pragma unroll
+        for(int j = 0; j < RB; j++) {
+            const int m = ms + pb0 + j * 4 * RPB;
+            const int iy = by_[j] * g.stride + offy, ix = bx_[j] * g.stride + offx;
+            const bool ok = cb_ok && m < m_end && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
+            const unsigned off = ok ? (unsigned)((((bn_[j] * g.H + iy) * g.W + ix) * g.ldx + cc) * 2) : OOB;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(sb + (wave + 4 * j) * 1024), 16, off, 0, 0, 0);
+            bx_[j] += BK;
+            while(bx_[j] >= g.Q) {
+                bx_[j] -= g.Q;
+                by_[j]++;
+            }
+            while(by_[j] >= g.P) {
+                by_[j] -= g.P;
+                bn_[j]++;
+            }
+        }
+        ms += BK;
+    };
+
+    float16_t acc[TM][TN];
+#pragma unroll
+    for(int i = 0; i < TM; i++)
+#pragma unroll
+        for(int j = 0; j < TN; j++)
+#pragma unroll
+            for(int v = 0; v < 16; v++)
+                acc[i][j][v] = 0.0f;
+
+    const int wm = (wave / WGN) * WTM, wn = (wave % WGN) * WTN;
+    // transposing fragment reads: this lane addresses pixel fp (+4 for the upper half, +16 per
+    // MFMA step) and channels fc .. fc+3 of a 32-channel tile
+    const int fp = 8 * (lane >> 5) + ((lane & 15) >> 2);
+    const int fc = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    const int fswa = GA == 16 ? (fp & 3) << 2 : ((fp >> 1) & 1) << 2;
+    const int fswb = GB == 16 ? (fp & 3) << 2 : ((fp >> 1) & 1) << 2;
+    int foa[TM], fob[TN];
+#pragma unroll
+    for(int i = 0; i < TM; i++) {
+        const int c = wm + i * 32 + fc;
+        foa[i] = fp * ROWA + (((c >> 3) ^ fswa) << 4) + (c & 7) * 2;
+    }
+#pragma unroll
+    for(int j = 0; j < TN; j++) {
+        const int c = wn + j * 32 + fc;
+        fob[j] = BK * ROWA + fp * ROWB + (((c >> 3) ^ fswb) << 4) + (c & 7) * 2;
+    }
+
+    const int KT = (m_end - m_begin + BK - 1) / BK;
+#pragma unroll
+    for(int st = 0; st < STAGES - 1; st++)
+        if(st < KT)
+            issue(st);
+
+    for(int kt = 0; kt < KT; kt++) {
+        if(kt + STAGES - 2 < KT)
+            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((RA + RB) * (STAGES - 2)) : "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+        if(kt + STAGES - 1 < KT)
+            issue((kt + STAGES - 1) % STAGES);
+        const char *sbase = smem + (kt % STAGES) * STAGE_BYTES;
+#pragma unroll
+        for(int kk = 0; kk < BK; kk += 16) {
+            half8_t fa[TM], fb[TN];
+#pragma unroll
+            for(int i = 0; i < TM; i++)
+                fa[i] = tr_read8(sbase + foa[i] + kk * ROWA, sbase + foa[i] + (kk + 4) * ROWA);
+#pragma unroll
+            for(int j = 0; j < TN; j++)
+                fb[j] = tr_read8(sbase + fob[j] + kk * ROWB, sbase + fob[j] + (kk + 4) * ROWB);
+#pragma unroll
+            for(int i = 0; i < TM; i++)
+#pragma unroll
+                for(int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+    }
+
+    float *out = g.partial + (int64_t)split * g.K * g.RSC;
+    const int ecol = lane & 31, erow = (lane >> 5) * 4;
+#pragma unroll
+    for(int i = 0; i < TM; i++) {
+#pragma unroll
+        for(int j = 0; j < TN; j++) {
+            const int cj = j0 + wn + j * 32 + ecol;
+            if(cj >= g.RSC)
+                continue;
+#pragma unroll
+            for(int v = 0; v < 16; v++) {
+                const int k = k0 + wm + i * 32 + (v >> 2) * 8 + erow + (v & 3);
+                if(k < g.K)
+                    out[(int64_t)k * g.RSC + cj] = acc[i][j][v];
+            }
+        }
+    }
+}
+
+// Sum of the split partials for tensors whose rows need no re-pitching: 16 lanes cover 64
+// consecutive elements with float4 loads, the 16 lane groups of a block take every 16th
+// partial, and LDS combines the groups in a fixed order (deterministic).
+__global__ void __launch_bounds__(256)
+    filter_reduce_v4(const float *__restrict__ partial, half_t *__restrict__ dw, int64_t n, int splits, float alpha,
+                     float beta)
+{
+    __shared__ float4_t red[16][16];
+    const int ev = threadIdx.x & 15, sl = threadIdx.x >> 4;
+    const int64_t e = ((int64_t)blockIdx.x * 16 + ev) * 4;
+    float4_t s = {0, 0, 0, 0};
+    if(e < n)
+        for(int p = sl; p < splits; p += 16)
+            s += *(const float4_t *)(partial + (int64_t)p * n + e);
+    red[sl][ev] = s;
+    __syncthreads();
+    if(sl == 0 && e < n) {
+#pragma unroll
+        for(int q = 1; q < 16; q++)
+            s += red[q][ev];
+#pragma unroll
+        for(int j = 0; j < 4; j++) {
+            float v = alpha * s[j];
+            if(beta != 0.0f)
+                v += beta * (float)dw[e + j];
+            dw[e + j] = (half_t)v;
+        }
+    }
+}
+
 // dw[row, c] = alpha * sum_p partial[p][row, c] + beta * dw ; rows = K*R*S, the partial rows are
 // Cp wide (Cp >= C when the input channels were padded)
 __global__ void __launch_bounds__(256)
@@ -944,13 +1163,25 @@ int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, cons
     a.tiles_k = p.tiles_k; a.tiles_c = p.tiles_c;
     a.splits = p.splits; a.m_per_split = p.m_per_split;
     const int blocks = p.tiles_k * p.tiles_c * p.splits;
-    if(p.bm == 128)
+    const int64_t xb = ((lx.rows - 1) * (int64_t)a.ldx + Cp) * 2, yb = ((ldy.rows - 1) * ldy.pitch + ldy.C) * 2;
+    if(dma_stages() >= 2 && xb < 0x7fffff00 && yb < 0x7fffff00) {
+        constexpr int ST = 3;
+        if(p.bm == 128)
+            conv_bwd_filter_dma<128, 128, ST><<<blocks, 256, ST * BK * 512, st>>>(a, (unsigned)xb, (unsigned)yb);
+        else
+            conv_bwd_filter_dma<64, 128, ST><<<blocks, 256, ST * BK * 384, st>>>(a, (unsigned)xb, (unsigned)yb);
+    } else if(p.bm == 128) {
         conv_bwd_filter_mfma<128, 128><<<blocks, 256, 0, st>>>(a);
-    else
+    } else {
         conv_bwd_filter_mfma<64, 128><<<blocks, 256, 0, st>>>(a);
+    }
     SAGA_CHECK_LAUNCH();
-    filter_reduce<<<grid_for(n, 256, 256 * 8), 256, 0, st>>>(a.partial, (half_t *)dw->ptr, n, g.C, Cp, p.splits, alpha,
-                                                            beta);
+    if(Cp == g.C && n % 4 == 0 && aligned16(a.partial) && ((uintptr_t)dw->ptr & 7) == 0)
+        filter_reduce_v4<<<(unsigned)((n / 4 + 15) / 16), 256, 0, st>>>(a.partial, (half_t *)dw->ptr, n, p.splits, alpha,
+                                                                       beta);
+    else
+        filter_reduce<<<grid_for(n, 256, 256 * 8), 256, 0, st>>>(a.partial, (half_t *)dw->ptr, n, g.C, Cp, p.splits,
+                                                                alpha, beta);
     SAGA_CHECK_LAUNCH();
     return 0;
 }
