@@ -45,6 +45,10 @@ struct GatherArgs {
     int nblocks;
     unsigned a_bytes;  // extent of the gathered tensor / of b, for range-checked buffer loads
     unsigned b_bytes;
+    int classes;       // backward data: stride*stride residue classes of output pixels (1: none)
+    int OHc, OWc, Mc;  // pixel grid and row count of one class (Mc = M when classes == 1)
+    int blocks_per_class;
+    unsigned char cls_ids[16]; // residue classes that get blocks (classes with no tap are left out)
 };
 
 __device__ __forceinline__ int xcd_remap(int b, int nblocks)
@@ -249,6 +253,25 @@ __global__ void __launch_bounds__(256) conv_gather_gemm(GatherArgs g)
 
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
 
+// Backward data with stride > 1 is split by the residue class (y % stride, x % stride) of the
+// output pixel: inside a class the set of filter taps that reach a pixel is the same for all
+// pixels (r = r0, r0+stride, ...), so a block of one class walks only those taps instead of
+// multiplying the zeros of the others.  g.classes = stride*stride (1: no split); a class's
+// pixels are numbered over the grid OHc x OWc = ceil(OH/stride) x ceil(OW/stride).
+//
+// The MFMA takes the filter tile as its first operand, so a lane ends up with 4 consecutive
+// output CHANNELS of one pixel per accumulator group; v_permlane32_swap pairs the two halves
+// of the wave and every lane stores (and, for beta != 0, loads) 16 contiguous bytes.
+
+__device__ __forceinline__ unsigned pack2(float a, float b)
+{
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    h2 v;
+    v[0] = (_Float16)a;
+    v[1] = (_Float16)b;
+    return __builtin_bit_cast(unsigned, v);
+}
+
 template <int BM, int BN, int WGM, int WGN, int STAGES, bool BWD>
 __global__ void __launch_bounds__(256) conv_gather_gemm_dma(GatherArgs g)
 {
@@ -265,9 +288,26 @@ __global__ void __launch_bounds__(256) conv_gather_gemm_dma(GatherArgs g)
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int bid = xcd_remap(blockIdx.x, g.nblocks);
+    int bid = xcd_remap(blockIdx.x, g.nblocks);
+    int py = 0, px = 0, r0 = 0, s0 = 0, nr = g.R, ns = g.S, rstep = 1;
+    int PH = g.OH, PW = g.OW; // pixel grid this block's rows are numbered over
+    if(BWD && g.classes > 1) {
+        const int ci = bid / g.blocks_per_class;
+        bid -= ci * g.blocks_per_class;
+        const int cls = g.cls_ids[ci];
+        py = cls >> g.sshift;
+        px = cls & (g.stride - 1);
+        r0 = (py + g.pad) & (g.stride - 1);
+        s0 = (px + g.pad) & (g.stride - 1);
+        nr = r0 < g.R ? (g.R - r0 + g.stride - 1) >> g.sshift : 0;
+        ns = s0 < g.S ? (g.S - s0 + g.stride - 1) >> g.sshift : 0;
+        rstep = g.stride;
+        PH = g.OHc;
+        PW = g.OWc;
+    }
     const int bm = bid / g.nblk_n, bn = bid - bm * g.nblk_n;
     const int m0 = bm * BM, n0 = bn * BN;
+    const int Mloc = BWD ? g.Mc : g.M;
 
     const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void *)g.a, 0, g.a_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void *)g.b, 0, g.b_bytes, 0x00020000);
@@ -281,16 +321,18 @@ __global__ void __launch_bounds__(256) conv_gather_gemm_dma(GatherArgs g)
 #pragma unroll
     for(int j = 0; j < AV; j++) {
         const int m = m0 + lrow + 64 * j;
-        a_ok[j] = m < g.M;
+        a_ok[j] = m < Mloc;
         const int mm = a_ok[j] ? m : 0;
-        const int ox = mm % g.OW;
-        const int t = mm / g.OW;
-        const int oy = t % g.OH;
-        const int n = t / g.OH;
+        const int ox = mm % PW;
+        const int t = mm / PW;
+        const int oy = t % PH;
+        const int n = t / PH;
         a_base[j] = n * g.IH * g.IW;
         if(BWD) {
-            a_y[j] = oy + g.pad;
-            a_x[j] = ox + g.pad;
+            const int y = oy * rstep + py, x = ox * rstep + px;
+            a_ok[j] = a_ok[j] && y < g.OH && x < g.OW;
+            a_y[j] = y + g.pad;
+            a_x[j] = x + g.pad;
         } else {
             a_y[j] = oy * g.stride - g.pad;
             a_x[j] = ox * g.stride - g.pad;
@@ -306,15 +348,16 @@ __global__ void __launch_bounds__(256) conv_gather_gemm_dma(GatherArgs g)
         b_off[j] = (b_ok[j] ? n : 0) * ktot;
     }
 
-    int r = 0, s = 0, c0 = 0; // tap and channel offset of the NEXT slice to be issued
+    int ri = 0, si = 0, c0 = 0; // tap counters and channel offset of the NEXT slice to be issued
     const int csteps = (g.Cred + BK - 1) / BK;
-    const int KT = g.R * g.S * csteps;
+    const int KT = nr * ns * csteps;
 
     auto issue = [&](int stage) {
         char *sa = smem + stage * STAGE_BYTES;
         char *sb = sa + BM * ROWB;
         const int c = c0 + kv;
         const bool cok = c < g.Cred;
+        const int r = r0 + ri * rstep, s = s0 + si * rstep;
 #pragma unroll
         for(int j = 0; j < AV; j++) {
             int iy, ix;
@@ -342,9 +385,9 @@ __global__ void __launch_bounds__(256) conv_gather_gemm_dma(GatherArgs g)
         c0 += BK;
         if(c0 >= g.Cred) {
             c0 = 0;
-            if(++s == g.S) {
-                s = 0;
-                ++r;
+            if(++si == ns) {
+                si = 0;
+                ++ri;
             }
         }
     };
@@ -397,27 +440,75 @@ __global__ void __launch_bounds__(256) conv_gather_gemm_dma(GatherArgs g)
             for(int i = 0; i < TM; i++)
 #pragma unroll
                 for(int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kk][i], fb[kk][j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk][j], fa[kk][i], acc[i][j], 0, 0, 0);
     }
 
-    const int ecol = lane & 31, erow = (lane >> 5) * 4;
+    // acc[i][j][v]: pixel wm + 32*i + lane%32, channel wn + 32*j + 8*(v/4) + 4*(lane/32) + v%4
+    const int hi = lane >> 5;
+    const bool vec_ok = (g.ldo & 7) == 0 && (g.Ngemm & 7) == 0 && ((uintptr_t)g.out & 15) == 0;
 #pragma unroll
     for(int i = 0; i < TM; i++) {
+        const int m = m0 + wm + i * 32 + (lane & 31);
+        bool ok = m < Mloc;
+        int64_t pix = m;
+        if(BWD && g.classes > 1) {
+            const int mm = ok ? m : 0;
+            const int ox = mm % PW;
+            const int t = mm / PW;
+            const int oy = t % PH;
+            const int n = t / PH;
+            const int y = oy * rstep + py, x = ox * rstep + px;
+            ok = ok && y < g.OH && x < g.OW;
+            pix = ((int64_t)n * g.OH + y) * g.OW + x;
+        }
+        half_t *orow = g.out + pix * g.ldo;
 #pragma unroll
         for(int j = 0; j < TN; j++) {
-            const int n = n0 + wn + j * 32 + ecol;
-            if(n >= g.Ngemm)
-                continue;
+            const int nb = n0 + wn + j * 32;
+            if(vec_ok) {
+                float f[16];
 #pragma unroll
-            for(int v = 0; v < 16; v++) {
-                const int m = m0 + wm + i * 32 + (v >> 2) * 8 + erow + (v & 3);
-                if(m >= g.M)
-                    continue;
-                half_t *o = g.out + (int64_t)m * g.ldo + n;
-                float val = g.alpha * acc[i][j][v];
-                if(g.beta != 0.0f)
-                    val += g.beta * (float)*o;
-                *o = (half_t)val;
+                for(int v = 0; v < 16; v++)
+                    f[v] = g.alpha * acc[i][j][v];
+                if(g.beta != 0.0f) {
+                    typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+#pragma unroll
+                    for(int q = 0; q < 4; q++) {
+                        const int n = nb + 8 * q + 4 * hi;
+                        if(ok && n < g.Ngemm) {
+                            const half4_t old = *(const half4_t *)(orow + n);
+#pragma unroll
+                            for(int e = 0; e < 4; e++)
+                                f[4 * q + e] += g.beta * (float)old[e];
+                        }
+                    }
+                }
+                // after the swaps: lower half-wave holds channels 0..7 (then 16..23) of the tile,
+                // upper half-wave 8..15 (24..31): one store covers 32 contiguous bytes per pixel
+#pragma unroll
+                for(int q = 0; q < 2; q++) {
+                    const unsigned x0 = pack2(f[8 * q + 0], f[8 * q + 1]), x1 = pack2(f[8 * q + 2], f[8 * q + 3]);
+                    const unsigned y0 = pack2(f[8 * q + 4], f[8 * q + 5]), y1 = pack2(f[8 * q + 6], f[8 * q + 7]);
+                    const auto s0_ = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+                    const auto s1_ = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+                    const int n = nb + 16 * q + 8 * hi;
+                    if(ok && n < g.Ngemm) {
+                        typedef unsigned u4 __attribute__((ext_vector_type(4)));
+                        const u4 o = {s0_[0], s1_[0], s0_[1], s1_[1]};
+                        *(u4 *)(orow + n) = o;
+                    }
+                }
+            } else if(ok) {
+#pragma unroll
+                for(int v = 0; v < 16; v++) {
+                    const int n = nb + (v >> 2) * 8 + hi * 4 + (v & 3);
+                    if(n >= g.Ngemm)
+                        continue;
+                    float val = g.alpha * acc[i][j][v];
+                    if(g.beta != 0.0f)
+                        val += g.beta * (float)orow[n];
+                    orow[n] = (half_t)val;
+                }
             }
         }
     }
@@ -939,6 +1030,18 @@ static int ilog2_exact(int v)
     return (1 << s) == v ? s : -1;
 }
 
+// out[row][0..C) = 0 for rows of pitch `pitch` elements (C and pitch multiples of 8, 16-byte aligned)
+__global__ void __launch_bounds__(256) zero_rows(half_t *__restrict__ out, int64_t rows, int C, int64_t pitch)
+{
+    const int groups = C / 8;
+    const int64_t total = rows * groups;
+    const half8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+    for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t r = i / groups;
+        *(half8_t *)(out + r * pitch + (i - r * groups) * 8) = z;
+    }
+}
+
 static int dma_stages()
 {
     static int v = -1;
@@ -951,28 +1054,45 @@ static int dma_stages()
 
 template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
 {
-    const int stages = dma_stages();
-    if(stages >= 2 && g.a_bytes && g.b_bytes) {
+    g.classes = 1;
+    g.Mc = g.M;
+    g.OHc = g.OH;
+    g.OWc = g.OW;
+    if(dma_stages() >= 2 && g.a_bytes && g.b_bytes) {
+        constexpr int ST = 3;
+        int active = 1;
+        if(BWD && g.stride > 1 && g.stride <= 4 && g.dil == 1) {
+            g.classes = g.stride * g.stride;
+            g.OHc = (g.OH + g.stride - 1) / g.stride;
+            g.OWc = (g.OW + g.stride - 1) / g.stride;
+            g.Mc = g.M / (g.OH * g.OW) * g.OHc * g.OWc;
+            // classes that no tap reaches produce beta*out: nothing to do for beta == 1, one
+            // coalesced fill for beta == 0 (a vectorisable output; otherwise they keep their blocks)
+            const bool can_fill = (g.ldo & 7) == 0 && (g.Ngemm & 7) == 0 && ((uintptr_t)g.out & 15) == 0;
+            const bool drop = g.beta == 1.0f || (g.beta == 0.0f && can_fill);
+            active = 0;
+            for(int c = 0; c < g.classes; c++) {
+                const int r0 = ((c >> g.sshift) + g.pad) & (g.stride - 1), s0 = ((c & (g.stride - 1)) + g.pad) & (g.stride - 1);
+                if(!drop || (r0 < g.R && s0 < g.S))
+                    g.cls_ids[active++] = (unsigned char)c;
+            }
+            if(active < g.classes && g.beta == 0.0f)
+                zero_rows<<<grid_for((int64_t)g.M * (g.Ngemm / 8), 256, 256 * 16), 256, 0, st>>>(g.out, g.M, g.Ngemm, g.ldo);
+            if(active == 0)
+                return 0;
+        }
         if(g.Ngemm > 64) {
             constexpr int BM = 128, BN = 128;
             g.nblk_n = (g.Ngemm + BN - 1) / BN;
-            g.nblocks = ((g.M + BM - 1) / BM) * g.nblk_n;
-            if(stages == 2)
-                conv_gather_gemm_dma<BM, BN, 2, 2, 2, BWD><<<g.nblocks, 256, 2 * (BM + BN) * 64, st>>>(g);
-            else if(stages == 3)
-                conv_gather_gemm_dma<BM, BN, 2, 2, 3, BWD><<<g.nblocks, 256, 3 * (BM + BN) * 64, st>>>(g);
-            else
-                conv_gather_gemm_dma<BM, BN, 2, 2, 4, BWD><<<g.nblocks, 256, 4 * (BM + BN) * 64, st>>>(g);
+            g.blocks_per_class = ((g.Mc + BM - 1) / BM) * g.nblk_n;
+            g.nblocks = g.blocks_per_class * active;
+            conv_gather_gemm_dma<BM, BN, 2, 2, ST, BWD><<<g.nblocks, 256, ST * (BM + BN) * 64, st>>>(g);
         } else {
             constexpr int BM = 256, BN = 64;
             g.nblk_n = (g.Ngemm + BN - 1) / BN;
-            g.nblocks = ((g.M + BM - 1) / BM) * g.nblk_n;
-            if(stages == 2)
-                conv_gather_gemm_dma<BM, BN, 4, 1, 2, BWD><<<g.nblocks, 256, 2 * (BM + BN) * 64, st>>>(g);
-            else if(stages == 3)
-                conv_gather_gemm_dma<BM, BN, 4, 1, 3, BWD><<<g.nblocks, 256, 3 * (BM + BN) * 64, st>>>(g);
-            else
-                conv_gather_gemm_dma<BM, BN, 4, 1, 4, BWD><<<g.nblocks, 256, 4 * (BM + BN) * 64, st>>>(g);
+            g.blocks_per_class = ((g.Mc + BM - 1) / BM) * g.nblk_n;
+            g.nblocks = g.blocks_per_class * active;
+            conv_gather_gemm_dma<BM, BN, 4, 1, ST, BWD><<<g.nblocks, 256, ST * (BM + BN) * 64, st>>>(g);
         }
         SAGA_CHECK_LAUNCH();
         return 0;

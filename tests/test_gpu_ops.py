@@ -39,6 +39,9 @@ CONV_CASES = [
     (2, 32, 8, 8, 16, 1, 0, 2, 1),
     (2, 8, 7, 7, 4, 3, 0, 1, 2),
     (3, 64, 14, 14, 64, 3, 1, 1, 1),
+    (2, 16, 13, 13, 24, 3, 0, 2, 1),
+    (1, 8, 17, 18, 8, 5, 2, 4, 1),
+    (2, 24, 9, 9, 40, 2, 1, 2, 1),
 ]
 
 
