@@ -20,6 +20,7 @@
 #include "conv.hpp"
 
 #include <stdlib.h>
+#include <stdio.h>
 
 namespace {
 
@@ -273,15 +274,17 @@ __device__ __forceinline__ unsigned pack2(float a, float b)
 }
 
 template <int BM, int BN, int WGM, int WGN, int STAGES, bool BWD>
-__global__ void __launch_bounds__(256) conv_gather_gemm_dma(GatherArgs g)
+__global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArgs g)
 {
+    constexpr int NW = WGM * WGN;                      // wavefronts per block
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
-    constexpr int AV = BM / 64, BV = BN / 64;
+    constexpr int RPR = 16 * NW;                       // tile rows one round of loads fills
+    constexpr int AV = BM / RPR, BV = BN / RPR;
     constexpr int ROWB = BK * 2;                       // bytes per LDS row (64)
     constexpr int STAGE_BYTES = (BM + BN) * ROWB;
     constexpr unsigned OOB = 0x7fffff00u;
-    static_assert(WGM * WGN == 4 && BK == 32, "layout");
+    static_assert(BK == 32 && AV >= 1 && BV >= 1 && TM >= 1 && TN >= 1, "layout");
 
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
@@ -320,7 +323,7 @@ __global__ void __launch_bounds__(256) conv_gather_gemm_dma(GatherArgs g)
     bool a_ok[AV];
 #pragma unroll
     for(int j = 0; j < AV; j++) {
-        const int m = m0 + lrow + 64 * j;
+        const int m = m0 + lrow + RPR * j;
         a_ok[j] = m < Mloc;
         const int mm = a_ok[j] ? m : 0;
         const int ox = mm % PW;
@@ -343,7 +346,7 @@ __global__ void __launch_bounds__(256) conv_gather_gemm_dma(GatherArgs g)
     bool b_ok[BV];
 #pragma unroll
     for(int j = 0; j < BV; j++) {
-        const int n = n0 + lrow + 64 * j;
+        const int n = n0 + lrow + RPR * j;
         b_ok[j] = n < g.Ngemm;
         b_off[j] = (b_ok[j] ? n : 0) * ktot;
     }
@@ -352,14 +355,16 @@ __global__ void __launch_bounds__(256) conv_gather_gemm_dma(GatherArgs g)
     const int csteps = (g.Cred + BK - 1) / BK;
     const int KT = nr * ns * csteps;
 
-    auto issue = [&](int stage) {
+    // one slice = AV + BV load instructions ("pieces"); issue_piece(stage, p) emits piece p of
+    // the next slice, advance() steps the slice cursor once all its pieces are out
+    auto issue_piece = [&](int stage, int p) {
         char *sa = smem + stage * STAGE_BYTES;
         char *sb = sa + BM * ROWB;
         const int c = c0 + kv;
         const bool cok = c < g.Cred;
         const int r = r0 + ri * rstep, s = s0 + si * rstep;
-#pragma unroll
-        for(int j = 0; j < AV; j++) {
+        if(p < AV) {
+            const int j = p;
             int iy, ix;
             bool ok = a_ok[j] && cok;
             if(BWD) {
@@ -374,14 +379,15 @@ __global__ void __launch_bounds__(256) conv_gather_gemm_dma(GatherArgs g)
             }
             ok = ok && iy < g.IH && ix < g.IW;
             const unsigned off = ok ? (unsigned)(((a_base[j] + iy * g.IW + ix) * g.lda + c) * 2) : OOB;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(sa + (j * 64 + wave * 16) * ROWB), 16, off, 0, 0, 0);
-        }
-        const int kb = (r * g.S + s) * g.Cred + c;
-#pragma unroll
-        for(int j = 0; j < BV; j++) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(sa + (j * RPR + wave * 16) * ROWB), 16, off, 0, 0, 0);
+        } else {
+            const int j = p - AV;
+            const int kb = (r * g.S + s) * g.Cred + c;
             const unsigned off = (b_ok[j] && cok) ? (unsigned)((b_off[j] + kb) * 2) : OOB;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(sb + (j * 64 + wave * 16) * ROWB), 16, off, 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(sb + (j * RPR + wave * 16) * ROWB), 16, off, 0, 0, 0);
         }
+    };
+    auto advance = [&]() {
         c0 += BK;
         if(c0 >= g.Cred) {
             c0 = 0;
@@ -390,6 +396,12 @@ __global__ void __launch_bounds__(256) conv_gather_gemm_dma(GatherArgs g)
                 ++ri;
             }
         }
+    };
+    auto issue = [&](int stage) {
+#pragma unroll
+        for(int p = 0; p < AV + BV; p++)
+            issue_piece(stage, p);
+        advance();
     };
 
     float16_t acc[TM][TN];
@@ -412,35 +424,46 @@ __global__ void __launch_bounds__(256) conv_gather_gemm_dma(GatherArgs g)
         if(st < KT)
             issue(st);
 
+    constexpr int NP = AV + BV, NQ = 2 * TM * TN; // load pieces and MFMAs per iteration
     for(int kt = 0; kt < KT; kt++) {
         // oldest outstanding slice = kt; newer ones may stay in flight
         // (a plain __syncthreads() would make the compiler drain every outstanding load)
         if(kt + STAGES - 2 < KT)
-            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((AV + BV) * (STAGES - 2)) : "memory");
+            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(NP * (STAGES - 2)) : "memory");
         else
             asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-        if(kt + STAGES - 1 < KT)
-            issue((kt + STAGES - 1) % STAGES);
+        const bool more = kt + STAGES - 1 < KT;
+        const int nst = (kt + STAGES - 1) % STAGES;
         const char *sa = smem + (kt % STAGES) * STAGE_BYTES;
         const char *sb = sa + BM * ROWB;
         half8_t fa[2][TM], fb[2][TN];
 #pragma unroll
-        for(int i = 0; i < TM; i++) {
-            fa[0][i] = *(const half8_t *)(sa + (wm + i * 32 + frow) * ROWB + fo0);
-            fa[1][i] = *(const half8_t *)(sa + (wm + i * 32 + frow) * ROWB + fo1);
-        }
-#pragma unroll
-        for(int j = 0; j < TN; j++) {
-            fb[0][j] = *(const half8_t *)(sb + (wn + j * 32 + frow) * ROWB + fo0);
-            fb[1][j] = *(const half8_t *)(sb + (wn + j * 32 + frow) * ROWB + fo1);
-        }
-#pragma unroll
-        for(int kk = 0; kk < 2; kk++)
+        for(int kk = 0; kk < 2; kk++) {
+            const int fo = kk ? fo1 : fo0;
 #pragma unroll
             for(int i = 0; i < TM; i++)
+                fa[kk][i] = *(const half8_t *)(sa + (wm + i * 32 + frow) * ROWB + fo);
 #pragma unroll
-                for(int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk][j], fa[kk][i], acc[i][j], 0, 0, 0);
+            for(int j = 0; j < TN; j++)
+                fb[kk][j] = *(const half8_t *)(sb + (wn + j * 32 + frow) * ROWB + fo);
+        }
+        // the next slice's loads go out between the MFMAs, so that a load waiting for the
+        // memory pipeline does not hold back this wavefront's matrix work
+#pragma unroll
+        for(int q = 0; q < NQ; q++) {
+            const int kk = q / (TM * TN), i = (q / TN) % TM, j = q % TN;
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk][j], fa[kk][i], acc[i][j], 0, 0, 0);
+#pragma unroll
+            for(int p = 0; p < NP; p++)
+                if(q == (p * NQ) / NP) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    if(more)
+                        issue_piece(nst, p);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+        }
+        if(more)
+            advance();
     }
 
     // acc[i][j][v]: pixel wm + 32*i + lane%32, channel wn + 32*j + 8*(v/4) + 4*(lane/32) + v%4
@@ -1052,6 +1075,16 @@ static int dma_stages()
     return v;
 }
 
+static int tile_override()
+{
+    static int v = -2;
+    if(v == -2) {
+        const char *e = getenv("SAGA_HIP_CONV_TILE");
+        v = e ? atoi(e) : -1;
+    }
+    return v;
+}
+
 template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
 {
     g.classes = 1;
@@ -1081,19 +1114,35 @@ template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
             if(active == 0)
                 return 0;
         }
-        if(g.Ngemm > 64) {
-            constexpr int BM = 128, BN = 128;
-            g.nblk_n = (g.Ngemm + BN - 1) / BN;
-            g.blocks_per_class = ((g.Mc + BM - 1) / BM) * g.nblk_n;
-            g.nblocks = g.blocks_per_class * active;
-            conv_gather_gemm_dma<BM, BN, 2, 2, ST, BWD><<<g.nblocks, 256, ST * (BM + BN) * 64, st>>>(g);
-        } else {
-            constexpr int BM = 256, BN = 64;
-            g.nblk_n = (g.Ngemm + BN - 1) / BN;
-            g.blocks_per_class = ((g.Mc + BM - 1) / BM) * g.nblk_n;
-            g.nblocks = g.blocks_per_class * active;
-            conv_gather_gemm_dma<BM, BN, 4, 1, ST, BWD><<<g.nblocks, 256, ST * (BM + BN) * 64, st>>>(g);
+        // tile: 256x128 on eight wavefronts (64x64 each) unless there are too few output
+        // channels to fill it; measured faster than 128x128 and than 256x256 on four or eight
+        // wavefronts on nearly every ResNet-50 layer
+        int tile = tile_override();
+        if(tile < 0)
+            tile = g.Ngemm <= 64 ? 3 : 5;
+#define LAUNCH(BM, BN, WGM, WGN)                                                                       \
+    do {                                                                                               \
+        auto kern = conv_gather_gemm_dma<BM, BN, WGM, WGN, ST, BWD>;                                    \
+        constexpr int lds = ST * (BM + BN) * 64;                                                       \
+        static bool once = false;                                                                      \
+        if(lds > 64 * 1024 && !once) {                                                                 \
+            const hipError_t e__ = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds); \
+            if(e__ != hipSuccess)                                                                      \
+                return (int)e__;                                                                       \
+            once = true;                                                                               \
+        }                                                                                              \
+        g.nblk_n = (g.Ngemm + BN - 1) / BN;                                                            \
+        g.blocks_per_class = ((g.Mc + BM - 1) / BM) * g.nblk_n;                                        \
+        g.nblocks = g.blocks_per_class * active;                                                       \
+        kern<<<g.nblocks, 64 * WGM * WGN, lds, st>>>(g);                                               \
+    } while(0)
+        switch(tile) {
+        case 2: LAUNCH(128, 128, 2, 2); break;
+        case 4: LAUNCH(256, 256, 2, 4); break;
+        case 5: LAUNCH(256, 128, 4, 2); break;
+        default: LAUNCH(256, 64, 4, 1); break;
         }
+#undef LAUNCH
         SAGA_CHECK_LAUNCH();
         return 0;
     }
