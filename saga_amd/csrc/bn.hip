@@ -33,6 +33,14 @@ template <typename T, int VN> struct Ld {
                 o[j] = (float)v[j];
         }
     }
+    static __device__ __forceinline__ V raw(const T *p) { return *(const V *)p; }
+    static __device__ __forceinline__ float at(const V &v, int j)
+    {
+        if constexpr(VN == 1)
+            return (float)v;
+        else
+            return (float)v[j];
+    }
     static __device__ __forceinline__ void store(T *p, const float (&o)[VN])
     {
         if constexpr(VN == 1) {
@@ -101,21 +109,42 @@ __global__ void __launch_bounds__(256)
         }
     }
     const bool relu = flags & SAGA_BN_RELU, add = flags & SAGA_BN_ADD;
-    for(int64_t r = (int64_t)blockIdx.x * rb + ty; r < rows; r += (int64_t)gridDim.x * rb) {
-        float xv[VN], zv[VN];
-        Ld<T, VN>::load(x + r * px + c0, xv);
-        if(add)
-            Ld<T, VN>::load(z + r * pz + c0, zv);
+    typedef Ld<T, VN> L;
+    typedef typename L::V V;
+    // MODE 1 runs right after the statistics pass over the same rows: walking them in the
+    // opposite direction meets the rows that pass touched last, which are the ones most
+    // likely to be still cached
+    const int64_t stride = (int64_t)gridDim.x * rb;
+    auto row = [&](int64_t r) { return MODE == 1 ? rows - 1 - r : r; };
+    auto finish = [&](const V &xr, const V &zr, int64_t r) {
+        float o[VN];
 #pragma unroll
         for(int j = 0; j < VN; j++) {
-            float o = xv[j] * sc[j] + sh[j];
+            float t = L::at(xr, j) * sc[j] + sh[j];
             if(add)
-                o += zv[j];
+                t += L::at(zr, j);
             if(relu)
-                o = (o != o) ? o : fmaxf(o, 0.0f);
-            xv[j] = o;
+                t = (t != t) ? t : fmaxf(t, 0.0f);
+            o[j] = t;
         }
-        Ld<T, VN>::store(y + r * py + c0, xv);
+        L::store(y + r * py + c0, o);
+    };
+    int64_t r = (int64_t)blockIdx.x * rb + ty;
+    for(; r + 3 * stride < rows; r += 4 * stride) {
+        V xr[4], zr[4];
+#pragma unroll
+        for(int u = 0; u < 4; u++) {
+            xr[u] = L::raw(x + row(r + u * stride) * px + c0);
+            zr[u] = add ? L::raw(z + row(r + u * stride) * pz + c0) : xr[u];
+        }
+#pragma unroll
+        for(int u = 0; u < 4; u++)
+            finish(xr[u], zr[u], row(r + u * stride));
+    }
+    for(; r < rows; r += stride) {
+        const V xr = L::raw(x + row(r) * px + c0);
+        const V zr = add ? L::raw(z + row(r) * pz + c0) : xr;
+        finish(xr, zr, row(r));
     }
 }
 
@@ -132,17 +161,30 @@ __global__ void __launch_bounds__(256)
     for(int j = 0; j < VN; j++)
         a0[j] = a1[j] = 0.0f;
     if(c0 < C) {
-        Ld<T, VN>::load(x + c0, k);
-        for(int64_t r = (int64_t)blockIdx.x * rb + ty; r < rows; r += (int64_t)gridDim.x * rb) {
-            float xv[VN];
-            Ld<T, VN>::load(x + r * px + c0, xv);
+        typedef Ld<T, VN> L;
+        typedef typename L::V V;
+        L::load(x + c0, k);
+        const int64_t stride = (int64_t)gridDim.x * rb;
+        auto add = [&](const V &xr) {
 #pragma unroll
             for(int j = 0; j < VN; j++) {
-                const float d = xv[j] - k[j];
+                const float d = L::at(xr, j) - k[j];
                 a0[j] += d;
                 a1[j] += d * d;
             }
+        };
+        int64_t r = (int64_t)blockIdx.x * rb + ty;
+        for(; r + 7 * stride < rows; r += 8 * stride) {
+            V xr[8];
+#pragma unroll
+            for(int u = 0; u < 8; u++)
+                xr[u] = L::raw(x + (r + u * stride) * px + c0);
+#pragma unroll
+            for(int u = 0; u < 8; u++)
+                add(xr[u]);
         }
+        for(; r < rows; r += stride)
+            add(L::raw(x + r * px + c0));
     }
 #pragma unroll
     for(int j = 0; j < VN; j++) {
@@ -237,20 +279,35 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
         for(int j = 0; j < VN; j++)
             mean[j] = save_mean[c0 + j];
-        for(int64_t r = (int64_t)blockIdx.x * rb + ty; r < rows; r += (int64_t)gridDim.x * rb) {
-            float xv[VN], gv[VN], yv[VN];
-            Ld<T, VN>::load(x + r * px + c0, xv);
-            Ld<T, VN>::load(dy + r * pdy + c0, gv);
-            if(relu)
-                Ld<T, VN>::load(y + r * py + c0, yv);
+        typedef Ld<T, VN> L;
+        typedef typename L::V V;
+        const int64_t stride = (int64_t)gridDim.x * rb;
+        auto add = [&](const V &xr, const V &gr, const V &yr) {
 #pragma unroll
             for(int j = 0; j < VN; j++) {
-                float g = gv[j];
-                if(relu && !(yv[j] > 0.0f))
+                float g = L::at(gr, j);
+                if(relu && !(L::at(yr, j) > 0.0f))
                     g = 0.0f;
                 a0[j] += g;
-                a1[j] += g * (xv[j] - mean[j]);
+                a1[j] += g * (L::at(xr, j) - mean[j]);
             }
+        };
+        int64_t r = (int64_t)blockIdx.x * rb + ty;
+        for(; r + 3 * stride < rows; r += 4 * stride) {
+            V xr[4], gr[4], yr[4];
+#pragma unroll
+            for(int u = 0; u < 4; u++) {
+                xr[u] = L::raw(x + (r + u * stride) * px + c0);
+                gr[u] = L::raw(dy + (r + u * stride) * pdy + c0);
+                yr[u] = relu ? L::raw(y + (r + u * stride) * py + c0) : gr[u];
+            }
+#pragma unroll
+            for(int u = 0; u < 4; u++)
+                add(xr[u], gr[u], yr[u]);
+        }
+        for(; r < rows; r += stride) {
+            const V xr = L::raw(x + r * px + c0), gr = L::raw(dy + r * pdy + c0);
+            add(xr, gr, relu ? L::raw(y + r * py + c0) : gr);
         }
     }
 #pragma unroll
@@ -326,34 +383,55 @@ __global__ void __launch_bounds__(256)
         k0[j] = coef[C + c0 + j];
         k1[j] = coef[2 * C + c0 + j];
     }
-    for(int64_t r = (int64_t)blockIdx.x * rb + ty; r < rows; r += (int64_t)gridDim.x * rb) {
-        float xv[VN], gv[VN], yv[VN], ov[VN];
-        Ld<T, VN>::load(x + r * px + c0, xv);
-        Ld<T, VN>::load(dy + r * pdy + c0, gv);
-        if(relu) {
-            Ld<T, VN>::load(y + r * py + c0, yv);
-#pragma unroll
-            for(int j = 0; j < VN; j++)
-                if(!(yv[j] > 0.0f))
-                    gv[j] = 0.0f;
-        }
-        if(beta_dx != 0.0f)
-            Ld<T, VN>::load(dx + r * pdx + c0, ov);
+    typedef Ld<T, VN> L;
+    typedef typename L::V V;
+    // rows are walked backwards: the statistics pass that ran just before ended at the top
+    const int64_t stride = (int64_t)gridDim.x * rb;
+    auto row = [&](int64_t r) { return rows - 1 - r; };
+    auto finish = [&](const V &xr, const V &gr, const V &yr, int64_t r) {
+        float gv[VN], ov[VN], res[VN];
 #pragma unroll
         for(int j = 0; j < VN; j++) {
-            const float v = a[j] * (gv[j] - k0[j] - (xv[j] - mean[j]) * k1[j]);
-            xv[j] = beta_dx != 0.0f ? v + beta_dx * ov[j] : v;
+            gv[j] = L::at(gr, j);
+            if(relu && !(L::at(yr, j) > 0.0f))
+                gv[j] = 0.0f;
         }
-        Ld<T, VN>::store(dx + r * pdx + c0, xv);
+        if(beta_dx != 0.0f)
+            L::load(dx + r * pdx + c0, ov);
+#pragma unroll
+        for(int j = 0; j < VN; j++) {
+            const float v = a[j] * (gv[j] - k0[j] - (L::at(xr, j) - mean[j]) * k1[j]);
+            res[j] = beta_dx != 0.0f ? v + beta_dx * ov[j] : v;
+        }
+        L::store(dx + r * pdx + c0, res);
         if(dz) {
             if(beta_dz != 0.0f) {
-                Ld<T, VN>::load(dz + r * pdz + c0, ov);
+                L::load(dz + r * pdz + c0, ov);
 #pragma unroll
                 for(int j = 0; j < VN; j++)
                     gv[j] += beta_dz * ov[j];
             }
-            Ld<T, VN>::store(dz + r * pdz + c0, gv);
+            L::store(dz + r * pdz + c0, gv);
         }
+    };
+    int64_t r = (int64_t)blockIdx.x * rb + ty;
+    for(; r + 3 * stride < rows; r += 4 * stride) {
+        V xr[4], gr[4], yr[4];
+#pragma unroll
+        for(int u = 0; u < 4; u++) {
+            const int64_t q = row(r + u * stride);
+            xr[u] = L::raw(x + q * px + c0);
+            gr[u] = L::raw(dy + q * pdy + c0);
+            yr[u] = relu ? L::raw(y + q * py + c0) : gr[u];
+        }
+#pragma unroll
+        for(int u = 0; u < 4; u++)
+            finish(xr[u], gr[u], yr[u], row(r + u * stride));
+    }
+    for(; r < rows; r += stride) {
+        const int64_t q = row(r);
+        const V xr = L::raw(x + q * px + c0), gr = L::raw(dy + q * pdy + c0);
+        finish(xr, gr, relu ? L::raw(y + q * py + c0) : gr, q);
     }
 }
 

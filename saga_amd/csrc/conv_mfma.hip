@@ -273,18 +273,23 @@ __device__ __forceinline__ unsigned pack2(float a, float b)
     return __builtin_bit_cast(unsigned, v);
 }
 
-template <int BM, int BN, int WGM, int WGN, int STAGES, bool BWD>
+template <int BM, int BN, int WGM, int WGN, int STAGES, int BKT, bool BWD>
 __global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArgs g)
 {
     constexpr int NW = WGM * WGN;                      // wavefronts per block
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
-    constexpr int RPR = 16 * NW;                       // tile rows one round of loads fills
+    constexpr int ROWB = BKT * 2;                      // bytes per LDS row (64 or 128)
+    constexpr int SLOTS = ROWB / 16;                   // 16-byte slots per row
+    constexpr int RPI = 64 / SLOTS;                    // rows one load instruction fills
+    constexpr int RPR = RPI * NW;                      // tile rows one round of loads fills
     constexpr int AV = BM / RPR, BV = BN / RPR;
-    constexpr int ROWB = BK * 2;                       // bytes per LDS row (64)
     constexpr int STAGE_BYTES = (BM + BN) * ROWB;
     constexpr unsigned OOB = 0x7fffff00u;
-    static_assert(BK == 32 && AV >= 1 && BV >= 1 && TM >= 1 && TN >= 1, "layout");
+    static_assert((BKT == 32 || BKT == 64) && RPR % 16 == 0 && AV >= 1 && BV >= 1 && TM >= 1 && TN >= 1, "layout");
+    // slot swizzle of a row: 64-byte rows alternate between four bank quarters, so rows
+    // 4 apart need different slots; 128-byte rows between two halves, rows 2 apart do
+    auto swz_of = [](int row) { return SLOTS == 4 ? (row >> 2) & 3 : (row >> 1) & 7; };
 
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
@@ -317,8 +322,8 @@ __global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArg
 
     // this lane fills slot (tid & 3) of row lrow (+64 per round) and fetches the logical
     // channel vector that the swizzle assigns to that slot
-    const int lrow = tid >> 2;
-    const int kv = (((tid & 3) ^ ((lrow >> 2) & 3))) * 8;
+    const int lrow = tid / SLOTS;
+    const int kv = ((tid % SLOTS) ^ swz_of(lrow)) * 8;
     int a_base[AV], a_y[AV], a_x[AV];
     bool a_ok[AV];
 #pragma unroll
@@ -352,7 +357,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArg
     }
 
     int ri = 0, si = 0, c0 = 0; // tap counters and channel offset of the NEXT slice to be issued
-    const int csteps = (g.Cred + BK - 1) / BK;
+    const int csteps = (g.Cred + BKT - 1) / BKT;
     const int KT = nr * ns * csteps;
 
     // one slice = AV + BV load instructions ("pieces"); issue_piece(stage, p) emits piece p of
@@ -379,16 +384,16 @@ __global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArg
             }
             ok = ok && iy < g.IH && ix < g.IW;
             const unsigned off = ok ? (unsigned)(((a_base[j] + iy * g.IW + ix) * g.lda + c) * 2) : OOB;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(sa + (j * RPR + wave * 16) * ROWB), 16, off, 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(sa + (j * RPR + wave * RPI) * ROWB), 16, off, 0, 0, 0);
         } else {
             const int j = p - AV;
             const int kb = (r * g.S + s) * g.Cred + c;
             const unsigned off = (b_ok[j] && cok) ? (unsigned)((b_off[j] + kb) * 2) : OOB;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(sb + (j * RPR + wave * 16) * ROWB), 16, off, 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(sb + (j * RPR + wave * RPI) * ROWB), 16, off, 0, 0, 0);
         }
     };
     auto advance = [&]() {
-        c0 += BK;
+        c0 += BKT;
         if(c0 >= g.Cred) {
             c0 = 0;
             if(++si == ns) {
@@ -415,16 +420,20 @@ __global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArg
 
     const int wm = (wave / WGN) * WTM, wn = (wave % WGN) * WTN;
     const int frow = lane & 31;
-    const int swz = (frow >> 2) & 3;
-    // byte offsets of this lane's two fragment vectors (k 0..15 and 16..31) inside a row
-    const int fo0 = ((0 + (lane >> 5)) ^ swz) * 16, fo1 = ((2 + (lane >> 5)) ^ swz) * 16;
+    const int swz = swz_of(frow);
+    // byte offset inside a row of this lane's fragment vector for MFMA step kk (k = 16*kk ..)
+    constexpr int KS = BKT / 16;
+    int fo[KS];
+#pragma unroll
+    for(int kk = 0; kk < KS; kk++)
+        fo[kk] = ((2 * kk + (lane >> 5)) ^ swz) * 16;
 
 #pragma unroll
     for(int st = 0; st < STAGES - 1; st++)
         if(st < KT)
             issue(st);
 
-    constexpr int NP = AV + BV, NQ = 2 * TM * TN; // load pieces and MFMAs per iteration
+    constexpr int NP = AV + BV, NQ = KS * TM * TN; // load pieces and MFMAs per iteration
     for(int kt = 0; kt < KT; kt++) {
         // oldest outstanding slice = kt; newer ones may stay in flight
         // (a plain __syncthreads() would make the compiler drain every outstanding load)
@@ -436,16 +445,15 @@ __global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArg
         const int nst = (kt + STAGES - 1) % STAGES;
         const char *sa = smem + (kt % STAGES) * STAGE_BYTES;
         const char *sb = sa + BM * ROWB;
-        half8_t fa[2][TM], fb[2][TN];
+        half8_t fa[KS][TM], fb[KS][TN];
 #pragma unroll
-        for(int kk = 0; kk < 2; kk++) {
-            const int fo = kk ? fo1 : fo0;
+        for(int kk = 0; kk < KS; kk++) {
 #pragma unroll
             for(int i = 0; i < TM; i++)
-                fa[kk][i] = *(const half8_t *)(sa + (wm + i * 32 + frow) * ROWB + fo);
+                fa[kk][i] = *(const half8_t *)(sa + (wm + i * 32 + frow) * ROWB + fo[kk]);
 #pragma unroll
             for(int j = 0; j < TN; j++)
-                fb[kk][j] = *(const half8_t *)(sb + (wn + j * 32 + frow) * ROWB + fo);
+                fb[kk][j] = *(const half8_t *)(sb + (wn + j * 32 + frow) * ROWB + fo[kk]);
         }
         // the next slice's loads go out between the MFMAs, so that a load waiting for the
         // memory pipeline does not hold back this wavefront's matrix work
@@ -1116,14 +1124,15 @@ template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
         }
         // tile: 256x128 on eight wavefronts (64x64 each) unless there are too few output
         // channels to fill it; measured faster than 128x128 and than 256x256 on four or eight
-        // wavefronts on nearly every ResNet-50 layer
+        // wavefronts on nearly every ResNet-50 layer, and faster than the same tiles with
+        // 64-wide reduction slices (which leave room for one block per CU only)
         int tile = tile_override();
         if(tile < 0)
             tile = g.Ngemm <= 64 ? 3 : 5;
-#define LAUNCH(BM, BN, WGM, WGN)                                                                       \
+#define LAUNCH(BM, BN, WGM, WGN, BKT)                                                                  \
     do {                                                                                               \
-        auto kern = conv_gather_gemm_dma<BM, BN, WGM, WGN, ST, BWD>;                                    \
-        constexpr int lds = ST * (BM + BN) * 64;                                                       \
+        auto kern = conv_gather_gemm_dma<BM, BN, WGM, WGN, ST, BKT, BWD>;                               \
+        constexpr int lds = ST * (BM + BN) * BKT * 2;                                                  \
         static bool once = false;                                                                      \
         if(lds > 64 * 1024 && !once) {                                                                 \
             const hipError_t e__ = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds); \
@@ -1137,10 +1146,9 @@ template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
         kern<<<g.nblocks, 64 * WGM * WGN, lds, st>>>(g);                                               \
     } while(0)
         switch(tile) {
-        case 2: LAUNCH(128, 128, 2, 2); break;
-        case 4: LAUNCH(256, 256, 2, 4); break;
-        case 5: LAUNCH(256, 128, 4, 2); break;
-        default: LAUNCH(256, 64, 4, 1); break;
+        case 2: LAUNCH(128, 128, 2, 2, 32); break;
+        case 5: LAUNCH(256, 128, 4, 2, 32); break;
+        default: LAUNCH(256, 64, 4, 1, 32); break;
         }
 #undef LAUNCH
         SAGA_CHECK_LAUNCH();
