@@ -71,6 +71,24 @@ def cpu_baseline(batch, image):
                       f"{dt:.1f} s of CPU work"}
 
 
+def copy_calibration():
+    """Five plain copies of 1 GiB (fp32 -> fp32 through saga_hip_axpby, alpha 1, beta 0): under
+    `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` the ew_flat kernel's counter value divided by
+    1 GiB is the factor that turns the counters of the other kernels into bytes."""
+    import ctypes as C
+    import torch
+    from saga_amd import kernels as K
+
+    n = 1 << 28
+    src = torch.ones(1, 1, 1, n, dtype=torch.float32, device="cuda")
+    dst = torch.zeros_like(src)
+    for _ in range(5):
+        K.check(K.lib().saga_hip_axpby(C.byref(K.view(src)), C.byref(K.view(dst)), 1.0, 0.0, None))
+    torch.cuda.synchronize()
+    assert float(dst[0, 0, 0, -1]) == 1.0
+    print(json.dumps({"copy_bytes": n * 4, "launches": 5}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -78,12 +96,16 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--batch", type=int, default=256)
     ap.add_argument("--image", type=int, default=224)
-    ap.add_argument("--cpu-batch", type=int, default=2)
+    ap.add_argument("--cpu-batch", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-profile", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run a plain 1 GiB device copy five times and exit (reference for the HBM counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build drives exactly one GPU (no collectives, no sharding); run with --gpus 1")
+    if args.copy_calibration:
+        return copy_calibration()
 
     from saga_amd import api as S
     from saga_amd import networks as N

@@ -217,6 +217,36 @@ __device__ __forceinline__ double wave_sum_f64(double v)
     return v;
 }
 
+// Adds the gx per-block partial pairs of channel c over one wavefront, in a fixed order.
+// The loads of a lane are independent: eight are issued before any is consumed, so the
+// wavefront pays the memory latency a few times, not once per partial.
+__device__ __forceinline__ void sum_partials(const float *__restrict__ partial, int gx, int C, int c, int lane,
+                                             double &s0, double &s1)
+{
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    const float2_t *p = (const float2_t *)partial + c;
+    double a0 = 0, a1 = 0;
+    int g = lane;
+    for(; g + 7 * 64 < gx; g += 8 * 64) {
+        float2_t v[8];
+#pragma unroll
+        for(int u = 0; u < 8; u++)
+            v[u] = p[(int64_t)(g + u * 64) * C];
+#pragma unroll
+        for(int u = 0; u < 8; u++) {
+            a0 += v[u][0];
+            a1 += v[u][1];
+        }
+    }
+    for(; g < gx; g += 64) {
+        const float2_t v = p[(int64_t)g * C];
+        a0 += v[0];
+        a1 += v[1];
+    }
+    s0 = wave_sum_f64(a0);
+    s1 = wave_sum_f64(a1);
+}
+
 // Finalize: mean, biased variance, invstd, running statistics, fused scale/shift.
 // One wavefront per channel adds the per-block partials (lanes stride over the blocks).
 template <typename T>
@@ -229,16 +259,14 @@ __global__ void __launch_bounds__(256)
     const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
     if(c >= C)
         return;
-    double s0 = 0, s1 = 0;
-    for(int g = lane; g < gx; g += 64) {
-        s0 += partial[((int64_t)g * C + c) * 2];
-        s1 += partial[((int64_t)g * C + c) * 2 + 1];
-    }
-    s0 = wave_sum_f64(s0);
-    s1 = wave_sum_f64(s1);
+    // parameter loads first: they overlap the partial-sum loads instead of following them
+    const double k = (double)(float)xrow0[c * kstride];
+    const float sv = s[c], bv = b[c];
+    const float rm_old = run_m ? run_m[c] : 0.0f, rv_old = run_v ? run_v[c] : 0.0f;
+    double s0, s1;
+    sum_partials(partial, gx, C, c, lane, s0, s1);
     if(lane != 0)
         return;
-    const double k = (double)(float)xrow0[c * kstride];
     const double dm = s0 / M;
     double var = s1 / M - dm * dm;
     if(var < 0)
@@ -250,14 +278,14 @@ __global__ void __launch_bounds__(256)
     if(save_invstd)
         save_invstd[c] = inv;
     if(run_m)
-        run_m[c] = (float)((1.0 - expavg) * run_m[c] + expavg * mean);
+        run_m[c] = (float)((1.0 - expavg) * rm_old + expavg * mean);
     if(run_v) {
         const double unb = M > 1 ? var * M / (M - 1.0) : var;
-        run_v[c] = (float)((1.0 - expavg) * run_v[c] + expavg * unb);
+        run_v[c] = (float)((1.0 - expavg) * rv_old + expavg * unb);
     }
-    const float sc = s[c] * inv;
+    const float sc = sv * inv;
     ss[c] = sc;
-    ss[C + c] = b[c] - (float)mean * sc;
+    ss[C + c] = bv - (float)mean * sc;
 }
 
 // Pass 1 of backward: partial sums of dy' and dy'*(x-mean); dy' = dy masked by y>0 when fused relu.
@@ -344,20 +372,17 @@ __global__ void __launch_bounds__(256)
     const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
     if(c >= C)
         return;
-    double s0 = 0, s1 = 0;
-    for(int g = lane; g < gx; g += 64) {
-        s0 += partial[((int64_t)g * C + c) * 2];
-        s1 += partial[((int64_t)g * C + c) * 2 + 1];
-    }
-    s0 = wave_sum_f64(s0);
-    s1 = wave_sum_f64(s1);
+    const double inv = save_invstd[c];
+    const float sv = s[c];
+    const float ds_old = beta_p != 0.0f ? ds[c] : 0.0f, db_old = beta_p != 0.0f ? db[c] : 0.0f;
+    double s0, s1;
+    sum_partials(partial, gx, C, c, lane, s0, s1);
     if(lane != 0)
         return;
-    const double inv = save_invstd[c];
     const double dsv = s1 * inv;
-    ds[c] = (float)(beta_p != 0.0f ? dsv + (double)beta_p * ds[c] : dsv);
-    db[c] = (float)(beta_p != 0.0f ? s0 + (double)beta_p * db[c] : s0);
-    coef[c] = (float)(s[c] * inv);
+    ds[c] = (float)(beta_p != 0.0f ? dsv + (double)beta_p * ds_old : dsv);
+    db[c] = (float)(beta_p != 0.0f ? s0 + (double)beta_p * db_old : s0);
+    coef[c] = (float)(sv * inv);
     coef[C + c] = (float)(s0 / M);
     coef[2 * C + c] = (float)(dsv * inv / M);
 }
@@ -484,10 +509,10 @@ __global__ void __launch_bounds__(256)
         if(save_invstd)
             save_invstd[c] = inv;
         if(run_m)
-            run_m[c] = (float)((1.0 - expavg) * run_m[c] + expavg * mean);
+            run_m[c] = (float)((1.0 - expavg) * rm_old + expavg * mean);
         if(run_v) {
             const double unb = M > 1 ? var * M / (M - 1.0) : var;
-            run_v[c] = (float)((1.0 - expavg) * run_v[c] + expavg * unb);
+            run_v[c] = (float)((1.0 - expavg) * rv_old + expavg * unb);
         }
         const float sc = s[c] * inv;
         ss[c] = sc;
