@@ -509,10 +509,10 @@ __global__ void __launch_bounds__(256)
         if(save_invstd)
             save_invstd[c] = inv;
         if(run_m)
-            run_m[c] = (float)((1.0 - expavg) * rm_old + expavg * mean);
+            run_m[c] = (float)((1.0 - expavg) * run_m[c] + expavg * mean);
         if(run_v) {
             const double unb = M > 1 ? var * M / (M - 1.0) : var;
-            run_v[c] = (float)((1.0 - expavg) * rv_old + expavg * unb);
+            run_v[c] = (float)((1.0 - expavg) * run_v[c] + expavg * unb);
         }
         const float sc = s[c] * inv;
         ss[c] = sc;
