@@ -20,6 +20,7 @@
 #include "conv.hpp"
 
 #include <stdlib.h>
+#include <algorithm>
 #include <stdio.h>
 
 namespace {
@@ -1061,6 +1062,88 @@ static int ilog2_exact(int v)
     return (1 << s) == v ? s : -1;
 }
 
+// ---------------------------------------------------------------- thin inputs (C <= 4)
+//
+// A convolution over 1..4 input channels (the RGB stem) would spend a 32-wide reduction slice
+// on the 3 channels of one tap.  Instead x is copied once into x4[N][H+2pad][Wp][4]
+// (spatially zero-padded, 4 halves = 8 bytes per pixel); the 8 pixels x4[n][iy][ix .. ix+7]
+// are then 32 contiguous halves holding the taps s = 0..7 of filter row r, so the same
+// gather kernels run a "virtual" convolution with R taps of 32 channels each: pixel pitch 4,
+// channel extent 32 (rows overlap), filter repacked to [K][R][s*4+c] with zeros for s >= S
+// and c >= C.  ix = ox*stride is even for even strides, which keeps every 16-byte load aligned.
+
+__global__ void __launch_bounds__(256)
+    pad_thin(const half_t *__restrict__ x, int64_t sp, int C, int H, int W, int pad, half_t *__restrict__ x4, int Hp,
+             int Wp, int64_t total)
+{
+    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+    for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        const int wp = (int)(i % Wp);
+        const int64_t t = i / Wp;
+        const int hp = (int)(t % Hp);
+        const int64_t n = t / Hp;
+        const int h = hp - pad, w = wp - pad;
+        h4 v = {0, 0, 0, 0};
+        if(h >= 0 && h < H && w >= 0 && w < W) {
+            const half_t *src = x + ((n * H + h) * W + w) * sp;
+            for(int c = 0; c < C; c++)
+                v[c] = src[c];
+        }
+        *(h4 *)(x4 + i * 4) = v;
+    }
+}
+
+// wv[k][r][s*4 + c] = w[k][r][s][c] (s < S, c < C), 0 elsewhere; 32 halves per (k, r)
+__global__ void __launch_bounds__(256)
+    repack_thin_filter(const half_t *__restrict__ w, half_t *__restrict__ wv, int C, int S, int64_t total)
+{
+    for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        const int e = (int)(i & 31), s = e >> 2, c = e & 3;
+        const int64_t kr = i >> 5;
+        wv[i] = (s < S && c < C) ? w[(kr * S + s) * C + c] : (half_t)0;
+    }
+}
+
+// dw[k][r][s][c] = alpha * sum_p partial[p][k][r][s*4 + c] + beta * dw
+__global__ void __launch_bounds__(256)
+    thin_filter_reduce(const float *__restrict__ partial, half_t *__restrict__ dw, int64_t n, int C, int S, int splits,
+                       float alpha, float beta)
+{
+    const int64_t np = n / (S * C) * 32;
+    for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        const int c = (int)(i % C);
+        const int64_t t = i / C;
+        const int s = (int)(t % S);
+        const int64_t j = (t / S) * 32 + s * 4 + c;
+        float acc = 0;
+        for(int p = 0; p < splits; p++)
+            acc += partial[(int64_t)p * np + j];
+        acc *= alpha;
+        if(beta != 0.0f)
+            acc += beta * (float)dw[i];
+        dw[i] = (half_t)acc;
+    }
+}
+
+struct ThinGeom {
+    int Hp, Wp;
+    size_t x4_bytes, wv_bytes;
+};
+
+static bool thin_ok(const ConvGeom &g, ThinGeom *t)
+{
+    if(g.C > 4 || g.S > 8 || g.dil != 1 || g.stride < 2 || (g.stride & 1) || g.group != 1)
+        return false;
+    t->Hp = g.H + 2 * g.pad;
+    t->Wp = (g.W + 2 * g.pad + 8 + 1) & ~1;
+    const int64_t px = (int64_t)g.N * t->Hp * t->Wp;
+    if(px * 8 >= 0x7fffff00)
+        return false;
+    t->x4_bytes = ((size_t)px * 8 + 255) & ~(size_t)255;
+    t->wv_bytes = ((size_t)g.K * g.R * 32 * sizeof(half_t) + 255) & ~(size_t)255;
+    return true;
+}
+
 // out[row][0..C) = 0 for rows of pitch `pitch` elements (C and pitch multiples of 8, 16-byte aligned)
 __global__ void __launch_bounds__(256) zero_rows(half_t *__restrict__ out, int64_t rows, int C, int64_t pitch)
 {
@@ -1207,15 +1290,25 @@ size_t conv_mfma_workspace(int kind, const SagaTensorView *x, const SagaTensorVi
     const size_t Cp = round8(g.C);
     const size_t xpad = ((size_t)g.N * g.H * g.W * Cp * sizeof(half_t) + 255) & ~(size_t)255;
     const size_t wpad = ((size_t)g.K * g.R * g.S * Cp * sizeof(half_t) + 255) & ~(size_t)255;
+    ThinGeom tg;
+    const bool thin = thin_ok(g, &tg);
     if(kind == SAGA_CONV_FWD)
-        return xpad + wpad + 256;
+        return std::max(xpad + wpad, thin ? tg.x4_bytes + tg.wv_bytes : 0) + 256;
     if(kind == SAGA_CONV_BWD_DATA)
         return (size_t)g.K * g.C * g.R * g.S * sizeof(half_t) + 256;
     if(kind == SAGA_CONV_BWD_FILTER) {
         ConvGeom gp = g;
         gp.C = (int)Cp;
         const FilterPlan p = plan_filter(gp);
-        return xpad + (size_t)p.splits * g.K * g.R * g.S * Cp * sizeof(float) + 256;
+        size_t need = xpad + (size_t)p.splits * g.K * g.R * g.S * Cp * sizeof(float);
+        if(thin) {
+            ConvGeom gv = g;
+            gv.C = 32;
+            gv.S = 1;
+            const FilterPlan pv = plan_filter(gv);
+            need = std::max(need, tg.x4_bytes + (size_t)pv.splits * g.K * g.R * 32 * sizeof(float));
+        }
+        return need + 256;
     }
     return 0;
 }
@@ -1227,6 +1320,32 @@ int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTe
     bool pad = false;
     if(!common_ok(x, w, y, g, &lx, &ly, &pad))
         return SAGA_HIP_EUNSUPPORTED;
+    ThinGeom tg;
+    if(dma_stages() >= 2 && thin_ok(g, &tg) && ly.rows * ly.pitch < ((int64_t)1 << 31)) {
+        if(!ws || ws_bytes < tg.x4_bytes + tg.wv_bytes || !aligned16(ws))
+            return SAGA_HIP_EWORKSPACE;
+        half_t *x4 = (half_t *)ws, *wv = (half_t *)((char *)ws + tg.x4_bytes);
+        const int64_t px = (int64_t)g.N * tg.Hp * tg.Wp, wn = (int64_t)g.K * g.R * 32;
+        pad_thin<<<grid_for(px, 256, 256 * 16), 256, 0, st>>>((const half_t *)x->ptr, lx.pitch, g.C, g.H, g.W, g.pad, x4,
+                                                              tg.Hp, tg.Wp, px);
+        repack_thin_filter<<<grid_for(wn, 256, 256 * 16), 256, 0, st>>>((const half_t *)w->ptr, wv, g.C, g.S, wn);
+        GatherArgs a;
+        a.a = x4;
+        a.b = wv;
+        a.out = (half_t *)y->ptr;
+        a.M = (int)ly.rows;
+        a.Ngemm = g.K;
+        a.Cred = 32;
+        a.IH = tg.Hp; a.IW = tg.Wp; a.OH = g.P; a.OW = g.Q;
+        a.R = g.R; a.S = 1;
+        a.pad = 0; a.stride = g.stride; a.dil = 1; a.sshift = 0;
+        a.lda = 4;
+        a.ldo = (int)ly.pitch;
+        a.alpha = alpha; a.beta = beta;
+        a.a_bytes = (unsigned)(px * 8);
+        a.b_bytes = (unsigned)(wn * 2);
+        return launch_gather<false>(a, st);
+    }
     GatherArgs a;
     a.a = (const half_t *)x->ptr;
     a.b = (const half_t *)w->ptr;
@@ -1311,11 +1430,51 @@ int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, cons
         return SAGA_HIP_EUNSUPPORTED;
     if(g.K % 8 || ldy.pitch % 8 || !aligned16(dy->ptr))
         return SAGA_HIP_EUNSUPPORTED;
+    const int64_t n = (int64_t)g.K * g.R * g.S * g.C;
+    ThinGeom tg;
+    if(dma_stages() >= 2 && thin_ok(g, &tg)) {
+        ConvGeom gv = g;
+        gv.C = 32;
+        gv.S = 1;
+        const FilterPlan p = plan_filter(gv);
+        const size_t need = tg.x4_bytes + (size_t)p.splits * g.K * g.R * 32 * sizeof(float);
+        const int64_t yb = ((ldy.rows - 1) * ldy.pitch + ldy.C) * 2;
+        if(!ws || ws_bytes < need || !aligned16(ws))
+            return SAGA_HIP_EWORKSPACE;
+        if(yb >= 0x7fffff00)
+            return SAGA_HIP_EUNSUPPORTED;
+        half_t *x4 = (half_t *)ws;
+        const int64_t px = (int64_t)g.N * tg.Hp * tg.Wp;
+        pad_thin<<<grid_for(px, 256, 256 * 16), 256, 0, st>>>((const half_t *)x->ptr, lx.pitch, g.C, g.H, g.W, g.pad, x4,
+                                                              tg.Hp, tg.Wp, px);
+        FilterArgs a;
+        a.x = x4;
+        a.ldx = 4;
+        a.dy = (const half_t *)dy->ptr;
+        a.partial = (float *)((char *)ws + tg.x4_bytes);
+        a.M = (int)ldy.rows;
+        a.K = g.K; a.C = 32; a.RSC = g.R * 32;
+        a.H = tg.Hp; a.W = tg.Wp; a.P = g.P; a.Q = g.Q; a.S = 1;
+        a.pad = 0; a.stride = g.stride; a.dil = 1;
+        a.ldy = (int)ldy.pitch;
+        a.tiles_k = p.tiles_k; a.tiles_c = p.tiles_c;
+        a.splits = p.splits; a.m_per_split = p.m_per_split;
+        const int blocks = p.tiles_k * p.tiles_c * p.splits;
+        constexpr int ST = 3;
+        if(p.bm == 128)
+            conv_bwd_filter_dma<128, 128, ST><<<blocks, 256, ST * BK * 512, st>>>(a, (unsigned)(px * 8), (unsigned)yb);
+        else
+            conv_bwd_filter_dma<64, 128, ST><<<blocks, 256, ST * BK * 384, st>>>(a, (unsigned)(px * 8), (unsigned)yb);
+        SAGA_CHECK_LAUNCH();
+        thin_filter_reduce<<<grid_for(n, 256, 256 * 8), 256, 0, st>>>(a.partial, (half_t *)dw->ptr, n, g.C, g.S, p.splits,
+                                                                    alpha, beta);
+        SAGA_CHECK_LAUNCH();
+        return 0;
+    }
     const int Cp = pad ? round8(g.C) : g.C;
     ConvGeom gp = g;
     gp.C = Cp;
     const FilterPlan p = plan_filter(gp);
-    const int64_t n = (int64_t)g.K * g.R * g.S * g.C;
     const size_t xpad = pad ? (((size_t)lx.rows * Cp * sizeof(half_t) + 255) & ~(size_t)255) : 0;
     const size_t need = xpad + (size_t)p.splits * g.K * g.R * g.S * Cp * sizeof(float);
     if(!ws || ws_bytes < need || !aligned16(ws))

@@ -42,6 +42,9 @@ CONV_CASES = [
     (2, 16, 13, 13, 24, 3, 0, 2, 1),
     (1, 8, 17, 18, 8, 5, 2, 4, 1),
     (2, 24, 9, 9, 40, 2, 1, 2, 1),
+    (2, 4, 12, 12, 16, 5, 2, 2, 1),
+    (2, 1, 10, 11, 8, 3, 1, 2, 1),
+    (1, 3, 21, 21, 72, 8, 3, 4, 1),
 ]
 
 
