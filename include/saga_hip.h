@@ -103,6 +103,21 @@ int saga_hip_conv2d_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy
                                const SagaConvParams *p, float alpha, float beta, void *workspace,
                                size_t ws_bytes, saga_stream_t stream);
 
+/* ---- convolution forward that also leaves, for a batch normalisation that consumes y, the
+ *      per-channel sum and sum of squares of y as partial[rows][K][2] (one row per block of
+ *      output pixels; *partial_rows receives the count).  The reference runs
+ *      cudnnConvolutionForward (src/cuda/cuda_dnn.cpp:207-221) and then
+ *      cudnnBatchNormalizationForwardTrainingEx (:1717-1741), which reads y once more for these
+ *      sums; here they fall out of the convolution's epilogue.  beta is 0.  Returns
+ *      SAGA_HIP_EUNSUPPORTED (nothing written to y) when the fp16 channels-last MFMA path does
+ *      not cover the problem: run saga_hip_conv2d_fwd and saga_hip_bn_train_fwd instead.
+ *      _size: bytes `partial` must hold (0: never supported for these operands). */
+size_t saga_hip_conv2d_fwd_bnstats_size(const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y,
+                                        const SagaConvParams *p);
+int saga_hip_conv2d_fwd_bnstats(const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y,
+                                const SagaConvParams *p, float alpha, void *workspace, size_t ws_bytes,
+                                float *partial, size_t partial_bytes, int *partial_rows, saga_stream_t stream);
+
 /* y[n,c,:,:] += b[c] : cudnnAddTensor of a {1,C,1,1} bias (src/cuda/cuda_dnn.cpp:39-68). b is fp32 or y's type. */
 int saga_hip_bias_add(const SagaTensorView *y, const SagaTensorView *b, saga_stream_t stream);
 /* db[c] = beta*db + sum_{n,h,w} dy : cudnnConvolutionBackwardBias (src/cuda/cuda_dnn.cpp:378-385). */
@@ -129,6 +144,13 @@ int saga_hip_bn_train_fwd(const SagaTensorView *x, const SagaTensorView *z, cons
                           const float *s, const float *b, float *run_m, float *run_v, float *save_mean,
                           float *save_invstd, float eps, float expavg, int flags, void *workspace,
                           size_t ws_bytes, saga_stream_t stream);
+/* training forward from per-channel partial sums of x that already exist (the output of
+ * saga_hip_conv2d_fwd_bnstats): finalises the statistics and normalises, without the pass
+ * over x that computes them.  workspace: 2*C floats.  Channels-last tensors only. */
+int saga_hip_bn_train_fwd_partials(const SagaTensorView *x, const SagaTensorView *z, const SagaTensorView *y,
+                                   const float *s, const float *b, float *run_m, float *run_v, float *save_mean,
+                                   float *save_invstd, float eps, float expavg, int flags, const float *partial,
+                                   int partial_rows, void *workspace, size_t ws_bytes, saga_stream_t stream);
 int saga_hip_bn_bwd(const SagaTensorView *x, const SagaTensorView *y, const SagaTensorView *dy,
                     const SagaTensorView *dx, const SagaTensorView *dz, const float *s, const float *save_mean,
                     const float *save_invstd, float *ds, float *db, float beta_dx, float beta_dz, float beta_p,

@@ -260,7 +260,7 @@ __global__ void __launch_bounds__(256)
     if(c >= C)
         return;
     // parameter loads first: they overlap the partial-sum loads instead of following them
-    const double k = (double)(float)xrow0[c * kstride];
+    const double k = xrow0 ? (double)(float)xrow0[c * kstride] : 0.0;
     const float sv = s[c], bv = b[c];
     const float rm_old = run_m ? run_m[c] : 0.0f, rv_old = run_v ? run_v[c] : 0.0f;
     double s0, s1;
@@ -755,6 +755,50 @@ int saga_hip_bn_train_fwd(const SagaTensorView *x, const SagaTensorView *z, cons
     } else {
         return SAGA_HIP_EUNSUPPORTED;
     }
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
+int saga_hip_bn_train_fwd_partials(const SagaTensorView *x, const SagaTensorView *z, const SagaTensorView *y,
+                                   const float *s, const float *b, float *run_m, float *run_v, float *save_mean,
+                                   float *save_invstd, float eps, float expavg, int flags, const float *partial,
+                                   int partial_rows, void *workspace, size_t ws_bytes, saga_stream_t stream)
+{
+    if(!valid_view(x) || !valid_view(y) || !s || !b || !partial || partial_rows < 1)
+        return SAGA_HIP_EINVAL;
+    const bool add = flags & SAGA_BN_ADD;
+    if(add && !valid_view(z))
+        return SAGA_HIP_EINVAL;
+    if(!same_dims(x, y) || (add && !same_dims(x, z)))
+        return SAGA_HIP_ESHAPE;
+    if(x->dtype != y->dtype || (add && z->dtype != x->dtype) || (x->dtype != SAGA_HALF && x->dtype != SAGA_FLOAT))
+        return SAGA_HIP_EUNSUPPORTED;
+    CLInfo lx, ly, lz = {};
+    if(!as_channels_last(x, &lx) || !as_channels_last(y, &ly) || (add && !as_channels_last(z, &lz)))
+        return SAGA_HIP_EUNSUPPORTED;
+    const int C = lx.C;
+    if(!workspace || ws_bytes < 2 * (size_t)C * sizeof(float))
+        return SAGA_HIP_EWORKSPACE;
+    hipStream_t st = as_stream(stream);
+    float *ss = (float *)workspace;
+    const int vn = vec_width(x->dtype, C, {x, y, add ? z : nullptr}, {lx.pitch, ly.pitch, add ? lz.pitch : 0});
+    Shape sh = plan(lx.rows, C / vn);
+    dim3 grid(sh.gx, sh.gy);
+#define GO(T, VN)                                                                                                   \
+    do {                                                                                                            \
+        bn_stats_finalize<T><<<(C + 3) / 4, 256, 0, st>>>(partial, partial_rows, (const T *)nullptr, 1, s, b, run_m, \
+                                                          run_v, save_mean, save_invstd, ss, (double)lx.rows, C,    \
+                                                          eps, expavg);                                             \
+        bn_apply_cl<T, VN, 1><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, add ? (const T *)z->ptr : nullptr,   \
+                                                    lz.pitch, (T *)y->ptr, ly.pitch, nullptr, nullptr, nullptr,     \
+                                                    nullptr, ss, eps, lx.rows, C, sh.cvb, flags);                   \
+    } while(0)
+    if(x->dtype == SAGA_HALF) {
+        if(vn == 8) GO(half_t, 8); else GO(half_t, 1);
+    } else {
+        if(vn == 4) GO(float, 4); else GO(float, 1);
+    }
+#undef GO
     SAGA_CHECK_LAUNCH();
     return 0;
 }

@@ -69,6 +69,31 @@ int saga_hip_conv2d_fwd(const SagaTensorView *x, const SagaTensorView *w, const 
     return conv_direct_fwd(x, w, y, g, alpha, beta, as_stream(stream));
 }
 
+size_t saga_hip_conv2d_fwd_bnstats_size(const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y,
+                                        const SagaConvParams *p)
+{
+    ConvGeom g;
+    if(geometry(x, w, y, p, &g) || x->dtype != SAGA_HALF || force_direct())
+        return 0;
+    return conv_mfma_stats_floats(g) * sizeof(float);
+}
+
+int saga_hip_conv2d_fwd_bnstats(const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y,
+                                const SagaConvParams *p, float alpha, void *workspace, size_t ws_bytes,
+                                float *partial, size_t partial_bytes, int *partial_rows, saga_stream_t stream)
+{
+    ConvGeom g;
+    int r = geometry(x, w, y, p, &g);
+    if(r)
+        return r;
+    if(!partial || !partial_rows)
+        return SAGA_HIP_EINVAL;
+    if(force_direct())
+        return SAGA_HIP_EUNSUPPORTED;
+    return conv_mfma_fwd(x, w, y, g, alpha, 0.0f, workspace, ws_bytes, as_stream(stream), partial,
+                         partial_bytes / sizeof(float), partial_rows);
+}
+
 int saga_hip_conv2d_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx,
                              const SagaConvParams *p, float alpha, float beta, void *workspace, size_t ws_bytes,
                              saga_stream_t stream)

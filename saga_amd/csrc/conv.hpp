@@ -21,8 +21,12 @@ int conv_direct_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, co
 // problem is outside what it covers, and the dispatcher falls back to the direct kernels.
 size_t conv_mfma_workspace(int kind, const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y,
                            const ConvGeom &g);
+// stats (optional): receives per block row and output channel the sum and the sum of squares of
+// the stored outputs, [*stats_rows][K][2] floats; needs beta == 0 and conv_mfma_stats_floats(g) floats
+size_t conv_mfma_stats_floats(const ConvGeom &g);
 int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y, const ConvGeom &g,
-                  float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st);
+                  float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st, float *stats = nullptr,
+                  size_t stats_floats = 0, int *stats_rows = nullptr);
 int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx,
                        const ConvGeom &g, float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st);
 int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, const SagaTensorView *dw,

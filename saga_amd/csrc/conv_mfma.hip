@@ -51,6 +51,9 @@ struct GatherArgs {
     int OHc, OWc, Mc;  // pixel grid and row count of one class (Mc = M when classes == 1)
     int blocks_per_class;
     unsigned char cls_ids[16]; // residue classes that get blocks (classes with no tap are left out)
+    float *stats;      // forward only, optional: per block row and output channel, sum and sum of
+                       // squares of the stored outputs, [ceil(M / BM)][Ngemm][2]
+    int stats_rows;    // out: block rows the launch wrote
 };
 
 __device__ __forceinline__ int xcd_remap(int b, int nblocks)
@@ -272,6 +275,23 @@ __device__ __forceinline__ unsigned pack2(float a, float b)
     v[0] = (_Float16)a;
     v[1] = (_Float16)b;
     return __builtin_bit_cast(unsigned, v);
+}
+
+// One step of a halving exchange over n live values per lane: the lane with bit m set keeps
+// the upper half, its partner (lane ^ m) the lower half, and each adds what the other held of
+// its half.  n is a template parameter so that every array index is a constant and the
+// arrays stay in registers.
+template <int n, int NV>
+__device__ __forceinline__ void halve_exchange(float (&a)[NV], float (&b)[NV], int lane, int m)
+{
+    const bool up = lane & m;
+#pragma unroll
+    for(int k = 0; k < n / 2; k++) {
+        const float ka = up ? a[k + n / 2] : a[k], sa = up ? a[k] : a[k + n / 2];
+        const float kb = up ? b[k + n / 2] : b[k], sb = up ? b[k] : b[k + n / 2];
+        a[k] = ka + __shfl_xor(sa, m, 64);
+        b[k] = kb + __shfl_xor(sb, m, 64);
+    }
 }
 
 template <int BM, int BN, int WGM, int WGN, int STAGES, int BKT, bool BWD>
@@ -541,6 +561,64 @@ __global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArg
                         val += g.beta * (float)orow[n];
                     orow[n] = (half_t)val;
                 }
+            }
+        }
+    }
+    // Optional: per-channel sum and sum of squares of this block's outputs (as stored, i.e.
+    // rounded to fp16), for a batch normalisation that follows.  Rows past M and columns past
+    // Ngemm hold zeros in the accumulators and add nothing.  Lanes of one half-wave hold
+    // different pixels of the same channels: a halving exchange (each step swaps half of the
+    // values with the lane 16, 8, .. 1 away) leaves every lane with the total of one channel;
+    // the wavefronts stacked along M are then added through LDS in a fixed order.
+    if constexpr(!BWD) {
+        if(g.stats) {
+            constexpr int NV = TN * 16;
+            static_assert(NV == 16 || NV == 32, "stats layout");
+            float sv[NV], qv[NV];
+#pragma unroll
+            for(int j = 0; j < TN; j++)
+#pragma unroll
+                for(int v = 0; v < 16; v++) {
+                    float a = 0.0f, q = 0.0f;
+#pragma unroll
+                    for(int i = 0; i < TM; i++) {
+                        const float r = (float)(half_t)(g.alpha * acc[i][j][v]);
+                        a += r;
+                        q += r * r;
+                    }
+                    sv[j * 16 + v] = a;
+                    qv[j * 16 + v] = q;
+                }
+            if constexpr(NV == 32) {
+                halve_exchange<32>(sv, qv, lane, 16);
+                halve_exchange<16>(sv, qv, lane, 8);
+                halve_exchange<8>(sv, qv, lane, 4);
+                halve_exchange<4>(sv, qv, lane, 2);
+                halve_exchange<2>(sv, qv, lane, 1);
+            } else {
+                halve_exchange<16>(sv, qv, lane, 16);
+                halve_exchange<8>(sv, qv, lane, 8);
+                halve_exchange<4>(sv, qv, lane, 4);
+                halve_exchange<2>(sv, qv, lane, 2);
+                sv[0] += __shfl_xor(sv[0], 1, 64);
+                qv[0] += __shfl_xor(qv[0], 1, 64);
+            }
+            const int idx = NV == 32 ? (lane & 31) : (lane & 31) >> 1;
+            const int chl = 32 * (idx >> 4) + 8 * ((idx & 15) >> 2) + 4 * hi + (idx & 3); // channel inside the wave tile
+            typedef float float2_t __attribute__((ext_vector_type(2)));
+            float2_t *red = (float2_t *)smem;
+            __syncthreads(); // every wavefront is done reading the last slice
+            if(NV == 32 || (lane & 1) == 0) {
+                float2_t v2 = {sv[0], qv[0]};
+                red[(wave / WGN) * BN + wn + chl] = v2;
+            }
+            __syncthreads();
+            if(tid < BN && n0 + tid < g.Ngemm) {
+                float2_t t = red[tid];
+#pragma unroll
+                for(int wy = 1; wy < WGM; wy++)
+                    t += red[wy * BN + tid];
+                *(float2_t *)(g.stats + ((int64_t)bm * g.Ngemm + n0 + tid) * 2) = t;
             }
         }
     }
@@ -1226,6 +1304,7 @@ template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
         g.nblk_n = (g.Ngemm + BN - 1) / BN;                                                            \
         g.blocks_per_class = ((g.Mc + BM - 1) / BM) * g.nblk_n;                                        \
         g.nblocks = g.blocks_per_class * active;                                                       \
+        g.stats_rows = (g.Mc + BM - 1) / BM;                                                           \
         kern<<<g.nblocks, 64 * WGM * WGN, lds, st>>>(g);                                               \
     } while(0)
         switch(tile) {
@@ -1237,6 +1316,8 @@ template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
         SAGA_CHECK_LAUNCH();
         return 0;
     }
+    if(g.stats)
+        return SAGA_HIP_EUNSUPPORTED;
     // tile choice by output-channel count; M tiles are 128 or 256 rows
     if(g.Ngemm > 64) {
         constexpr int BM = 128, BN = 128;
@@ -1280,6 +1361,13 @@ static bool common_ok(const SagaTensorView *act_in, const SagaTensorView *w, con
 
 } // namespace
 
+// floats a forward launch may write into its statistics buffer: the smallest M tile is 128 rows
+size_t conv_mfma_stats_floats(const ConvGeom &g)
+{
+    const int64_t M = (int64_t)g.N * g.P * g.Q;
+    return (size_t)((M + 127) / 128) * g.K * 2;
+}
+
 size_t conv_mfma_workspace(int kind, const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y,
                            const ConvGeom &g)
 {
@@ -1314,8 +1402,11 @@ size_t conv_mfma_workspace(int kind, const SagaTensorView *x, const SagaTensorVi
 }
 
 int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y, const ConvGeom &g,
-                  float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st)
+                  float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st, float *stats, size_t stats_floats,
+                  int *stats_rows)
 {
+    if(stats && (beta != 0.0f || stats_floats < conv_mfma_stats_floats(g)))
+        return SAGA_HIP_EINVAL;
     CLInfo lx, ly;
     bool pad = false;
     if(!common_ok(x, w, y, g, &lx, &ly, &pad))
@@ -1344,7 +1435,11 @@ int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTe
         a.alpha = alpha; a.beta = beta;
         a.a_bytes = (unsigned)(px * 8);
         a.b_bytes = (unsigned)(wn * 2);
-        return launch_gather<false>(a, st);
+        a.stats = stats;
+        const int rc = launch_gather<false>(a, st);
+        if(stats_rows)
+            *stats_rows = a.stats_rows;
+        return rc;
     }
     GatherArgs a;
     a.a = (const half_t *)x->ptr;
@@ -1381,7 +1476,11 @@ int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTe
         a.a_bytes = ab < 0x7fffff00 ? (unsigned)ab : 0;
         a.b_bytes = bb < 0x7fffff00 ? (unsigned)bb : 0;
     }
-    return launch_gather<false>(a, st);
+    a.stats = stats;
+    const int rc = launch_gather<false>(a, st);
+    if(stats_rows)
+        *stats_rows = a.stats_rows;
+    return rc;
 }
 
 int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx,
@@ -1418,6 +1517,7 @@ int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const 
         a.a_bytes = ab < 0x7fffff00 ? (unsigned)ab : 0;
         a.b_bytes = bb < 0x7fffff00 ? (unsigned)bb : 0;
     }
+    a.stats = nullptr;
     return launch_gather<true>(a, st);
 }
 

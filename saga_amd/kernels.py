@@ -38,6 +38,9 @@ SIGNATURES = {
     "saga_hip_init": (_I, [_I, C.POINTER(C.c_int)]),
     "saga_hip_conv2d_workspace_size": (_SZ, [_I, _TV, _TV, _TV, C.POINTER(ConvParams)]),
     "saga_hip_conv2d_fwd": (_I, [_TV, _TV, _TV, C.POINTER(ConvParams), _F, _F, _VP, _SZ, _VP]),
+    "saga_hip_conv2d_fwd_bnstats_size": (_SZ, [_TV, _TV, _TV, C.POINTER(ConvParams)]),
+    "saga_hip_conv2d_fwd_bnstats": (_I, [_TV, _TV, _TV, C.POINTER(ConvParams), _F, _VP, _SZ, _VP, _SZ,
+                                         C.POINTER(C.c_int), _VP]),
     "saga_hip_conv2d_bwd_data": (_I, [_TV, _TV, _TV, C.POINTER(ConvParams), _F, _F, _VP, _SZ, _VP]),
     "saga_hip_conv2d_bwd_filter": (_I, [_TV, _TV, _TV, C.POINTER(ConvParams), _F, _F, _VP, _SZ, _VP]),
     "saga_hip_bias_add": (_I, [_TV, _TV, _VP]),
@@ -46,6 +49,8 @@ SIGNATURES = {
     "saga_hip_bn_infer": (_I, [_TV, _TV, _TV, _VP, _VP, _VP, _VP, _F, _I, _VP]),
     "saga_hip_bn_workspace_size": (_SZ, [_TV]),
     "saga_hip_bn_train_fwd": (_I, [_TV, _TV, _TV, _VP, _VP, _VP, _VP, _VP, _VP, _F, _F, _I, _VP, _SZ, _VP]),
+    "saga_hip_bn_train_fwd_partials": (_I, [_TV, _TV, _TV, _VP, _VP, _VP, _VP, _VP, _VP, _F, _F, _I, _VP, _I, _VP,
+                                            _SZ, _VP]),
     "saga_hip_bn_bwd": (_I, [_TV, _TV, _TV, _TV, _TV, _VP, _VP, _VP, _VP, _VP, _F, _F, _F, _I, _VP, _SZ, _VP]),
     "saga_hip_act_fwd": (_I, [_I, _F, _TV, _TV, _F, _VP]),
     "saga_hip_act_bwd": (_I, [_I, _F, _TV, _TV, _TV, _TV, _F, _VP]),

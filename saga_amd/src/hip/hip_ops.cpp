@@ -34,18 +34,54 @@ struct ConvDesc {
     SagaConvParams params;
 };
 
+// Per-channel partial sums of a convolution's output, handed from the ConvFwd that produces
+// them in its epilogue to the BnTrain that would otherwise read the tensor once more.
+struct ConvStatsLink {
+    std::shared_ptr<HipMemory> partial;
+    int rows = 0;
+    bool valid = false; // set by every ConvFwd::exec, consumed by the BnTrain::exec that follows
+};
+
 struct ConvFwd : public HipOperation {
     const T x_, w_, y_;
     const SagaConvParams cp_;
     float beta_ = 0;
+    std::shared_ptr<ConvStatsLink> stats_;
     ConvFwd(HipProgram &p, T x, T w, T y, SagaConvParams cp) : HipOperation("convfwd"), x_(x), w_(w), y_(y), cp_(cp)
     {
         const SagaTensorView vx = x->view(), vw = w->view(), vy = y->view();
         p.m_ctx->m_workspace.request(saga_hip_conv2d_workspace_size(SAGA_CONV_FWD, &vx, &vw, &vy, &cp_));
     }
+    // called by a batch normalisation that consumes y; nullptr if this convolution cannot supply them
+    std::shared_ptr<ConvStatsLink> offerStats()
+    {
+        if(stats_)
+            return stats_;
+        const SagaTensorView vx = x_->view(), vw = w_->view(), vy = y_->view();
+        const size_t bytes = saga_hip_conv2d_fwd_bnstats_size(&vx, &vw, &vy, &cp_);
+        if(!bytes)
+            return nullptr;
+        stats_ = std::make_shared<ConvStatsLink>();
+        stats_->partial = std::make_shared<HipMemory>(bytes);
+        return stats_;
+    }
     void exec(HipProgram &p) override
     {
         const SagaTensorView vx = x_->view(), vw = w_->view(), vy = y_->view();
+        if(stats_) {
+            stats_->valid = false;
+            if(beta_ == 0.0f) {
+                const int r = saga_hip_conv2d_fwd_bnstats(&vx, &vw, &vy, &cp_, 1.0f, p.m_ctx->m_workspace.ptr(),
+                                                          p.m_ctx->m_workspace.size(), (float *)stats_->partial->m_ptr,
+                                                          stats_->partial->m_bytes, &stats_->rows, S(p));
+                if(r == 0) {
+                    stats_->valid = true;
+                    return;
+                }
+                if(r != SAGA_HIP_EUNSUPPORTED)
+                    chkSaga(r);
+            }
+        }
         chkSaga(saga_hip_conv2d_fwd(&vx, &vw, &vy, &cp_, 1.0f, beta_, p.m_ctx->m_workspace.ptr(),
                                     p.m_ctx->m_workspace.size(), S(p)));
     }
@@ -560,6 +596,7 @@ struct BnTrain : public HipOperation {
     const int flags_;
     float expavg_ = NAN;
     float m_beta_ = 1.0f, v_beta_ = 1.0f; // running statistics are read-modify-write
+    std::shared_ptr<ConvStatsLink> stats_; // the producer of x leaves the per-channel sums here
     BnTrain(HipProgram &p, T x, T z, T s, T b, T m, T v, T y, T sm, T sv, float eps, int flags)
       : HipOperation(flags ? "bntrain.fused" : "bntrain")
       , x_(x), z_(z), s_(s), b_(b), m_(m), v_(v), y_(y), sm_(sm), sv_(sv), eps_(eps), flags_(flags)
@@ -576,6 +613,20 @@ struct BnTrain : public HipOperation {
         SagaTensorView vz;
         if(z_)
             vz = z_->view();
+        if(stats_ && stats_->valid) {
+            stats_->valid = false;
+            const int r = saga_hip_bn_train_fwd_partials(
+                &vx, z_ ? &vz : nullptr, &vy, (const float *)s_->deviceMem(), (const float *)b_->deviceMem(),
+                (float *)m_->deviceMem(), (float *)v_->deviceMem(), (float *)sm_->deviceMem(), (float *)sv_->deviceMem(),
+                eps_, expavg_, flags_, (const float *)stats_->partial->m_ptr, stats_->rows, p.m_ctx->m_workspace.ptr(),
+                p.m_ctx->m_workspace.size(), S(p));
+            if(r == 0) {
+                expavg_ = p.m_pc.bn_expavg;
+                return;
+            }
+            if(r != SAGA_HIP_EUNSUPPORTED)
+                chkSaga(r);
+        }
         chkSaga(saga_hip_bn_train_fwd(&vx, z_ ? &vz : nullptr, &vy, (const float *)s_->deviceMem(),
                                       (const float *)b_->deviceMem(), (float *)m_->deviceMem(),
                                       (float *)v_->deviceMem(), (float *)sm_->deviceMem(), (float *)sv_->deviceMem(),
@@ -591,8 +642,8 @@ struct BnTrain : public HipOperation {
         return r;
     }
     HipOpArgs listOutputs() const override { return {{"y", y_}, {"m", m_}, {"v", v_}, {"sm", sm_}, {"sv", sv_}}; }
-    // statistics pass reads x, normalise pass reads x (+z) and writes y
-    double bytes() const override { return (z_ ? 4 : 3) * nbytes(x_); }
+    // statistics pass reads x (unless the producer supplied the sums), normalise pass reads x (+z), writes y
+    double bytes() const override { return ((z_ ? 4 : 3) - (stats_ ? 1 : 0)) * nbytes(x_); }
     float *getBeta(const T &t) override
     {
         if(t == m_)
@@ -693,6 +744,19 @@ void batchnorm_lower(HipProgram &p, HipProgramUnit &pu, const Node &n, std::shar
     auto sm = std::make_shared<HipTensor>(Tensor::DataType::FLOAT, *m, m->namePostfix("smean"));
     auto sv = std::make_shared<HipTensor>(Tensor::DataType::FLOAT, *v, v->namePostfix("svar"));
     auto f = std::make_shared<BnTrain>(p, x, z, s, b, m, v, y, sm, sv, eps, flags);
+    // if the op that wrote x last is a convolution and nothing else writes x, take the sums from it
+    {
+        ConvFwd *producer = nullptr;
+        int writers = 0;
+        for(const auto &op : pu.m_fwd)
+            for(const auto &o : op->listOutputs())
+                if(o.second->m_storage == x->m_storage) {
+                    writers++;
+                    producer = o.second == x ? dynamic_cast<ConvFwd *>(op.get()) : nullptr;
+                }
+        if(writers == 1 && producer)
+            f->stats_ = producer->offerStats();
+    }
     pu.fwd(f);
 
     auto dx = p.lowerGrad(pu, xh);

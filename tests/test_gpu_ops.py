@@ -80,6 +80,67 @@ def test_conv_fwd_bwd(case, layout, padc, dtype):
     assert_close(host(dwd), 2 * dw_ref, dtype, "dw beta=1")
 
 
+BNSTATS_CASES = [
+    # N, C, H, K, R, pad, stride, relu+add
+    (2, 64, 14, 64, 3, 1, 1, False),
+    (3, 32, 9, 160, 1, 0, 1, True),
+    (2, 128, 13, 24, 3, 1, 2, True),
+    (2, 3, 30, 64, 7, 3, 2, False),
+]
+
+
+@pytest.mark.parametrize("case", BNSTATS_CASES)
+def test_conv_bnstats_then_bn_from_partials(case):
+    """Convolution that leaves the batch-norm partial sums, followed by the batch norm that starts
+    from them: same results as the separate conv and batch-norm entry points."""
+    N, Cc, H, Kk, R, pad, stride, fused = case
+    dtype = torch.float16
+    rng = np.random.default_rng(Cc * 7 + Kk)
+    x = rnd(rng, N, Cc, H, H, dtype=dtype)
+    w = rnd(rng, Kk, Cc, R, R, dtype=dtype, scale=(2.0 / (Cc * R * R)) ** 0.5)
+    y_ref = ref.round_half(ref.conv2d_fwd(x, w, pad, stride))
+    L = K.lib()
+    xd, wd = dev(x, dtype, "nhwc"), dev(w, dtype, "nhwc")
+    yd = dev(np.zeros_like(y_ref), dtype, "nhwc")
+    p = K.ConvParams(pad, stride, 1, 1)
+    vx, vw, vy = K.view(xd), K.view(wd), K.view(yd)
+    nbytes = L.saga_hip_conv2d_fwd_bnstats_size(C.byref(vx), C.byref(vw), C.byref(vy), C.byref(p))
+    assert nbytes > 0
+    partial = torch.full((nbytes // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    ws = torch.zeros(max(1, L.saga_hip_conv2d_workspace_size(K.CONV_FWD, C.byref(vx), C.byref(vw), C.byref(vy),
+                                                             C.byref(p))), dtype=torch.uint8, device="cuda")
+    rows = C.c_int(0)
+    K.check(L.saga_hip_conv2d_fwd_bnstats(C.byref(vx), C.byref(vw), C.byref(vy), C.byref(p), 1.0, K.ptr(ws), ws.numel(),
+                                          K.ptr(partial), nbytes, C.byref(rows), S()))
+    assert_close(host(yd), y_ref, dtype, "y")
+    # the partial rows add up to the sums over the stored (rounded) output
+    yh = host(yd).astype(np.float64)
+    got = host(partial)[: rows.value * Kk * 2].reshape(rows.value, Kk, 2).astype(np.float64).sum(0)
+    np.testing.assert_allclose(got[:, 0], yh.sum((0, 2, 3)), rtol=1e-4, atol=1e-3)
+    np.testing.assert_allclose(got[:, 1], (yh * yh).sum((0, 2, 3)), rtol=1e-4, atol=1e-3)
+
+    flags = (K.BN_RELU | K.BN_ADD) if fused else 0
+    z = rnd(rng, *y_ref.shape, dtype=dtype)
+    s, b = (1 + 0.2 * rng.standard_normal(Kk)).astype(np.float32), (0.1 * rng.standard_normal(Kk)).astype(np.float32)
+    m, v = np.zeros(Kk, np.float32), np.ones(Kk, np.float32)
+    zd, od = dev(z, dtype, "nhwc"), dev(np.zeros_like(y_ref), dtype, "nhwc")
+    sd, bd, md, vd = (dev(t) for t in (s, b, m, v))
+    sm, sv = dev(np.zeros(Kk, np.float32)), dev(np.zeros(Kk, np.float32))
+    ws2 = torch.zeros(2 * Kk, dtype=torch.float32, device="cuda")
+    K.check(L.saga_hip_bn_train_fwd_partials(C.byref(K.view(yd)), C.byref(K.view(zd)) if fused else None,
+                                             C.byref(K.view(od)), K.ptr(sd), K.ptr(bd), K.ptr(md), K.ptr(vd),
+                                             K.ptr(sm), K.ptr(sv), 1e-5, 0.1, flags, K.ptr(partial), rows.value,
+                                             K.ptr(ws2), ws2.numel() * 4, S()))
+    o_ref, rsm, rsv, rm, rv = ref.bn_train_fwd(host(yd), s, b, m, v, 1e-5, 0.1)
+    if fused:
+        o_ref = ref.act_fwd(o_ref + z)
+    assert_close(host(od), o_ref, dtype, "bn y")
+    assert_close(host(sm), rsm, torch.float32, "saved mean", 1e-3)
+    assert_close(host(sv), rsv, torch.float32, "saved invstd", 1e-3)
+    assert_close(host(md), rm, torch.float32, "running mean", 1e-3)
+    assert_close(host(vd), rv, torch.float32, "running var", 1e-3)
+
+
 @pytest.mark.parametrize("dtype", DT)
 def test_conv_golden(golden, dtype):
     g = golden["ops"]
