@@ -28,6 +28,14 @@ PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 matrix
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
 MATRIX_KINDS = ("convfwd", "convbwddata", "convbwdfilter", "fc.")
+CONV_KINDS = ("convfwd", "convbwddata", "convbwdfilter")
+
+# HBM bytes per launch of each operation kind, averaged over the launches of one training step:
+# rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE over this benchmark, summed over the kernels an
+# operation launches, each counter scaled by what it reads for a plain copy of known size
+# (FETCH_SIZE reads 0.5 of the bytes a 1 GiB copy fetches, WRITE_SIZE 1.0).  The command lines and
+# the per-kernel table are in profiles/resnet50_b256_fp16_hbm_counters.txt.
+MEASURED_HBM_BYTES_PER_LAUNCH = {}
 
 
 def profile_rows(rows):
@@ -125,31 +133,46 @@ def main():
     train.finalize()
     infer.finalize()
 
-    # ---- training: W warm-up steps, then exactly K timed steps (each step ends in a stream sync)
+    import torch  # device-wide synchronisation around the timed regions
+
+    # ---- training: W warm-up steps, then exactly K timed steps
     train.run(args.warmup)
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
     train.run(args.steps)
+    torch.cuda.synchronize()
     t_train = time.perf_counter() - t0
     mean_loss = float(loss.read().mean())
 
     # ---- inference on the same weights
     infer.run(args.warmup)
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
     infer.run(args.steps)
+    torch.cuda.synchronize()
     t_infer = time.perf_counter() - t0
     pred.read()
 
-    kernels, roof = [], None
+    kernels, roof, conv = [], None, None
     if not args.no_profile:
         train.set_profiling(True)
         train.run(args.steps)
-        kernels = profile_rows(train.profile())
+        rows = train.profile()
+        kernels = profile_rows(rows)
         train.set_profiling(False)
         if kernels:
             d = kernels[0]
             roof = {"kernel": d["kind"], "bound": d["bound"], "achieved": d["achieved"], "peak": d["peak"],
-                    "unit": d["unit"], "frac": d["frac"], "traffic": None,
+                    "unit": d["unit"], "frac": d["frac"],
+                    "traffic": MEASURED_HBM_BYTES_PER_LAUNCH.get(d["kind"]),
                     "avg_launch_us": d["avg_us"], "launches": d["launches"]}
+        # the three convolution kinds together: the "conv MFMA util %" half of the metric
+        cr = [r for r in rows if r["kind"] in CONV_KINDS and r["ms"] > 0]
+        if cr:
+            tf = sum(r["flops"] for r in cr) / (sum(r["ms"] for r in cr) * 1e-3) / 1e12
+            conv = {"bound": "mfma", "achieved": round(tf, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(tf / PEAK_FP16_TFLOPS, 4), "mfma_util_pct": round(100 * tf / PEAK_FP16_TFLOPS, 2),
+                    "ms_per_step": round(sum(r["ms"] for r in cr) / args.steps, 3)}
 
     flops_step = 3 * net.flops_fwd * args.batch  # fwd + bwd-data + bwd-filter (the stem has no bwd-data)
     ips = args.batch * args.steps / t_train
@@ -176,6 +199,7 @@ def main():
         "loss_scale": train.loss_scale(),
         "mean_loss": round(mean_loss, 4),
         "roofline": roof,
+        "conv": conv,
         "kernels": kernels,
     }
     if not args.no_cpu:

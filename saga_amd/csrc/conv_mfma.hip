@@ -876,9 +876,13 @@ __global__ void __launch_bounds__(256) conv_bwd_filter_dma(FilterArgs g, unsigne
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    int b = blockIdx.x;
-    const int split = b % g.splits;
-    b /= g.splits;
+    // tiles are the fast index and every XCD gets a contiguous run of block ids, so the
+    // blocks that read the same pixel range of x and dy (one split, all tiles) run on one
+    // XCD at about the same time and share the range through its L2
+    int b = xcd_remap(blockIdx.x, gridDim.x);
+    const int ntiles = g.tiles_k * g.tiles_c;
+    const int split = b / ntiles;
+    b -= split * ntiles;
     const int tc = b % g.tiles_c, tk = b / g.tiles_c;
     const int k0 = tk * BM, j0 = tc * BN;
     const int m_begin = split * g.m_per_split;
