@@ -858,19 +858,19 @@ __device__ __forceinline__ half8_t tr_read8(const char *lo, const char *hi)
     return __builtin_bit_cast(half8_t, v);
 }
 
-template <int BM, int BN, int STAGES>
-__global__ void __launch_bounds__(256) conv_bwd_filter_dma(FilterArgs g, unsigned x_bytes, unsigned dy_bytes)
+template <int BM, int BN, int STAGES, int NW>
+__global__ void __launch_bounds__(64 * NW) conv_bwd_filter_dma(FilterArgs g, unsigned x_bytes, unsigned dy_bytes)
 {
     constexpr int GA = BM / 8, GB = BN / 8;             // 16-byte granules per LDS row
     constexpr int RPA = 64 / GA, RPB = 64 / GB;         // pixel rows one wave instruction fills
-    constexpr int RA = BK / (4 * RPA), RB = BK / (4 * RPB);
+    constexpr int RA = BK / (NW * RPA), RB = BK / (NW * RPB);
     constexpr int ROWA = BM * 2, ROWB = BN * 2;
     constexpr int STAGE_BYTES = BK * (ROWA + ROWB);
-    constexpr int WGM = BM >= 128 ? 2 : 1, WGN = 4 / WGM;
+    constexpr int WGM = BM >= 128 ? 2 : 1, WGN = NW / WGM;
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
     constexpr unsigned OOB = 0x7fffff00u;
-    static_assert(RA >= 1 && RB >= 1 && (GA == 8 || GA == 16) && (GB == 8 || GB == 16), "tile");
+    static_assert(RA >= 1 && RB >= 1 && (GA == 8 || GA == 16 || GA == 32) && (GB == 8 || GB == 16), "tile");
 
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
@@ -895,7 +895,7 @@ __global__ void __launch_bounds__(256) conv_bwd_filter_dma(FilterArgs g, unsigne
 
     // A (dy): this lane fills physical granule lane % GA of pixel row pa0 (+ 4*RPA per round)
     const int pa0 = wave * RPA + lane / GA;
-    const int swa = GA == 16 ? (pa0 & 3) << 2 : ((pa0 >> 1) & 1) << 2;
+    const int swa = GA >= 16 ? (pa0 & 3) << 2 : ((pa0 >> 1) & 1) << 2;
     const int ka = k0 + (((lane % GA) ^ swa) << 3);
     const bool ka_ok = ka < g.K;
     // B (x): likewise; the logical granule fixes this lane's (tap, c)
@@ -911,7 +911,7 @@ __global__ void __launch_bounds__(256) conv_bwd_filter_dma(FilterArgs g, unsigne
     int bn_[RB], by_[RB], bx_[RB];
 #pragma unroll
     for(int j = 0; j < RB; j++) {
-        const int m = m_begin + pb0 + j * 4 * RPB;
+        const int m = m_begin + pb0 + j * NW * RPB;
         const int mm = m < g.M ? m : 0;
         bx_[j] = mm % g.Q;
         const int t = mm / g.Q;
@@ -925,17 +925,17 @@ __global__ void __launch_bounds__(256) conv_bwd_filter_dma(FilterArgs g, unsigne
         char *sb = sa + BK * ROWA;
 #pragma unroll
         for(int j = 0; j < RA; j++) {
-            const int m = ms + pa0 + j * 4 * RPA;
+            const int m = ms + pa0 + j * NW * RPA;
             const unsigned off = (ka_ok && m < m_end) ? (unsigned)((m * g.ldy + ka) * 2) : OOB;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(ry, (lds_ptr_t)(sa + (wave + 4 * j) * 1024), 16, off, 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ry, (lds_ptr_t)(sa + (wave + NW * j) * 1024), 16, off, 0, 0, 0);
         }
 #pragma unroll
         for(int j = 0; j < RB; j++) {
-            const int m = ms + pb0 + j * 4 * RPB;
+            const int m = ms + pb0 + j * NW * RPB;
             const int iy = by_[j] * g.stride + offy, ix = bx_[j] * g.stride + offx;
             const bool ok = cb_ok && m < m_end && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
             const unsigned off = ok ? (unsigned)((((bn_[j] * g.H + iy) * g.W + ix) * g.ldx + cc) * 2) : OOB;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(sb + (wave + 4 * j) * 1024), 16, off, 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(sb + (wave + NW * j) * 1024), 16, off, 0, 0, 0);
             bx_[j] += BK;
             while(bx_[j] >= g.Q) {
                 bx_[j] -= g.Q;
@@ -963,7 +963,7 @@ __global__ void __launch_bounds__(256) conv_bwd_filter_dma(FilterArgs g, unsigne
     // MFMA step) and channels fc .. fc+3 of a 32-channel tile
     const int fp = 8 * (lane >> 5) + ((lane & 15) >> 2);
     const int fc = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-    const int fswa = GA == 16 ? (fp & 3) << 2 : ((fp >> 1) & 1) << 2;
+    const int fswa = GA >= 16 ? (fp & 3) << 2 : ((fp >> 1) & 1) << 2;
     const int fswb = GB == 16 ? (fp & 3) << 2 : ((fp >> 1) & 1) << 2;
     int foa[TM], fob[TN];
 #pragma unroll
@@ -1104,12 +1104,13 @@ static FilterPlan plan_filter(const ConvGeom &g)
     FilterPlan p;
     const int RSC = g.R * g.S * g.C;
     const int64_t M = (int64_t)g.N * g.P * g.Q;
-    p.bm = g.K > 64 ? 128 : 64;
+    p.bm = g.K > 64 ? 128 : 64; // 256x128 tiles were measured slower on every ResNet-50 layer
     p.bn = 128;
     p.tiles_k = (g.K + p.bm - 1) / p.bm;
     p.tiles_c = (RSC + p.bn - 1) / p.bn;
     const int tiles = p.tiles_k * p.tiles_c;
-    int64_t want = (1024 + tiles - 1) / tiles;
+    // three blocks fit a CU: 768 blocks are one full round of the chip (measured best of 512..2048)
+    int64_t want = (768 + tiles - 1) / tiles;
     const int64_t maxs = (M + 255) / 256; // at least 256 pixels per split
     if(want > maxs)
         want = maxs;
@@ -1564,11 +1565,11 @@ int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, cons
         a.tiles_k = p.tiles_k; a.tiles_c = p.tiles_c;
         a.splits = p.splits; a.m_per_split = p.m_per_split;
         const int blocks = p.tiles_k * p.tiles_c * p.splits;
-        constexpr int ST = 3;
+        constexpr int ST = 3, FNW = 8;
         if(p.bm == 128)
-            conv_bwd_filter_dma<128, 128, ST><<<blocks, 256, ST * BK * 512, st>>>(a, (unsigned)(px * 8), (unsigned)yb);
+            conv_bwd_filter_dma<128, 128, ST, FNW><<<blocks, 64 * FNW, ST * BK * 512, st>>>(a, (unsigned)(px * 8), (unsigned)yb);
         else
-            conv_bwd_filter_dma<64, 128, ST><<<blocks, 256, ST * BK * 384, st>>>(a, (unsigned)(px * 8), (unsigned)yb);
+            conv_bwd_filter_dma<64, 128, ST, 4><<<blocks, 256, ST * BK * 384, st>>>(a, (unsigned)(px * 8), (unsigned)yb);
         SAGA_CHECK_LAUNCH();
         thin_filter_reduce<<<grid_for(n, 256, 256 * 8), 256, 0, st>>>(a.partial, (half_t *)dw->ptr, n, g.C, g.S, p.splits,
                                                                     alpha, beta);
@@ -1605,11 +1606,11 @@ int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, cons
     const int blocks = p.tiles_k * p.tiles_c * p.splits;
     const int64_t xb = ((lx.rows - 1) * (int64_t)a.ldx + Cp) * 2, yb = ((ldy.rows - 1) * ldy.pitch + ldy.C) * 2;
     if(dma_stages() >= 2 && xb < 0x7fffff00 && yb < 0x7fffff00) {
-        constexpr int ST = 3;
+        constexpr int ST = 3, FNW = 8;
         if(p.bm == 128)
-            conv_bwd_filter_dma<128, 128, ST><<<blocks, 256, ST * BK * 512, st>>>(a, (unsigned)xb, (unsigned)yb);
+            conv_bwd_filter_dma<128, 128, ST, FNW><<<blocks, 64 * FNW, ST * BK * 512, st>>>(a, (unsigned)xb, (unsigned)yb);
         else
-            conv_bwd_filter_dma<64, 128, ST><<<blocks, 256, ST * BK * 384, st>>>(a, (unsigned)xb, (unsigned)yb);
+            conv_bwd_filter_dma<64, 128, ST, 4><<<blocks, 256, ST * BK * 384, st>>>(a, (unsigned)xb, (unsigned)yb);
     } else if(p.bm == 128) {
         conv_bwd_filter_mfma<128, 128><<<blocks, 256, 0, st>>>(a);
     } else {
