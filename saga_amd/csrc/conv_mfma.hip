@@ -50,6 +50,7 @@ struct GatherArgs {
     int classes;       // backward data: stride*stride residue classes of output pixels (1: none)
     int OHc, OWc, Mc;  // pixel grid and row count of one class (Mc = M when classes == 1)
     int blocks_per_class;
+    int nactive;       // classes that get blocks
     unsigned char cls_ids[16]; // residue classes that get blocks (classes with no tap are left out)
     float *stats;      // forward only, optional: per block row and output channel, sum and sum of
                        // squares of the stored outputs, [ceil(M / BM)][Ngemm][2]
@@ -321,8 +322,10 @@ __global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArg
     int py = 0, px = 0, r0 = 0, s0 = 0, nr = g.R, ns = g.S, rstep = 1;
     int PH = g.OH, PW = g.OW; // pixel grid this block's rows are numbered over
     if(BWD && g.classes > 1) {
-        const int ci = bid / g.blocks_per_class;
-        bid -= ci * g.blocks_per_class;
+        // the classes of one tile position are neighbours in block order: they read the same
+        // rows of dy and write interleaved pixels of the same rows of dx, which L2 then shares
+        const int ci = bid % g.nactive;
+        bid /= g.nactive;
         const int cls = g.cls_ids[ci];
         py = cls >> g.sshift;
         px = cls & (g.stride - 1);
@@ -1309,6 +1312,7 @@ template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
         g.nblk_n = (g.Ngemm + BN - 1) / BN;                                                            \
         g.blocks_per_class = ((g.Mc + BM - 1) / BM) * g.nblk_n;                                        \
         g.nblocks = g.blocks_per_class * active;                                                       \
+        g.nactive = active;                                                                            \
         g.stats_rows = (g.Mc + BM - 1) / BM;                                                           \
         kern<<<g.nblocks, 64 * WGM * WGN, lds, st>>>(g);                                               \
     } while(0)
