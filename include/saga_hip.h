@@ -156,6 +156,16 @@ int saga_hip_bn_bwd(const SagaTensorView *x, const SagaTensorView *y, const Saga
                     const float *save_invstd, float *ds, float *db, float beta_dx, float beta_dz, float beta_p,
                     int flags, void *workspace, size_t ws_bytes, saga_stream_t stream);
 
+/* bwd with the bias b at hand, as cudnnBatchNormalizationBackwardEx receives it
+ * (src/cuda/cuda_dnn.cpp:2138-2163): for SAGA_BN_RELU without SAGA_BN_ADD on channels-last tensors
+ * the relu mask is recomputed from x (the forward's own expression, rounded as it was stored)
+ * and y may be NULL - one tensor less to read in each of the two passes.  b NULL: as saga_hip_bn_bwd. */
+int saga_hip_bn_bwd_ex(const SagaTensorView *x, const SagaTensorView *y, const SagaTensorView *dy,
+                       const SagaTensorView *dx, const SagaTensorView *dz, const float *s, const float *b,
+                       const float *save_mean, const float *save_invstd, float *ds, float *db, float beta_dx,
+                       float beta_dz, float beta_p, int flags, void *workspace, size_t ws_bytes,
+                       saga_stream_t stream);
+
 /* ---- activations: cudnnActivationForward / Backward (src/cuda/cuda_dnn.cpp:631-638, :668-676),
  *      leaky relu kernel (src/cuda/cuda_kernels.cu:478-495).  y = act(x) + beta*y ; dx = dy*act'(x) + beta*dx. */
 int saga_hip_act_fwd(int mode, float alpha, const SagaTensorView *x, const SagaTensorView *y, float beta,

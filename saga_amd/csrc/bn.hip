@@ -12,6 +12,8 @@
 // the cancellation in E[x^2] - E[x]^2 when |mean| >> stddev.
 #include "common.hpp"
 
+#include <stdlib.h>
+
 namespace {
 
 template <typename T, int VN> struct VecT;
@@ -120,7 +122,7 @@ __global__ void __launch_bounds__(256)
         float o[VN];
 #pragma unroll
         for(int j = 0; j < VN; j++) {
-            float t = L::at(xr, j) * sc[j] + sh[j];
+            float t = __builtin_fmaf(L::at(xr, j), sc[j], sh[j]);
             if(add)
                 t += L::at(zr, j);
             if(relu)
@@ -285,28 +287,34 @@ __global__ void __launch_bounds__(256)
     }
     const float sc = sv * inv;
     ss[c] = sc;
-    ss[C + c] = bv - (float)mean * sc;
+    ss[C + c] = __builtin_fmaf(-(float)mean, sc, bv); // same expression as the backward mask recompute
 }
 
 // Pass 1 of backward: partial sums of dy' and dy'*(x-mean); dy' = dy masked by y>0 when fused relu.
-template <typename T, int VN>
+template <typename T, int VN, bool RC>
 __global__ void __launch_bounds__(256)
     bn_bwd_stats_cl(const T *__restrict__ x, int64_t px, const T *__restrict__ y, int64_t py, const T *__restrict__ dy,
                     int64_t pdy, const float *__restrict__ save_mean, float *__restrict__ partial, int64_t rows, int C,
-                    int cvb, int flags)
+                    int cvb, int flags, const float *__restrict__ rs, const float *__restrict__ rb_, const float *__restrict__ rinv)
 {
+    // rs/rb_/rinv (scale, bias, saved 1/std) set: the relu mask is recomputed from x as
+    // half(fma(x, sc, sh)) > 0, exactly what the forward stored, and y is not read
     __shared__ float red[256 * VN * 2];
     const int tx = threadIdx.x % cvb, ty = threadIdx.x / cvb, rb = 256 / cvb;
     const int c0 = (blockIdx.y * cvb + tx) * VN;
     const bool relu = flags & SAGA_BN_RELU;
-    float a0[VN], a1[VN], mean[VN];
+    constexpr bool recompute = RC;
+    float a0[VN], a1[VN], mean[VN], sc[VN], sh[VN];
 #pragma unroll
     for(int j = 0; j < VN; j++)
         a0[j] = a1[j] = 0.0f;
     if(c0 < C) {
 #pragma unroll
-        for(int j = 0; j < VN; j++)
+        for(int j = 0; j < VN; j++) {
             mean[j] = save_mean[c0 + j];
+            sc[j] = recompute ? rs[c0 + j] * rinv[c0 + j] : 0.0f;
+            sh[j] = recompute ? __builtin_fmaf(-mean[j], sc[j], rb_[c0 + j]) : 0.0f;
+        }
         typedef Ld<T, VN> L;
         typedef typename L::V V;
         const int64_t stride = (int64_t)gridDim.x * rb;
@@ -314,7 +322,8 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
             for(int j = 0; j < VN; j++) {
                 float g = L::at(gr, j);
-                if(relu && !(L::at(yr, j) > 0.0f))
+                const float yv = recompute ? (float)(T)__builtin_fmaf(L::at(xr, j), sc[j], sh[j]) : L::at(yr, j);
+                if(relu && !(yv > 0.0f))
                     g = 0.0f;
                 a0[j] += g;
                 a1[j] += g * (L::at(xr, j) - mean[j]);
@@ -327,7 +336,7 @@ __global__ void __launch_bounds__(256)
             for(int u = 0; u < 4; u++) {
                 xr[u] = L::raw(x + (r + u * stride) * px + c0);
                 gr[u] = L::raw(dy + (r + u * stride) * pdy + c0);
-                yr[u] = relu ? L::raw(y + (r + u * stride) * py + c0) : gr[u];
+                yr[u] = relu && !recompute ? L::raw(y + (r + u * stride) * py + c0) : gr[u];
             }
 #pragma unroll
             for(int u = 0; u < 4; u++)
@@ -335,7 +344,7 @@ __global__ void __launch_bounds__(256)
         }
         for(; r < rows; r += stride) {
             const V xr = L::raw(x + r * px + c0), gr = L::raw(dy + r * pdy + c0);
-            add(xr, gr, relu ? L::raw(y + r * py + c0) : gr);
+            add(xr, gr, relu && !recompute ? L::raw(y + r * py + c0) : gr);
         }
     }
 #pragma unroll
@@ -388,25 +397,27 @@ __global__ void __launch_bounds__(256)
 }
 
 // Pass 2 of backward: dx = s*invstd*(dy' - db/M - (x-mean)*invstd*ds/M) ; dz = dy'.
-template <typename T, int VN>
+template <typename T, int VN, bool RC>
 __global__ void __launch_bounds__(256)
     bn_bwd_apply_cl(const T *__restrict__ x, int64_t px, const T *__restrict__ y, int64_t py, const T *__restrict__ dy,
                     int64_t pdy, T *__restrict__ dx, int64_t pdx, T *__restrict__ dz, int64_t pdz,
                     const float *__restrict__ save_mean, const float *__restrict__ coef, int64_t rows, int C, int cvb,
-                    int flags, float beta_dx, float beta_dz)
+                    int flags, float beta_dx, float beta_dz, const float *__restrict__ rb_)
 {
     const int tx = threadIdx.x % cvb, ty = threadIdx.x / cvb, rb = 256 / cvb;
     const int c0 = (blockIdx.y * cvb + tx) * VN;
     if(c0 >= C)
         return;
     const bool relu = flags & SAGA_BN_RELU;
-    float mean[VN], a[VN], k0[VN], k1[VN];
+    constexpr bool recompute = RC;
+    float mean[VN], a[VN], k0[VN], k1[VN], sh[VN];
 #pragma unroll
     for(int j = 0; j < VN; j++) {
         mean[j] = save_mean[c0 + j];
-        a[j] = coef[c0 + j];
+        a[j] = coef[c0 + j]; // s * invstd: also the forward's scale
         k0[j] = coef[C + c0 + j];
         k1[j] = coef[2 * C + c0 + j];
+        sh[j] = recompute ? __builtin_fmaf(-mean[j], a[j], rb_[c0 + j]) : 0.0f;
     }
     typedef Ld<T, VN> L;
     typedef typename L::V V;
@@ -418,7 +429,8 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
         for(int j = 0; j < VN; j++) {
             gv[j] = L::at(gr, j);
-            if(relu && !(L::at(yr, j) > 0.0f))
+            const float yv = recompute ? (float)(T)__builtin_fmaf(L::at(xr, j), a[j], sh[j]) : L::at(yr, j);
+            if(relu && !(yv > 0.0f))
                 gv[j] = 0.0f;
         }
         if(beta_dx != 0.0f)
@@ -447,7 +459,7 @@ __global__ void __launch_bounds__(256)
             const int64_t q = row(r + u * stride);
             xr[u] = L::raw(x + q * px + c0);
             gr[u] = L::raw(dy + q * pdy + c0);
-            yr[u] = relu ? L::raw(y + q * py + c0) : gr[u];
+            yr[u] = relu && !recompute ? L::raw(y + q * py + c0) : gr[u];
         }
 #pragma unroll
         for(int u = 0; u < 4; u++)
@@ -456,7 +468,7 @@ __global__ void __launch_bounds__(256)
     for(; r < rows; r += stride) {
         const int64_t q = row(r);
         const V xr = L::raw(x + q * px + c0), gr = L::raw(dy + q * pdy + c0);
-        finish(xr, gr, relu ? L::raw(y + q * py + c0) : gr, q);
+        finish(xr, gr, relu && !recompute ? L::raw(y + q * py + c0) : gr, q);
     }
 }
 
@@ -617,6 +629,16 @@ static int vec_width(int dtype, int C, std::initializer_list<const SagaTensorVie
         if(p % vn)
             return 1;
     return vn;
+}
+
+static bool force_y_mask()
+{
+    static int v = -1;
+    if(v < 0) {
+        const char *e = getenv("SAGA_HIP_BN_MASK_FROM_Y");
+        v = (e && *e && *e != '0') ? 1 : 0;
+    }
+    return v == 1;
 }
 
 static size_t ws_floats(int64_t rows, int C, int dtype)
@@ -808,11 +830,29 @@ int saga_hip_bn_bwd(const SagaTensorView *x, const SagaTensorView *y, const Saga
                     const float *save_invstd, float *ds, float *db, float beta_dx, float beta_dz, float beta_p,
                     int flags, void *workspace, size_t ws_bytes, saga_stream_t stream)
 {
+    return saga_hip_bn_bwd_ex(x, y, dy, dx, dz, s, nullptr, save_mean, save_invstd, ds, db, beta_dx, beta_dz, beta_p,
+                              flags, workspace, ws_bytes, stream);
+}
+
+int saga_hip_bn_bwd_ex(const SagaTensorView *x, const SagaTensorView *y, const SagaTensorView *dy,
+                       const SagaTensorView *dx, const SagaTensorView *dz, const float *s, const float *b,
+                       const float *save_mean, const float *save_invstd, float *ds, float *db, float beta_dx,
+                       float beta_dz, float beta_p, int flags, void *workspace, size_t ws_bytes,
+                       saga_stream_t stream)
+{
     if(!valid_view(x) || !valid_view(dy) || !valid_view(dx) || !s || !save_mean || !save_invstd || !ds || !db)
         return SAGA_HIP_EINVAL;
-    const bool relu = flags & SAGA_BN_RELU;
-    if(relu && !valid_view(y))
+    bool relu = flags & SAGA_BN_RELU;
+    // with the bias at hand and no residual, the relu mask is a function of x: y is not needed
+    CLInfo cl_probe;
+    const bool recompute = relu && b && !(flags & SAGA_BN_ADD) && !force_y_mask() && as_channels_last(x, &cl_probe) &&
+                           as_channels_last(dy, &cl_probe) && as_channels_last(dx, &cl_probe);
+    if(relu && !recompute && !valid_view(y))
         return SAGA_HIP_EINVAL;
+    if(recompute)
+        y = nullptr;
+    const bool need_y = relu && !recompute;
+    relu = need_y; // below, "relu" guards every use of y
     if(dz && !valid_view(dz))
         return SAGA_HIP_EINVAL;
     if(!same_dims(x, dy) || !same_dims(x, dx) || (relu && !same_dims(x, y)) || (dz && !same_dims(x, dz)))
@@ -837,15 +877,24 @@ int saga_hip_bn_bwd(const SagaTensorView *x, const SagaTensorView *y, const Saga
         float *partial = ws, *coef = ws + (size_t)sh.gx * C * 2;
 #define GO(T, VN)                                                                                                    \
     do {                                                                                                             \
-        bn_bwd_stats_cl<T, VN><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, relu ? (const T *)y->ptr : nullptr,  \
+        if(recompute)                                                                                                \
+            GO2(T, VN, true);                                                                                        \
+        else                                                                                                         \
+            GO2(T, VN, false);                                                                                       \
+    } while(0)
+#define GO2(T, VN, RC)                                                                                               \
+    do {                                                                                                             \
+        bn_bwd_stats_cl<T, VN, RC><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, relu ? (const T *)y->ptr : nullptr,  \
                                                      ly.pitch, (const T *)dy->ptr, ldy.pitch, save_mean, partial,    \
-                                                     lx.rows, C, sh.cvb, flags);                                     \
+                                                     lx.rows, C, sh.cvb, flags, recompute ? s : nullptr,             \
+                                                     recompute ? b : nullptr, recompute ? save_invstd : nullptr);    \
         bn_bwd_finalize<<<(C + 3) / 4, 256, 0, st>>>(partial, sh.gx, s, save_invstd, ds, db, coef,                \
                                                          (double)lx.rows, C, beta_p);                                \
-        bn_bwd_apply_cl<T, VN><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, relu ? (const T *)y->ptr : nullptr,  \
+        bn_bwd_apply_cl<T, VN, RC><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, relu ? (const T *)y->ptr : nullptr,  \
                                                      ly.pitch, (const T *)dy->ptr, ldy.pitch, (T *)dx->ptr,          \
                                                      ldx.pitch, dz ? (T *)dz->ptr : nullptr, ldz.pitch, save_mean,   \
-                                                     coef, lx.rows, C, sh.cvb, flags, beta_dx, beta_dz);             \
+                                                     coef, lx.rows, C, sh.cvb, flags, beta_dx, beta_dz,              \
+                                                     recompute ? b : nullptr);                                       \
     } while(0)
         if(dt == SAGA_HALF) {
             if(vn == 8) GO(half_t, 8); else GO(half_t, 1);
@@ -853,7 +902,8 @@ int saga_hip_bn_bwd(const SagaTensorView *x, const SagaTensorView *y, const Saga
             if(vn == 4) GO(float, 4); else GO(float, 1);
         }
 #undef GO
-    } else if(as_channels_first(x, &fx) && as_channels_first(dy, &fdy) && as_channels_first(dx, &fdx) &&
+#undef GO2
+    } else if(!recompute && as_channels_first(x, &fx) && as_channels_first(dy, &fdy) && as_channels_first(dx, &fdx) &&
               (!relu || as_channels_first(y, &fy)) && (!dz || as_channels_first(dz, &fdz))) {
 #define GO(T)                                                                                                         \
     bn_bwd_cf<T><<<fx.C, 256, 0, st>>>((const T *)x->ptr, fx.npitch, relu ? (const T *)y->ptr : nullptr, fy.npitch,     \

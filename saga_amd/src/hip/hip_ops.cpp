@@ -672,8 +672,10 @@ struct BnBwd : public HipOperation {
         SagaTensorView vdz;
         if(dz_)
             vdz = dz_->view();
-        chkSaga(saga_hip_bn_bwd(&vx, relu ? &vy : nullptr, &vdy, &vdx, dz_ ? &vdz : nullptr,
-                                (const float *)fwd_->s_->deviceMem(), (const float *)fwd_->sm_->deviceMem(),
+        // the bias lets the kernels rebuild the relu mask from x when there is no residual
+        chkSaga(saga_hip_bn_bwd_ex(&vx, relu ? &vy : nullptr, &vdy, &vdx, dz_ ? &vdz : nullptr,
+                                (const float *)fwd_->s_->deviceMem(), (const float *)fwd_->b_->deviceMem(),
+                                (const float *)fwd_->sm_->deviceMem(),
                                 (const float *)fwd_->sv_->deviceMem(), (float *)ds_->deviceMem(),
                                 (float *)db_->deviceMem(), dx_beta_, dz_beta_, ds_beta_, flags_,
                                 p.m_ctx->m_workspace.ptr(), p.m_ctx->m_workspace.size(), S(p)));
@@ -704,7 +706,8 @@ struct BnBwd : public HipOperation {
     double bytes() const override
     {
         const double e = nbytes(dx_);
-        return e * (4 + ((flags_ & SAGA_BN_RELU) ? 2 : 0) + 1 + (dz_ ? 1 : 0) + (dx_beta_ != 0 ? 1 : 0) +
+        const bool reads_y = (flags_ & SAGA_BN_RELU) && (flags_ & SAGA_BN_ADD);
+        return e * (4 + (reads_y ? 2 : 0) + 1 + (dz_ ? 1 : 0) + (dx_beta_ != 0 ? 1 : 0) +
                     (dz_ && dz_beta_ != 0 ? 1 : 0));
     }
     float *getBeta(const T &t) override

@@ -281,6 +281,20 @@ def test_batchnorm(shape, flags, layout, padc, dtype):
     assert_close(host(dbd), db_ref, torch.float32, "bn db", 1e-4 if dtype == torch.float32 else 5e-3)
     if flags & K.BN_ADD:
         assert_close(host(dzd), dyp, dtype, "bn dz")
+    if flags & K.BN_RELU and not flags & K.BN_ADD:
+        # with the bias, the mask comes from x (y = NULL): same gradients.  The mask is rebuilt from
+        # the statistics passed in, so the forward's own statistics and output are used here.
+        y_own = host(yd)
+        dyp2 = dy * (y_own > 0)
+        dx2_ref, ds2_ref, db2_ref = ref.bn_bwd(x, dyp2, s, host(sm), host(sv))
+        dx2 = dev(np.zeros(shape, np.float32), dtype, layout, padc)
+        y_arg = None if layout.startswith("nhwc") else C.byref(K.view(yd))  # only channels-last can do without y
+        K.check(L.saga_hip_bn_bwd_ex(C.byref(K.view(xd)), y_arg, C.byref(K.view(dyd)), C.byref(K.view(dx2)), None,
+                                     K.ptr(sd), K.ptr(bd), K.ptr(sm), K.ptr(sv), K.ptr(dsd), K.ptr(dbd), 0.0, 0.0,
+                                     0.0, flags, K.ptr(ws), ws.numel(), S()))
+        assert_close(host(dx2), dx2_ref, dtype, "bn dx (mask from x)")
+        assert_close(host(dsd), ds2_ref, torch.float32, "bn ds (mask from x)", 1e-4 if dtype == torch.float32 else 5e-3)
+        assert_close(host(dbd), db2_ref, torch.float32, "bn db (mask from x)", 1e-4 if dtype == torch.float32 else 5e-3)
 
 
 def test_batchnorm_golden(golden):
