@@ -295,8 +295,11 @@ template <typename T, int VN, bool RC>
 __global__ void __launch_bounds__(256)
     bn_bwd_stats_cl(const T *__restrict__ x, int64_t px, const T *__restrict__ y, int64_t py, const T *__restrict__ dy,
                     int64_t pdy, const float *__restrict__ save_mean, float *__restrict__ partial, int64_t rows, int C,
-                    int cvb, int flags, const float *__restrict__ rs, const float *__restrict__ rb_, const float *__restrict__ rinv)
+                    int cvb, int flags, const float *__restrict__ rs, const float *__restrict__ rb_, const float *__restrict__ rinv,
+                    T *__restrict__ dz, int64_t pdz)
 {
+    // dz set: the masked gradient dy' is stored there on the way (it is the residual branch's
+    // gradient anyway), and the second pass reads it instead of y and dy
     // rs/rb_/rinv (scale, bias, saved 1/std) set: the relu mask is recomputed from x as
     // half(fma(x, sc, sh)) > 0, exactly what the forward stored, and y is not read
     __shared__ float red[256 * VN * 2];
@@ -318,7 +321,8 @@ __global__ void __launch_bounds__(256)
         typedef Ld<T, VN> L;
         typedef typename L::V V;
         const int64_t stride = (int64_t)gridDim.x * rb;
-        auto add = [&](const V &xr, const V &gr, const V &yr) {
+        auto add = [&](const V &xr, const V &gr, const V &yr, int64_t r) {
+            float gm[VN];
 #pragma unroll
             for(int j = 0; j < VN; j++) {
                 float g = L::at(gr, j);
@@ -327,7 +331,10 @@ __global__ void __launch_bounds__(256)
                     g = 0.0f;
                 a0[j] += g;
                 a1[j] += g * (L::at(xr, j) - mean[j]);
+                gm[j] = g;
             }
+            if(dz)
+                L::store(dz + r * pdz + c0, gm);
         };
         int64_t r = (int64_t)blockIdx.x * rb + ty;
         for(; r + 3 * stride < rows; r += 4 * stride) {
@@ -340,11 +347,11 @@ __global__ void __launch_bounds__(256)
             }
 #pragma unroll
             for(int u = 0; u < 4; u++)
-                add(xr[u], gr[u], yr[u]);
+                add(xr[u], gr[u], yr[u], r + u * stride);
         }
         for(; r < rows; r += stride) {
             const V xr = L::raw(x + r * px + c0), gr = L::raw(dy + r * pdy + c0);
-            add(xr, gr, relu && !recompute ? L::raw(y + r * py + c0) : gr);
+            add(xr, gr, relu && !recompute ? L::raw(y + r * py + c0) : gr, r);
         }
     }
 #pragma unroll
@@ -875,6 +882,9 @@ int saga_hip_bn_bwd_ex(const SagaTensorView *x, const SagaTensorView *y, const S
         Shape sh = plan(lx.rows, C / vn);
         dim3 grid(sh.gx, sh.gy);
         float *partial = ws, *coef = ws + (size_t)sh.gx * C * 2;
+        // residual layers: the first pass leaves dy' in dz, the second reads it in place of y and dy
+        const bool early_dz = dz && beta_dz == 0.0f && relu && !recompute && dz->ptr != dy->ptr && dz->ptr != x->ptr &&
+                              dz->ptr != y->ptr;
 #define GO(T, VN)                                                                                                    \
     do {                                                                                                             \
         if(recompute)                                                                                                \
@@ -887,14 +897,21 @@ int saga_hip_bn_bwd_ex(const SagaTensorView *x, const SagaTensorView *y, const S
         bn_bwd_stats_cl<T, VN, RC><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, relu ? (const T *)y->ptr : nullptr,  \
                                                      ly.pitch, (const T *)dy->ptr, ldy.pitch, save_mean, partial,    \
                                                      lx.rows, C, sh.cvb, flags, recompute ? s : nullptr,             \
-                                                     recompute ? b : nullptr, recompute ? save_invstd : nullptr);    \
+                                                     recompute ? b : nullptr, recompute ? save_invstd : nullptr,     \
+                                                     early_dz ? (T *)dz->ptr : nullptr, ldz.pitch);                  \
         bn_bwd_finalize<<<(C + 3) / 4, 256, 0, st>>>(partial, sh.gx, s, save_invstd, ds, db, coef,                \
                                                          (double)lx.rows, C, beta_p);                                \
-        bn_bwd_apply_cl<T, VN, RC><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, relu ? (const T *)y->ptr : nullptr,  \
-                                                     ly.pitch, (const T *)dy->ptr, ldy.pitch, (T *)dx->ptr,          \
-                                                     ldx.pitch, dz ? (T *)dz->ptr : nullptr, ldz.pitch, save_mean,   \
-                                                     coef, lx.rows, C, sh.cvb, flags, beta_dx, beta_dz,              \
-                                                     recompute ? b : nullptr);                                       \
+        if(early_dz)                                                                                                 \
+            bn_bwd_apply_cl<T, VN, false><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, nullptr, 0,              \
+                                                                (const T *)dz->ptr, ldz.pitch, (T *)dx->ptr,          \
+                                                                ldx.pitch, nullptr, 0, save_mean, coef, lx.rows, C,   \
+                                                                sh.cvb, flags & ~SAGA_BN_RELU, beta_dx, 0.0f,         \
+                                                                nullptr);                                             \
+        else                                                                                                         \
+            bn_bwd_apply_cl<T, VN, RC><<<grid, 256, 0, st>>>(                                                        \
+                (const T *)x->ptr, lx.pitch, relu ? (const T *)y->ptr : nullptr, ly.pitch, (const T *)dy->ptr,       \
+                ldy.pitch, (T *)dx->ptr, ldx.pitch, dz ? (T *)dz->ptr : nullptr, ldz.pitch, save_mean, coef,         \
+                lx.rows, C, sh.cvb, flags, beta_dx, beta_dz, recompute ? b : nullptr);                               \
     } while(0)
         if(dt == SAGA_HALF) {
             if(vn == 8) GO(half_t, 8); else GO(half_t, 1);

@@ -707,6 +707,8 @@ struct BnBwd : public HipOperation {
     {
         const double e = nbytes(dx_);
         const bool reads_y = (flags_ & SAGA_BN_RELU) && (flags_ & SAGA_BN_ADD);
+        if(reads_y && dz_ && dz_beta_ == 0) // pass 1: x, y, dy -> dz ; pass 2: x, dz -> dx
+            return e * (7 + (dx_beta_ != 0 ? 1 : 0));
         return e * (4 + (reads_y ? 2 : 0) + 1 + (dz_ ? 1 : 0) + (dx_beta_ != 0 ? 1 : 0) +
                     (dz_ && dz_beta_ != 0 ? 1 : 0));
     }
