@@ -348,8 +348,8 @@ class Program:
 
     def profile(self):
         """[{kind, launches, ms, flops, bytes}] accumulated since set_profiling(True)."""
-        rows = (_ProfileRow * 64)()
-        n = lib().saga_program_profile(self._h, rows, 64)
+        rows = (_ProfileRow * 1024)()
+        n = lib().saga_program_profile(self._h, rows, 1024)
         if n < 0:
             raise _err("profile")
         return [{"kind": rows[i].kind.decode(), "launches": rows[i].launches, "ms": rows[i].ms,

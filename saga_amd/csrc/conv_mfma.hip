@@ -344,31 +344,52 @@ __global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArg
     const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void *)g.a, 0, g.a_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void *)g.b, 0, g.b_bytes, 0x00020000);
 
-    // this lane fills slot (tid & 3) of row lrow (+64 per round) and fetches the logical
+    // this lane fills slot (tid % SLOTS) of row lrow (+RPR per round) and fetches the logical
     // channel vector that the swizzle assigns to that slot
     const int lrow = tid / SLOTS;
     const int kv = ((tid % SLOTS) ^ swz_of(lrow)) * 8;
-    int a_base[AV], a_y[AV], a_x[AV];
-    bool a_ok[AV];
+
+    // Address generation is hoisted out of the main loop: the input position of tap (ri, si)
+    // is (iy0 + ri*sy, ix0 + si*sy), sy = dil forward and -1 backward (inside a residue class
+    // consecutive taps are one input row / column apart), so a row's byte offset is
+    // rowoff + a term that is the same for every lane (kept in scalar registers), and which
+    // taps fall inside the image is one bit each of a 64-bit mask computed once per row.
+    const int sy = BWD ? -1 : g.dil;
+    int rowoff[AV];
+    unsigned long long amask[AV];
 #pragma unroll
     for(int j = 0; j < AV; j++) {
         const int m = m0 + lrow + RPR * j;
-        a_ok[j] = m < Mloc;
-        const int mm = a_ok[j] ? m : 0;
+        bool ok = m < Mloc;
+        const int mm = ok ? m : 0;
         const int ox = mm % PW;
         const int t = mm / PW;
         const int oy = t % PH;
         const int n = t / PH;
-        a_base[j] = n * g.IH * g.IW;
+        int iy0, ix0;
         if(BWD) {
             const int y = oy * rstep + py, x = ox * rstep + px;
-            a_ok[j] = a_ok[j] && y < g.OH && x < g.OW;
-            a_y[j] = y + g.pad;
-            a_x[j] = x + g.pad;
+            ok = ok && y < g.OH && x < g.OW;
+            iy0 = (y + g.pad - r0) >> g.sshift;
+            ix0 = (x + g.pad - s0) >> g.sshift;
         } else {
-            a_y[j] = oy * g.stride - g.pad;
-            a_x[j] = ox * g.stride - g.pad;
+            iy0 = oy * g.stride - g.pad;
+            ix0 = ox * g.stride - g.pad;
         }
+        rowoff[j] = (((n * g.IH + iy0) * g.IW + ix0) * g.lda + kv) * 2;
+        unsigned long long mk = 0;
+        if(ok)
+            for(int a = 0; a < nr; a++) {
+                const int iy = iy0 + a * sy;
+                if(iy < 0 || iy >= g.IH)
+                    continue;
+                for(int b = 0; b < ns; b++) {
+                    const int ix = ix0 + b * sy;
+                    if(ix >= 0 && ix < g.IW)
+                        mk |= 1ull << (a * ns + b);
+                }
+            }
+        amask[j] = mk;
     }
     const int ktot = g.R * g.S * g.Cred;
     int b_off[BV];
@@ -377,7 +398,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArg
     for(int j = 0; j < BV; j++) {
         const int n = n0 + lrow + RPR * j;
         b_ok[j] = n < g.Ngemm;
-        b_off[j] = (b_ok[j] ? n : 0) * ktot;
+        b_off[j] = ((b_ok[j] ? n : 0) * ktot + kv) * 2;
     }
 
     int ri = 0, si = 0, c0 = 0; // tap counters and channel offset of the NEXT slice to be issued
@@ -389,30 +410,18 @@ __global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArg
     auto issue_piece = [&](int stage, int p) {
         char *sa = smem + stage * STAGE_BYTES;
         char *sb = sa + BM * ROWB;
-        const int c = c0 + kv;
-        const bool cok = c < g.Cred;
-        const int r = r0 + ri * rstep, s = s0 + si * rstep;
+        const bool cok = c0 + kv < g.Cred;
         if(p < AV) {
             const int j = p;
-            int iy, ix;
-            bool ok = a_ok[j] && cok;
-            if(BWD) {
-                const int ty = a_y[j] - r * g.dil, tx = a_x[j] - s * g.dil;
-                ok = ok && ty >= 0 && tx >= 0 && ((ty | tx) & (g.stride - 1)) == 0;
-                iy = ty >> g.sshift;
-                ix = tx >> g.sshift;
-            } else {
-                iy = a_y[j] + r * g.dil;
-                ix = a_x[j] + s * g.dil;
-                ok = ok && iy >= 0 && ix >= 0;
-            }
-            ok = ok && iy < g.IH && ix < g.IW;
-            const unsigned off = ok ? (unsigned)(((a_base[j] + iy * g.IW + ix) * g.lda + c) * 2) : OOB;
+            const int tapoff = ((ri * g.IW + si) * sy * g.lda + c0) * 2; // same for all lanes
+            const bool ok = cok && ((amask[j] >> (ri * ns + si)) & 1);
+            const unsigned off = ok ? (unsigned)(rowoff[j] + tapoff) : OOB;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(sa + (j * RPR + wave * RPI) * ROWB), 16, off, 0, 0, 0);
         } else {
             const int j = p - AV;
-            const int kb = (r * g.S + s) * g.Cred + c;
-            const unsigned off = (b_ok[j] && cok) ? (unsigned)((b_off[j] + kb) * 2) : OOB;
+            const int r = r0 + ri * rstep, s = s0 + si * rstep;
+            const int kb = ((r * g.S + s) * g.Cred + c0) * 2;
+            const unsigned off = (b_ok[j] && cok) ? (unsigned)(b_off[j] + kb) : OOB;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(sb + (j * RPR + wave * RPI) * ROWB), 16, off, 0, 0, 0);
         }
     };
@@ -1268,7 +1277,12 @@ template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
     g.Mc = g.M;
     g.OHc = g.OH;
     g.OWc = g.OW;
-    if(dma_stages() >= 2 && g.a_bytes && g.b_bytes) {
+    // the pipelined kernel keeps one validity bit per tap (of a residue class) in a 64-bit mask
+    // and, backward, steps one input row / column per tap: dilation 1, stride 1 or a class split
+    const int sdiv = BWD ? g.stride : 1;
+    const bool fits = ((g.R + sdiv - 1) / sdiv) * ((g.S + sdiv - 1) / sdiv) <= 64 &&
+                      (!BWD || (g.dil == 1 && g.stride <= 4));
+    if(dma_stages() >= 2 && g.a_bytes && g.b_bytes && fits) {
         constexpr int ST = 3;
         int active = 1;
         if(BWD && g.stride > 1 && g.stride <= 4 && g.dil == 1) {

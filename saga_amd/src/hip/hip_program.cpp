@@ -536,8 +536,11 @@ void HipProgram::collectProfile()
         float ms = 0;
         if(hipEventElapsedTime(&ms, m_events[i], m_events[i + 1]) != hipSuccess)
             continue;
-        auto &row = m_profile[m_ops[i]->name()];
-        row.kind = m_ops[i]->name();
+        // SAGA_HIP_PROFILE_PER_OP=1: one row per operation (kind#position) instead of per kind
+        static const bool per_op = getenv("SAGA_HIP_PROFILE_PER_OP") != nullptr;
+        const std::string key = per_op ? fmt("%s#%03zu", m_ops[i]->name().c_str(), i) : m_ops[i]->name();
+        auto &row = m_profile[key];
+        row.kind = key;
         row.launches++;
         row.ms += ms;
         row.flops += m_ops[i]->flops();
