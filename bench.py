@@ -35,7 +35,13 @@ CONV_KINDS = ("convfwd", "convbwddata", "convbwdfilter")
 # operation launches, each counter scaled by what it reads for a plain copy of known size
 # (FETCH_SIZE reads 0.5 of the bytes a 1 GiB copy fetches, WRITE_SIZE 1.0).  The command lines and
 # the per-kernel table are in profiles/resnet50_b256_fp16_hbm_counters.txt.
-MEASURED_HBM_BYTES_PER_LAUNCH = {}
+MEASURED_HBM_BYTES_PER_LAUNCH = {
+    # the counters cannot tell fused from plain batch-norm launches (same kernels): both kinds carry
+    # the average over all 53 batch-norm launches of a step
+    "bnbwd.fused": 666484230, "bnbwd": 666484230,
+    "bntrain.fused": 275035172, "bntrain": 275035172,
+    "convfwd": 229309974, "convbwddata": 290906476, "convbwdfilter": 302333026,
+}
 
 
 def profile_rows(rows):
