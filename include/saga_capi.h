@@ -84,6 +84,10 @@ saga_context_t saga_context_create(void);
 void saga_context_release(saga_context_t c);
 int saga_context_reset(saga_context_t c);
 saga_tensor_t saga_context_resolve(saga_context_t c, saga_tensor_t t);
+/* Storage reuse of the context (the role of the reference's liveness + best-fit layout,
+ * src/cuda/cuda_analysis.cpp:194-547): bytes of the shared arena and the sum of the sizes of the
+ * storages laid out in it.  Both 0 before a program is finalized or with SAGA_HIP_NO_ARENA set. */
+int saga_context_memory(saga_context_t c, size_t *arena_bytes, size_t *planned_bytes);
 
 /* phases: 1 PRE, 2 POST, 3 both */
 saga_program_t saga_program_create(saga_context_t c, saga_graph_t g, int batch_size, int training,

@@ -74,6 +74,7 @@ SIGNATURES = {
     "saga_context_release": (None, [_VP]),
     "saga_context_reset": (C.c_int, [_VP]),
     "saga_context_resolve": (_VP, [_VP, _VP]),
+    "saga_context_memory": (C.c_int, [_VP, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
     "saga_program_create": (_VP, [_VP, _VP, C.c_int, C.c_int, C.POINTER(_Config), C.c_int, C.POINTER(_VP),
                                   C.POINTER(C.c_int)]),
     "saga_program_release": (None, [_VP]),
@@ -298,6 +299,13 @@ class Context:
     def reset(self):
         if lib().saga_context_reset(self._h):
             raise _err("reset")
+
+    def memory(self):
+        """(arena bytes, total bytes of the storages laid out in the arena)."""
+        a, b = C.c_size_t(0), C.c_size_t(0)
+        if lib().saga_context_memory(self._h, C.byref(a), C.byref(b)):
+            raise _err("memory")
+        return a.value, b.value
 
     def resolve(self, t):
         """Context::resolveTensor: the device tensor behind front-end tensor t (None if unused)."""

@@ -334,6 +334,19 @@ int saga_program_run(saga_program_t p, long batches)
     return g ? g : rc;
 }
 
+int saga_context_memory(saga_context_t c, size_t *arena_bytes, size_t *planned_bytes)
+{
+    return guard([&] {
+        auto hc = std::dynamic_pointer_cast<HipContext>(((ContextBox *)c)->c);
+        if(!hc)
+            throw std::runtime_error("not a hip context");
+        if(arena_bytes)
+            *arena_bytes = hc->m_arena_bytes;
+        if(planned_bytes)
+            *planned_bytes = hc->m_planned_bytes;
+    });
+}
+
 double saga_program_loss_scale(saga_program_t p) { return ((ProgramBox *)p)->p->getMPS(); }
 
 int saga_program_set_profiling(saga_program_t p, int on)

@@ -69,11 +69,22 @@ public:
     HipStorage(Tensor::DataType dt, size_t elements, HipContext *ctx);
     virtual ~HipStorage() {}
 
-    virtual void *deviceMem() const { return m_data; }
+    // Device memory is attached on first use: either an allocation of its own, or - for
+    // storages whose contents live only within one step - a slot of the context's arena,
+    // assigned by HipContext::planMemory() when a program is finalized.
+    virtual void *deviceMem() const
+    {
+        if(!m_data)
+            const_cast<HipStorage *>(this)->allocOwn();
+        return m_data;
+    }
+    bool allocated() const { return m_data != nullptr; }
     // host staging: whole-storage copies around TensorAccess lifetimes
     virtual bool doubleBuffered() const { return false; }
 
     void rehome(const std::shared_ptr<HipMemory> &mem, void *ptr);
+    void allocOwn();
+    size_t bytes() const { return m_elements * m_element_size; }
 
     HipContext *const m_ctx;
     const Tensor::DataType m_data_type;
@@ -82,6 +93,7 @@ public:
     const int m_id;
     std::shared_ptr<HipMemory> m_memory;
     void *m_data = nullptr;
+    bool m_in_arena = false; // m_data points into the context's arena (contents do not survive a step)
     bool m_nonfinite_is_valid = false;
 };
 
@@ -127,6 +139,9 @@ public:
     void *deviceMem() const;
     // the 4-D view handed to the kernel library (rank < 4 is padded; rank 1 becomes [1,C,1,1])
     SagaTensorView view() const;
+    // the same with a placeholder address when no memory is attached yet: for size queries at
+    // set-up time, which must not trigger an allocation
+    SagaTensorView shapeView() const;
     // [rows, cols] matrices for the fc path
     bool cpacked() const; // channel stride 1 (NHWC-like) for rank-4 tensors
     bool rowMajor() const;
@@ -217,6 +232,16 @@ public:
     std::unordered_map<std::shared_ptr<HipTensor>, std::shared_ptr<Tensor>> m_deferred_copy;
     // storages handed out to the host: kept by the dead-code elimination
     std::vector<std::shared_ptr<HipStorage>> m_exported;
+
+    // ---- storage reuse (role of the reference's src/cuda/cuda_analysis.cpp:194-547)
+    // Finalized programs of this context; planMemory() lays the storages that live only within a
+    // step of every program that touches them into one arena, overlapping those whose live
+    // ranges never intersect.
+    std::vector<class HipProgram *> m_programs;
+    std::shared_ptr<HipMemory> m_arena;
+    size_t m_arena_bytes = 0;    // size of the arena
+    size_t m_planned_bytes = 0;  // sum of the sizes of the storages laid out in it
+    void planMemory();
 };
 
 class HipProgram : public Program {

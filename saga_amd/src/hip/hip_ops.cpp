@@ -49,7 +49,7 @@ struct ConvFwd : public HipOperation {
     std::shared_ptr<ConvStatsLink> stats_;
     ConvFwd(HipProgram &p, T x, T w, T y, SagaConvParams cp) : HipOperation("convfwd"), x_(x), w_(w), y_(y), cp_(cp)
     {
-        const SagaTensorView vx = x->view(), vw = w->view(), vy = y->view();
+        const SagaTensorView vx = x->shapeView(), vw = w->shapeView(), vy = y->shapeView();
         p.m_ctx->m_workspace.request(saga_hip_conv2d_workspace_size(SAGA_CONV_FWD, &vx, &vw, &vy, &cp_));
     }
     // called by a batch normalisation that consumes y; nullptr if this convolution cannot supply them
@@ -57,7 +57,7 @@ struct ConvFwd : public HipOperation {
     {
         if(stats_)
             return stats_;
-        const SagaTensorView vx = x_->view(), vw = w_->view(), vy = y_->view();
+        const SagaTensorView vx = x_->shapeView(), vw = w_->shapeView(), vy = y_->shapeView();
         const size_t bytes = saga_hip_conv2d_fwd_bnstats_size(&vx, &vw, &vy, &cp_);
         if(!bytes)
             return nullptr;
@@ -99,7 +99,7 @@ struct ConvBwdData : public HipOperation {
     ConvBwdData(HipProgram &p, T w, T dy, T dx, SagaConvParams cp)
       : HipOperation("convbwddata"), w_(w), dy_(dy), dx_(dx), cp_(cp)
     {
-        const SagaTensorView vx = dx->view(), vw = w->view(), vy = dy->view();
+        const SagaTensorView vx = dx->shapeView(), vw = w->shapeView(), vy = dy->shapeView();
         p.m_ctx->m_workspace.request(saga_hip_conv2d_workspace_size(SAGA_CONV_BWD_DATA, &vx, &vw, &vy, &cp_));
     }
     void exec(HipProgram &p) override
@@ -122,7 +122,7 @@ struct ConvBwdFilter : public HipOperation {
     ConvBwdFilter(HipProgram &p, T x, T dy, T dw, SagaConvParams cp)
       : HipOperation("convbwdfilter"), x_(x), dy_(dy), dw_(dw), cp_(cp)
     {
-        const SagaTensorView vx = x->view(), vw = dw->view(), vy = dy->view();
+        const SagaTensorView vx = x->shapeView(), vw = dw->shapeView(), vy = dy->shapeView();
         p.m_ctx->m_workspace.request(saga_hip_conv2d_workspace_size(SAGA_CONV_BWD_FILTER, &vx, &vw, &vy, &cp_));
     }
     void exec(HipProgram &p) override
@@ -601,7 +601,7 @@ struct BnTrain : public HipOperation {
       : HipOperation(flags ? "bntrain.fused" : "bntrain")
       , x_(x), z_(z), s_(s), b_(b), m_(m), v_(v), y_(y), sm_(sm), sv_(sv), eps_(eps), flags_(flags)
     {
-        const SagaTensorView vx = x->view();
+        const SagaTensorView vx = x->shapeView();
         p.m_ctx->m_workspace.request(saga_hip_bn_workspace_size(&vx));
     }
     void exec(HipProgram &p) override

@@ -9,7 +9,9 @@
 
 #include <algorithm>
 #include <cmath>
+#include <set>
 #include <sstream>
+#include <unordered_map>
 
 #include "hip_common.hpp"
 // after saga.hpp: the registry header relies on its declarations
@@ -174,7 +176,126 @@ std::shared_ptr<Tensor> HipContext::resolveTensor(std::shared_ptr<Tensor> src)
     if(it == m_tensors.end())
         return nullptr;
     m_exported.push_back(it->second->m_storage);
+    // a tensor the host holds keeps its contents between steps: out of the shared arena
+    // (reference: src/cuda/cuda_common.cpp:145-158)
+    auto &st = it->second->m_storage;
+    if(st->m_in_arena) {
+        // memory of its own from here on; what the arena slot holds right now moves along
+        sync();
+        auto keep = st->m_memory;
+        void *old = st->m_data;
+        st->allocOwn();
+        chkHip(hipMemcpy(st->m_data, old, st->bytes(), hipMemcpyDeviceToDevice));
+    }
     return it->second;
+}
+
+// Storage reuse.  A storage qualifies when, in every finalized program that touches it, the
+// first operation to touch it overwrites it (nothing is carried over from the previous step or
+// from the host), the host holds no reference to it, and it has no memory of its own yet
+// (weights, optimizer state and anything the host wrote have).  Two such storages may share
+// addresses unless some program uses both with overlapping live ranges [first touch, last
+// touch].  Placement is first-fit by decreasing size against the already placed storages that
+// conflict.  The reference walks one program with a best-fit free list
+// (src/cuda/cuda_analysis.cpp:472-530); planning per context instead keeps an inference and a
+// training program that share activations from overwriting each other's tensors.
+void HipContext::planMemory()
+{
+    static const bool disabled = getenv("SAGA_HIP_NO_ARENA") != nullptr;
+    if(disabled)
+        return;
+    struct Range {
+        int prog, first, last;
+    };
+    struct Item {
+        HipStorage *s;
+        size_t bytes, offset;
+        std::vector<Range> ranges;
+    };
+    std::unordered_map<HipStorage *, Item> items;
+    std::set<HipStorage *> carried;
+    for(size_t pi = 0; pi < m_programs.size(); pi++) {
+        const HipOps &ops = m_programs[pi]->m_ops;
+        std::unordered_map<HipStorage *, Range> seen;
+        for(size_t i = 0; i < ops.size(); i++) {
+            auto touch = [&](const HipOpArgs &args, bool reads) {
+                for(const auto &a : args) {
+                    HipStorage *st = a.second->m_storage.get();
+                    auto it = seen.find(st);
+                    if(it == seen.end()) {
+                        seen[st] = Range{(int)pi, (int)i, (int)i};
+                        // a partial first write leaves the rest of the storage as it was
+                        if(reads || a.second->m_dims.elements() != st->m_elements)
+                            carried.insert(st);
+                    } else {
+                        it->second.last = (int)i;
+                    }
+                }
+            };
+            touch(ops[i]->getInputs(), true);
+            touch(ops[i]->getOutputs(), false);
+        }
+        for(const auto &kv : seen) {
+            auto &it = items[kv.first];
+            it.s = kv.first;
+            it.ranges.push_back(kv.second);
+        }
+    }
+    std::set<HipStorage *> exported;
+    for(const auto &e : m_exported)
+        exported.insert(e.get());
+    std::vector<Item *> cand;
+    for(auto &kv : items) {
+        HipStorage *st = kv.first;
+        if(carried.count(st) || exported.count(st) || st->doubleBuffered())
+            continue;
+        if(st->allocated() && !st->m_in_arena)
+            continue;
+        kv.second.bytes = (st->bytes() + 255) & ~(size_t)255;
+        cand.push_back(&kv.second);
+    }
+    std::sort(cand.begin(), cand.end(), [](const Item *a, const Item *b) {
+        return a->bytes != b->bytes ? a->bytes > b->bytes : a->s->m_id < b->s->m_id;
+    });
+    auto conflict = [](const Item &a, const Item &b) {
+        for(const auto &ra : a.ranges)
+            for(const auto &rb : b.ranges)
+                if(ra.prog == rb.prog && ra.first <= rb.last && rb.first <= ra.last)
+                    return true;
+        return false;
+    };
+    std::vector<Item *> placed;
+    size_t total = 0, planned = 0;
+    for(Item *it : cand) {
+        std::vector<std::pair<size_t, size_t>> busy; // [begin, end) of conflicting storages
+        for(Item *q : placed)
+            if(conflict(*it, *q))
+                busy.emplace_back(q->offset, q->offset + q->bytes);
+        std::sort(busy.begin(), busy.end());
+        size_t off = 0;
+        for(const auto &b : busy) {
+            if(off + it->bytes <= b.first)
+                break;
+            off = std::max(off, b.second);
+        }
+        it->offset = off;
+        placed.push_back(it);
+        total = std::max(total, off + it->bytes);
+        planned += it->bytes;
+    }
+    if(placed.empty())
+        return;
+    auto arena = std::make_shared<HipMemory>(total); // zero filled once; slots are not cleared on reuse
+    for(Item *it : placed) {
+        it->s->rehome(arena, (char *)arena->m_ptr + it->offset);
+        it->s->m_in_arena = true;
+    }
+    m_arena = arena;
+    m_arena_bytes = total;
+    m_planned_bytes = planned;
+    if(getenv("SAGA_HIP_VERBOSE"))
+        fprintf(stderr, "hip: arena %.1f MB holds %zu storages of %.1f MB in total\n", total / 1e6, placed.size(),
+                planned / 1e6);
 }
 
 // reference: src/cuda/cuda_common.cpp:322-399
@@ -239,6 +360,8 @@ HipProgram::HipProgram(std::shared_ptr<HipContext> ctx, ProgramType pt, const Pr
 HipProgram::~HipProgram()
 {
     m_ctx->sync();
+    auto &ps = m_ctx->m_programs;
+    ps.erase(std::remove(ps.begin(), ps.end(), this), ps.end());
     for(auto e : m_events)
         (void)hipEventDestroy(e);
     (void)hipHostFree(m_aux);
@@ -449,6 +572,8 @@ void HipProgram::finalize()
     eliminateDeadOps();
 
     m_ctx->m_workspace.alloc();
+    m_ctx->m_programs.push_back(this);
+    m_ctx->planMemory();
 }
 
 // ---------------------------------------------------------------- run loop

@@ -46,6 +46,13 @@ void HipStorage::rehome(const std::shared_ptr<HipMemory> &mem, void *ptr)
 {
     m_memory = mem;
     m_data = ptr;
+    m_in_arena = false;
+}
+
+void HipStorage::allocOwn()
+{
+    auto mem = std::make_shared<HipMemory>(bytes()); // zero filled
+    rehome(mem, mem->m_ptr);
 }
 
 HipDoubleBuffer::HipDoubleBuffer(Tensor::DataType dt, size_t elements, HipContext *ctx) : HipStorage(dt, elements, ctx)
@@ -134,8 +141,6 @@ HipTensor::HipTensor(DataType dt, const Dims &dims, HipLayout layout, HipContext
   : Tensor(dt, dims, name), m_strides(hip_strides(dims, layout))
 {
     m_storage = std::make_shared<HipStorage>(dt, dims.elements(), ctx);
-    auto mem = std::make_shared<HipMemory>(dims.elements() * DataTypeSize(dt));
-    m_storage->rehome(mem, mem->m_ptr);
 }
 
 HipTensor::HipTensor(std::shared_ptr<HipStorage> storage, const Dims &dims, const std::vector<int64_t> &strides,
@@ -151,8 +156,6 @@ HipTensor::HipTensor(DataType dt, const HipTensor &like, const std::optional<con
     const bool nhwc = like.m_dims.size() == 4 && like.cpacked();
     m_strides = hip_strides(like.m_dims, nhwc ? HipLayout::NHWC : HipLayout::NCHW);
     m_storage = std::make_shared<HipStorage>(dt, like.m_dims.elements(), like.m_storage->m_ctx);
-    auto mem = std::make_shared<HipMemory>(like.m_dims.elements() * DataTypeSize(dt));
-    m_storage->rehome(mem, mem->m_ptr);
 }
 
 void *HipTensor::deviceMem() const
@@ -171,6 +174,18 @@ bool HipTensor::rowMajor() const
         acc *= (int)m_dims[i];
     }
     return true;
+}
+
+SagaTensorView HipTensor::shapeView() const
+{
+    if(m_storage->allocated() || m_storage->doubleBuffered())
+        return view();
+    HipStorage *s = m_storage.get();
+    void *const keep = s->m_data;
+    s->m_data = (void *)(uintptr_t)4096; // aligned placeholder, never dereferenced
+    SagaTensorView v = view();
+    s->m_data = keep;
+    return v;
 }
 
 SagaTensorView HipTensor::view() const

@@ -165,3 +165,31 @@ def test_unet_training_fp16():
     net.output = b.fc(b.pool("avgpool", net.output, global_=True), "cls", 8)
     run_training(net, 6, steps=1, lr=1e-3, loss_scale=256.0,
                  check_params=["down0a-w", "up3-t-w", "up0-t-w", "up0a-w", "head-w", "up2-t-b"])
+
+
+def test_storage_reuse_arena():
+    """Activations and gradients that live only within a step share one arena (the role of the
+    reference's liveness + best-fit layout, src/cuda/cuda_analysis.cpp:194-547): it is smaller
+    than the storages laid out in it, tensors the host resolved stay out of it and keep their
+    values, and a tensor resolved only after the first step moves out with its contents."""
+    net = N.resnet20(8)
+    x, labels = inputs(net, 3)
+    ctx = S.Context()
+    g, t = N.build_graph(net, x)
+    p = ctx.create_program(g, net.batch, training=True, learning_rate=1e-3)
+    logits = ctx.resolve(t[net.output])
+    ctx.resolve(t["labels"]).write(labels)
+    assert ctx.memory() == (0, 0)
+    p.run(1)
+    arena, planned = ctx.memory()
+    print(f"arena {arena} bytes for {planned} bytes of storages")
+    assert 0 < arena < 0.7 * planned
+    first = logits.read().astype(np.float32)
+    assert np.isfinite(first).all() and np.abs(first).max() > 0
+    # the classifier's gradient is the last tensor written into its arena slot before Adam runs
+    dlogits = ctx.resolve(t[net.output].grad())
+    late = dlogits.read().astype(np.float32)
+    assert np.abs(late).max() > 0
+    p.run(1)
+    assert np.abs(dlogits.read().astype(np.float32)).max() > 0
+    assert not np.array_equal(logits.read().astype(np.float32), first)  # the weights moved
