@@ -291,6 +291,10 @@ public:
     std::string m_name;
 
     HipOps m_ops;
+    // anomaly detection: arena storages to fill with NaN bytes before the operation that defines
+    // them and after the last one that uses them (reference: m_pre_invalidate / m_post_invalidate,
+    // src/cuda/cuda_analysis.cpp:486-517), indexed like m_ops
+    std::vector<std::vector<HipStorage *>> m_poison_before, m_poison_after;
     HipOps m_opt;
     std::vector<HipProgramUnit> m_units;
 

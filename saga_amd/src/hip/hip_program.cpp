@@ -290,6 +290,17 @@ void HipContext::planMemory()
         it->s->rehome(arena, (char *)arena->m_ptr + it->offset);
         it->s->m_in_arena = true;
     }
+    for(size_t pi = 0; pi < m_programs.size(); pi++) {
+        HipProgram *pr = m_programs[pi];
+        pr->m_poison_before.assign(pr->m_ops.size(), {});
+        pr->m_poison_after.assign(pr->m_ops.size(), {});
+        for(Item *it : placed)
+            for(const auto &r : it->ranges)
+                if(r.prog == (int)pi) {
+                    pr->m_poison_before[r.first].push_back(it->s);
+                    pr->m_poison_after[r.last].push_back(it->s);
+                }
+    }
     m_arena = arena;
     m_arena_bytes = total;
     m_planned_bytes = planned;
@@ -684,7 +695,15 @@ void HipProgram::runOps(const HipOps &ops)
         chkHip(hipEventRecord(m_events[0], m_ctx->m_stream));
     }
     size_t index = 0;
+    const bool poison = m_pc.anomaly_detect && &ops == &m_ops && m_poison_before.size() == ops.size();
+    auto fill_nan = [&](const std::vector<HipStorage *> &list) {
+        for(HipStorage *s : list)
+            if(s->m_in_arena)
+                chkSaga(saga_hip_fill(s->m_data, 0xff, s->bytes(), (saga_stream_t)m_ctx->m_stream));
+    };
     for(const auto &op : ops) {
+        if(poison)
+            fill_nan(m_poison_before[index]);
         if(m_pc.anomaly_detect)
             checkAnomaly(*op, op->getInputs(), "input");
         try {
@@ -694,6 +713,8 @@ void HipProgram::runOps(const HipOps &ops)
         }
         if(m_pc.anomaly_detect)
             checkAnomaly(*op, op->getOutputs(), "output");
+        if(poison)
+            fill_nan(m_poison_after[index]);
         index++;
         if(m_profiling)
             chkHip(hipEventRecord(m_events[index], m_ctx->m_stream));

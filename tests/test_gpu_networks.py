@@ -193,3 +193,19 @@ def test_storage_reuse_arena():
     p.run(1)
     assert np.abs(dlogits.read().astype(np.float32)).max() > 0
     assert not np.array_equal(logits.read().astype(np.float32), first)  # the weights moved
+
+
+def test_storage_reuse_under_anomaly_detection():
+    """With anomaly detection on, every arena slot is filled with NaN bytes before the operation that
+    defines it and after the last one that uses it (reference: src/cuda/cuda_analysis.cpp:486-517)
+    and every operation's inputs and outputs are checked: a read outside a live range would trip."""
+    net = N.resnet20(8)
+    x, labels = inputs(net, 5)
+    ctx = S.Context()
+    g, t = N.build_graph(net, x)
+    p = ctx.create_program(g, net.batch, training=True, learning_rate=1e-3, anomaly_detect=True)
+    logits = ctx.resolve(t[net.output])
+    ctx.resolve(t["labels"]).write(labels)
+    p.run(3)
+    assert ctx.memory()[0] > 0
+    assert np.isfinite(logits.read().astype(np.float32)).all()
