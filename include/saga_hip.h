@@ -118,6 +118,18 @@ int saga_hip_conv2d_fwd_bnstats(const SagaTensorView *x, const SagaTensorView *w
                                 const SagaConvParams *p, float alpha, void *workspace, size_t ws_bytes,
                                 float *partial, size_t partial_bytes, int *partial_rows, saga_stream_t stream);
 
+/* ---- convolution forward with the batch-norm INFERENCE that follows it (and that norm's optional
+ *      residual add and relu) applied in the epilogue: y = act(s*(conv(x,w) - m)/sqrt(v+eps) + b (+ z)).
+ *      The reference runs cudnnConvolutionForward (src/cuda/cuda_dnn.cpp:207-221) and
+ *      cudnnBatchNormalizationForwardInference (:1641-1651) as two passes over the tensor; here the
+ *      convolution's output never reaches memory un-normalised (and is not rounded to fp16 in
+ *      between).  Returns SAGA_HIP_EUNSUPPORTED, with nothing written, outside the fp16
+ *      channels-last MFMA path: run saga_hip_conv2d_fwd and saga_hip_bn_infer instead. */
+int saga_hip_conv2d_fwd_bn_infer(const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y,
+                                 const SagaTensorView *z, const SagaConvParams *p, const float *s, const float *b,
+                                 const float *m, const float *v, float eps, int flags, void *workspace,
+                                 size_t ws_bytes, saga_stream_t stream);
+
 /* y[n,c,:,:] += b[c] : cudnnAddTensor of a {1,C,1,1} bias (src/cuda/cuda_dnn.cpp:39-68). b is fp32 or y's type. */
 int saga_hip_bias_add(const SagaTensorView *y, const SagaTensorView *b, saga_stream_t stream);
 /* db[c] = beta*db + sum_{n,h,w} dy : cudnnConvolutionBackwardBias (src/cuda/cuda_dnn.cpp:378-385). */

@@ -94,6 +94,23 @@ int saga_hip_conv2d_fwd_bnstats(const SagaTensorView *x, const SagaTensorView *w
                          partial_bytes / sizeof(float), partial_rows);
 }
 
+int saga_hip_conv2d_fwd_bn_infer(const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y,
+                                 const SagaTensorView *z, const SagaConvParams *p, const float *s, const float *b,
+                                 const float *m, const float *v, float eps, int flags, void *workspace,
+                                 size_t ws_bytes, saga_stream_t stream)
+{
+    ConvGeom g;
+    int r = geometry(x, w, y, p, &g);
+    if(r)
+        return r;
+    if(!s || !b || !m || !v || ((flags & SAGA_BN_ADD) && !z))
+        return SAGA_HIP_EINVAL;
+    if(force_direct())
+        return SAGA_HIP_EUNSUPPORTED;
+    const ConvBnFold bn = {s, b, m, v, eps, flags, z};
+    return conv_mfma_fwd(x, w, y, g, 1.0f, 0.0f, workspace, ws_bytes, as_stream(stream), nullptr, 0, nullptr, &bn);
+}
+
 int saga_hip_conv2d_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx,
                              const SagaConvParams *p, float alpha, float beta, void *workspace, size_t ws_bytes,
                              saga_stream_t stream)

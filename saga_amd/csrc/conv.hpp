@@ -24,9 +24,16 @@ size_t conv_mfma_workspace(int kind, const SagaTensorView *x, const SagaTensorVi
 // stats (optional): receives per block row and output channel the sum and the sum of squares of
 // the stored outputs, [*stats_rows][K][2] floats; needs beta == 0 and conv_mfma_stats_floats(g) floats
 size_t conv_mfma_stats_floats(const ConvGeom &g);
+// batch-norm inference (+ residual + relu) folded into the forward epilogue
+struct ConvBnFold {
+    const float *s, *b, *m, *v;
+    float eps;
+    int flags;
+    const SagaTensorView *z;
+};
 int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y, const ConvGeom &g,
                   float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st, float *stats = nullptr,
-                  size_t stats_floats = 0, int *stats_rows = nullptr);
+                  size_t stats_floats = 0, int *stats_rows = nullptr, const ConvBnFold *bn = nullptr);
 int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx,
                        const ConvGeom &g, float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st);
 int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, const SagaTensorView *dw,

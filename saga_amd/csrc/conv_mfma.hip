@@ -52,6 +52,13 @@ struct GatherArgs {
     int blocks_per_class;
     int nactive;       // classes that get blocks
     unsigned char cls_ids[16]; // residue classes that get blocks (classes with no tap are left out)
+    // forward only, optional: y = act(conv * sc[c] + sh[c] (+ z)) with sc = s*rsqrt(v+eps),
+    // sh = b - m*sc (batch-norm inference folded into the epilogue)
+    const float *bn_s, *bn_b, *bn_m, *bn_v;
+    float bn_eps;
+    int bn_flags;      // SAGA_BN_RELU | SAGA_BN_ADD
+    const half_t *z;   // residual, [M][ldz]
+    int ldz;
     float *stats;      // forward only, optional: per block row and output channel, sum and sum of
                        // squares of the stored outputs, [ceil(M / BM)][Ngemm][2]
     int stats_rows;    // out: block rows the launch wrote
@@ -534,8 +541,8 @@ __global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArg
 #pragma unroll
                 for(int v = 0; v < 16; v++)
                     f[v] = g.alpha * acc[i][j][v];
+                typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
                 if(g.beta != 0.0f) {
-                    typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 #pragma unroll
                     for(int q = 0; q < 4; q++) {
                         const int n = nb + 8 * q + 4 * hi;
@@ -544,6 +551,31 @@ __global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArg
 #pragma unroll
                             for(int e = 0; e < 4; e++)
                                 f[4 * q + e] += g.beta * (float)old[e];
+                        }
+                    }
+                }
+                if constexpr(!BWD) {
+                    if(g.bn_s) {
+#pragma unroll
+                        for(int q = 0; q < 4; q++) {
+                            const int n = nb + 8 * q + 4 * hi;
+                            if(n < g.Ngemm) {
+                                const float4_t vs = *(const float4_t *)(g.bn_s + n), vb = *(const float4_t *)(g.bn_b + n);
+                                const float4_t vm = *(const float4_t *)(g.bn_m + n), vv = *(const float4_t *)(g.bn_v + n);
+                                half4_t zz = {0, 0, 0, 0};
+                                if((g.bn_flags & SAGA_BN_ADD) && ok)
+                                    zz = *(const half4_t *)(g.z + pix * g.ldz + n);
+#pragma unroll
+                                for(int e = 0; e < 4; e++) {
+                                    const float sc = vs[e] * rsqrtf(vv[e] + g.bn_eps);
+                                    float t = __builtin_fmaf(f[4 * q + e], sc, vb[e] - vm[e] * sc);
+                                    if(g.bn_flags & SAGA_BN_ADD)
+                                        t += (float)zz[e];
+                                    if(g.bn_flags & SAGA_BN_RELU)
+                                        t = (t != t) ? t : fmaxf(t, 0.0f);
+                                    f[4 * q + e] = t;
+                                }
+                            }
                         }
                     }
                 }
@@ -571,6 +603,16 @@ __global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArg
                     float val = g.alpha * acc[i][j][v];
                     if(g.beta != 0.0f)
                         val += g.beta * (float)orow[n];
+                    if constexpr(!BWD) {
+                        if(g.bn_s) {
+                            const float sc = g.bn_s[n] * rsqrtf(g.bn_v[n] + g.bn_eps);
+                            val = __builtin_fmaf(val, sc, g.bn_b[n] - g.bn_m[n] * sc);
+                            if(g.bn_flags & SAGA_BN_ADD)
+                                val += (float)g.z[pix * g.ldz + n];
+                            if(g.bn_flags & SAGA_BN_RELU)
+                                val = (val != val) ? val : fmaxf(val, 0.0f);
+                        }
+                    }
                     orow[n] = (half_t)val;
                 }
             }
@@ -1339,7 +1381,7 @@ template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
         SAGA_CHECK_LAUNCH();
         return 0;
     }
-    if(g.stats)
+    if(g.stats || (!BWD && g.bn_s))
         return SAGA_HIP_EUNSUPPORTED;
     // tile choice by output-channel count; M tiles are 128 or 256 rows
     if(g.Ngemm > 64) {
@@ -1379,6 +1421,35 @@ static bool common_ok(const SagaTensorView *act_in, const SagaTensorView *w, con
         return false;
     if((int64_t)g.K * g.R * g.S * g.C >= (int64_t)1 << 31)
         return false;
+    return true;
+}
+
+// fills the batch-norm fold of a forward launch; false if the residual cannot be read in place
+static bool set_bn(GatherArgs &a, const ConvBnFold *bn, const SagaTensorView *y, const CLInfo &ly)
+{
+    a.bn_s = nullptr;
+    a.z = nullptr;
+    a.ldz = 0;
+    a.bn_flags = 0;
+    a.bn_eps = 0;
+    if(!bn)
+        return true;
+    a.bn_s = bn->s; a.bn_b = bn->b; a.bn_m = bn->m; a.bn_v = bn->v;
+    a.bn_eps = bn->eps;
+    a.bn_flags = bn->flags;
+    if(bn->flags & SAGA_BN_ADD) {
+        CLInfo lz;
+        if(!bn->z || bn->z->dtype != SAGA_HALF || !same_dims(bn->z, y) || !as_channels_last(bn->z, &lz) || lz.rows != ly.rows)
+            return false;
+        // 8-byte loads of 4 channels
+        if(lz.pitch % 4 || ((uintptr_t)bn->z->ptr & 7) || ((uintptr_t)bn->s & 15) || ((uintptr_t)bn->b & 15) ||
+           ((uintptr_t)bn->m & 15) || ((uintptr_t)bn->v & 15))
+            return false;
+        a.z = (const half_t *)bn->z->ptr;
+        a.ldz = (int)lz.pitch;
+    } else if(((uintptr_t)bn->s & 15) || ((uintptr_t)bn->b & 15) || ((uintptr_t)bn->m & 15) || ((uintptr_t)bn->v & 15)) {
+        return false;
+    }
     return true;
 }
 
@@ -1426,8 +1497,10 @@ size_t conv_mfma_workspace(int kind, const SagaTensorView *x, const SagaTensorVi
 
 int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y, const ConvGeom &g,
                   float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st, float *stats, size_t stats_floats,
-                  int *stats_rows)
+                  int *stats_rows, const ConvBnFold *bn)
 {
+    if(bn && (stats || beta != 0.0f))
+        return SAGA_HIP_EINVAL;
     if(stats && (beta != 0.0f || stats_floats < conv_mfma_stats_floats(g)))
         return SAGA_HIP_EINVAL;
     CLInfo lx, ly;
@@ -1459,6 +1532,8 @@ int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTe
         a.a_bytes = (unsigned)(px * 8);
         a.b_bytes = (unsigned)(wn * 2);
         a.stats = stats;
+        if(!set_bn(a, bn, y, ly))
+            return SAGA_HIP_EUNSUPPORTED;
         const int rc = launch_gather<false>(a, st);
         if(stats_rows)
             *stats_rows = a.stats_rows;
@@ -1500,6 +1575,8 @@ int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTe
         a.b_bytes = bb < 0x7fffff00 ? (unsigned)bb : 0;
     }
     a.stats = stats;
+    if(!set_bn(a, bn, y, ly))
+        return SAGA_HIP_EUNSUPPORTED;
     const int rc = launch_gather<false>(a, st);
     if(stats_rows)
         *stats_rows = a.stats_rows;
@@ -1541,6 +1618,7 @@ int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const 
         a.b_bytes = bb < 0x7fffff00 ? (unsigned)bb : 0;
     }
     a.stats = nullptr;
+    a.bn_s = nullptr;
     return launch_gather<true>(a, st);
 }
 

@@ -41,6 +41,8 @@ SIGNATURES = {
     "saga_hip_conv2d_fwd_bnstats_size": (_SZ, [_TV, _TV, _TV, C.POINTER(ConvParams)]),
     "saga_hip_conv2d_fwd_bnstats": (_I, [_TV, _TV, _TV, C.POINTER(ConvParams), _F, _VP, _SZ, _VP, _SZ,
                                          C.POINTER(C.c_int), _VP]),
+    "saga_hip_conv2d_fwd_bn_infer": (_I, [_TV, _TV, _TV, _TV, C.POINTER(ConvParams), _VP, _VP, _VP, _VP, _F, _I, _VP, _SZ,
+                                          _VP]),
     "saga_hip_conv2d_bwd_data": (_I, [_TV, _TV, _TV, C.POINTER(ConvParams), _F, _F, _VP, _SZ, _VP]),
     "saga_hip_conv2d_bwd_filter": (_I, [_TV, _TV, _TV, C.POINTER(ConvParams), _F, _F, _VP, _SZ, _VP]),
     "saga_hip_bias_add": (_I, [_TV, _TV, _VP]),

@@ -47,6 +47,11 @@ struct ConvFwd : public HipOperation {
     const SagaConvParams cp_;
     float beta_ = 0;
     std::shared_ptr<ConvStatsLink> stats_;
+    // inference: the batch norm that consumes y (with its residual and relu) runs in the epilogue
+    // and the result goes straight to the norm's output
+    T bn_s_, bn_b_, bn_m_, bn_v_, bn_z_, bn_y_;
+    float bn_eps_ = 0;
+    int bn_flags_ = 0;
     ConvFwd(HipProgram &p, T x, T w, T y, SagaConvParams cp) : HipOperation("convfwd"), x_(x), w_(w), y_(y), cp_(cp)
     {
         const SagaTensorView vx = x->shapeView(), vw = w->shapeView(), vy = y->shapeView();
@@ -65,8 +70,40 @@ struct ConvFwd : public HipOperation {
         stats_->partial = std::make_shared<HipMemory>(bytes);
         return stats_;
     }
+    bool foldBn(T s, T b, T m, T v, T z, T y, float eps, int flags)
+    {
+        if(stats_ || bn_y_ || x_->m_data_type != Tensor::DataType::HALF)
+            return false;
+        bn_s_ = s; bn_b_ = b; bn_m_ = m; bn_v_ = v; bn_z_ = z; bn_y_ = y;
+        bn_eps_ = eps;
+        bn_flags_ = flags;
+        m_kind = "convfwd.bn";
+        return true;
+    }
+    void execFolded(HipProgram &p)
+    {
+        const SagaTensorView vx = x_->view(), vw = w_->view(), vo = bn_y_->view();
+        SagaTensorView vz;
+        if(bn_z_)
+            vz = bn_z_->view();
+        const float *s = (const float *)bn_s_->deviceMem(), *b = (const float *)bn_b_->deviceMem();
+        const float *m = (const float *)bn_m_->deviceMem(), *v = (const float *)bn_v_->deviceMem();
+        const int r = saga_hip_conv2d_fwd_bn_infer(&vx, &vw, &vo, bn_z_ ? &vz : nullptr, &cp_, s, b, m, v, bn_eps_, bn_flags_,
+                                                   p.m_ctx->m_workspace.ptr(), p.m_ctx->m_workspace.size(), S(p));
+        if(r == 0)
+            return;
+        if(r != SAGA_HIP_EUNSUPPORTED)
+            chkSaga(r);
+        // two passes through the convolution's own output tensor
+        const SagaTensorView vy = y_->view();
+        chkSaga(saga_hip_conv2d_fwd(&vx, &vw, &vy, &cp_, 1.0f, 0.0f, p.m_ctx->m_workspace.ptr(),
+                                    p.m_ctx->m_workspace.size(), S(p)));
+        chkSaga(saga_hip_bn_infer(&vy, bn_z_ ? &vz : nullptr, &vo, s, b, m, v, bn_eps_, bn_flags_, S(p)));
+    }
     void exec(HipProgram &p) override
     {
+        if(bn_y_)
+            return execFolded(p);
         const SagaTensorView vx = x_->view(), vw = w_->view(), vy = y_->view();
         if(stats_) {
             stats_->valid = false;
@@ -85,11 +122,23 @@ struct ConvFwd : public HipOperation {
         chkSaga(saga_hip_conv2d_fwd(&vx, &vw, &vy, &cp_, 1.0f, beta_, p.m_ctx->m_workspace.ptr(),
                                     p.m_ctx->m_workspace.size(), S(p)));
     }
-    HipOpArgs listInputs() const override { return {{"x", x_}, {"w", w_}}; }
-    HipOpArgs listOutputs() const override { return {{"y", y_}}; }
-    float *getBeta(const T &t) override { return t == y_ ? &beta_ : nullptr; }
+    HipOpArgs listInputs() const override
+    {
+        HipOpArgs r{{"x", x_}, {"w", w_}};
+        if(bn_y_) {
+            r.insert(r.end(), {{"s", bn_s_}, {"b", bn_b_}, {"m", bn_m_}, {"v", bn_v_}});
+            if(bn_z_)
+                r.push_back({"z", bn_z_});
+        }
+        return r;
+    }
+    HipOpArgs listOutputs() const override { return {{"y", bn_y_ ? bn_y_ : y_}}; }
+    float *getBeta(const T &t) override { return !bn_y_ && t == y_ ? &beta_ : nullptr; }
     double flops() const override { return conv_flops(x_, w_, y_, cp_.group); }
-    double bytes() const override { return nbytes(x_) + nbytes(w_) + nbytes(y_) * (beta_ != 0 ? 2 : 1); }
+    double bytes() const override
+    {
+        return nbytes(x_) + nbytes(w_) + nbytes(y_) * (beta_ != 0 ? 2 : 1) + (bn_z_ ? nbytes(bn_z_) : 0);
+    }
 };
 
 struct ConvBwdData : public HipOperation {
@@ -726,6 +775,8 @@ struct BnBwd : public HipOperation {
     }
 };
 
+bool single_consumer(const Nodes &nodes, const std::shared_ptr<Tensor> &t);
+
 // x0 = normalised input, x1 = residual (optional); flags from the "relu" attribute
 void batchnorm_lower(HipProgram &p, HipProgramUnit &pu, const Node &n, std::shared_ptr<Tensor> xh,
                      std::shared_ptr<Tensor> zh, int flags)
@@ -742,15 +793,8 @@ void batchnorm_lower(HipProgram &p, HipProgramUnit &pu, const Node &n, std::shar
             throw std::runtime_error("batchnorm parameters must be fp32 vectors of C elements");
     const float eps = n.m_attributes.get("epsilon", 1e-5f);
 
-    if(p.m_pt == ProgramType::INFERENCE) {
-        pu.fwd(std::make_shared<BnInference>(x, z, s, b, m, v, y, eps, flags));
-        return;
-    }
-    auto sm = std::make_shared<HipTensor>(Tensor::DataType::FLOAT, *m, m->namePostfix("smean"));
-    auto sv = std::make_shared<HipTensor>(Tensor::DataType::FLOAT, *v, v->namePostfix("svar"));
-    auto f = std::make_shared<BnTrain>(p, x, z, s, b, m, v, y, sm, sv, eps, flags);
-    // if the op that wrote x last is a convolution and nothing else writes x, take the sums from it
-    {
+    // the operation that alone writes x, if it is a convolution
+    auto conv_producer = [&]() -> ConvFwd * {
         ConvFwd *producer = nullptr;
         int writers = 0;
         for(const auto &op : pu.m_fwd)
@@ -759,9 +803,25 @@ void batchnorm_lower(HipProgram &p, HipProgramUnit &pu, const Node &n, std::shar
                     writers++;
                     producer = o.second == x ? dynamic_cast<ConvFwd *>(op.get()) : nullptr;
                 }
-        if(writers == 1 && producer)
-            f->stats_ = producer->offerStats();
+        return writers == 1 ? producer : nullptr;
+    };
+    if(p.m_pt == ProgramType::INFERENCE) {
+        // conv -> batch norm with nobody else looking at the convolution's output: one kernel
+        ConvFwd *producer = conv_producer();
+        const auto &ex = p.m_ctx->m_exported;
+        const bool held = std::any_of(ex.begin(), ex.end(), [&](const auto &e) { return e == x->m_storage; });
+        if(producer && !held && !p.m_pc.disable_op_fusing && single_consumer(pu.m_transformed, xh) &&
+           producer->foldBn(s, b, m, v, z, y, eps, flags))
+            return;
+        pu.fwd(std::make_shared<BnInference>(x, z, s, b, m, v, y, eps, flags));
+        return;
     }
+    auto sm = std::make_shared<HipTensor>(Tensor::DataType::FLOAT, *m, m->namePostfix("smean"));
+    auto sv = std::make_shared<HipTensor>(Tensor::DataType::FLOAT, *v, v->namePostfix("svar"));
+    auto f = std::make_shared<BnTrain>(p, x, z, s, b, m, v, y, sm, sv, eps, flags);
+    // if the op that wrote x last is a convolution and nothing else writes x, take the sums from it
+    if(ConvFwd *producer = conv_producer())
+        f->stats_ = producer->offerStats();
     pu.fwd(f);
 
     auto dx = p.lowerGrad(pu, xh);

@@ -80,6 +80,39 @@ def test_conv_fwd_bwd(case, layout, padc, dtype):
     assert_close(host(dwd), 2 * dw_ref, dtype, "dw beta=1")
 
 
+@pytest.mark.parametrize("case", [(2, 64, 14, 64, 3, 1, 1, 3), (3, 32, 9, 160, 1, 0, 1, 1), (2, 128, 13, 24, 3, 1, 2, 0),
+                                  (2, 3, 30, 64, 7, 3, 2, 3), (2, 16, 8, 20, 3, 1, 1, 3)])
+def test_conv_with_folded_bn_inference(case):
+    """Convolution with the inference batch norm (+ residual + relu) in its epilogue against the two
+    separate operators of the oracle."""
+    N, Cc, H, Kk, R, pad, stride, flags = case
+    dtype = torch.float16
+    rng = np.random.default_rng(Cc * 5 + Kk)
+    x = rnd(rng, N, Cc, H, H, dtype=dtype)
+    w = rnd(rng, Kk, Cc, R, R, dtype=dtype, scale=(2.0 / (Cc * R * R)) ** 0.5)
+    y_conv = ref.round_half(ref.conv2d_fwd(x, w, pad, stride))
+    z = rnd(rng, *y_conv.shape, dtype=dtype)
+    s, b = (1 + 0.2 * rng.standard_normal(Kk)).astype(np.float32), (0.1 * rng.standard_normal(Kk)).astype(np.float32)
+    m, v = (0.3 * rng.standard_normal(Kk)).astype(np.float32), rng.uniform(0.5, 1.5, Kk).astype(np.float32)
+    want = ref.bn_infer(y_conv, s, b, m, v, 1e-5)
+    if flags & K.BN_ADD:
+        want = want + z
+    if flags & K.BN_RELU:
+        want = ref.act_fwd(want)
+    L = K.lib()
+    xd, wd, zd = dev(x, dtype, "nhwc"), dev(w, dtype, "nhwc"), dev(z, dtype, "nhwc")
+    yd = dev(np.zeros_like(y_conv), dtype, "nhwc")
+    sd, bd, md, vd = (dev(t) for t in (s, b, m, v))
+    p = K.ConvParams(pad, stride, 1, 1)
+    vx, vw, vy = K.view(xd), K.view(wd), K.view(yd)
+    ws = torch.zeros(max(1, L.saga_hip_conv2d_workspace_size(K.CONV_FWD, C.byref(vx), C.byref(vw), C.byref(vy),
+                                                             C.byref(p))), dtype=torch.uint8, device="cuda")
+    K.check(L.saga_hip_conv2d_fwd_bn_infer(C.byref(vx), C.byref(vw), C.byref(vy),
+                                           C.byref(K.view(zd)) if flags & K.BN_ADD else None, C.byref(p), K.ptr(sd),
+                                           K.ptr(bd), K.ptr(md), K.ptr(vd), 1e-5, flags, K.ptr(ws), ws.numel(), S()))
+    assert_close(host(yd), want, dtype, "conv+bn")
+
+
 BNSTATS_CASES = [
     # N, C, H, K, R, pad, stride, relu+add
     (2, 64, 14, 64, 3, 1, 1, False),
