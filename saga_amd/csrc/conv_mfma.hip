@@ -302,8 +302,8 @@ __device__ __forceinline__ void halve_exchange(float (&a)[NV], float (&b)[NV], i
     }
 }
 
-template <int BM, int BN, int WGM, int WGN, int STAGES, int BKT, bool BWD>
-__global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArgs g)
+template <int BM, int BN, int WGM, int WGN, int STAGES, int BKT, bool BWD, int PROD = 0>
+__global__ void __launch_bounds__(64 * (WGM * WGN + PROD), PROD ? (WGM * WGN + PROD + 3) / 4 : 1) conv_gather_gemm_dma(GatherArgs g)
 {
     constexpr int NW = WGM * WGN;                      // wavefronts per block
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
@@ -351,22 +351,13 @@ __global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArg
     const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void *)g.a, 0, g.a_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void *)g.b, 0, g.b_bytes, 0x00020000);
 
-    // this lane fills slot (tid % SLOTS) of row lrow (+RPR per round) and fetches the logical
-    // channel vector that the swizzle assigns to that slot
-    const int lrow = tid / SLOTS;
-    const int kv = ((tid % SLOTS) ^ swz_of(lrow)) * 8;
-
     // Address generation is hoisted out of the main loop: the input position of tap (ri, si)
     // is (iy0 + ri*sy, ix0 + si*sy), sy = dil forward and -1 backward (inside a residue class
     // consecutive taps are one input row / column apart), so a row's byte offset is
     // rowoff + a term that is the same for every lane (kept in scalar registers), and which
     // taps fall inside the image is one bit each of a 64-bit mask computed once per row.
     const int sy = BWD ? -1 : g.dil;
-    int rowoff[AV];
-    unsigned long long amask[AV];
-#pragma unroll
-    for(int j = 0; j < AV; j++) {
-        const int m = m0 + lrow + RPR * j;
+    auto row_setup = [&](int m, int kvv, int &ro, unsigned long long &mask) {
         bool ok = m < Mloc;
         const int mm = ok ? m : 0;
         const int ox = mm % PW;
@@ -383,7 +374,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArg
             iy0 = oy * g.stride - g.pad;
             ix0 = ox * g.stride - g.pad;
         }
-        rowoff[j] = (((n * g.IH + iy0) * g.IW + ix0) * g.lda + kv) * 2;
+        ro = (((n * g.IH + iy0) * g.IW + ix0) * g.lda + kvv) * 2;
         unsigned long long mk = 0;
         if(ok)
             for(int a = 0; a < nr; a++) {
@@ -396,21 +387,109 @@ __global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArg
                         mk |= 1ull << (a * ns + b);
                 }
             }
-        amask[j] = mk;
-    }
+        mask = mk;
+    };
     const int ktot = g.R * g.S * g.Cred;
-    int b_off[BV];
-    bool b_ok[BV];
-#pragma unroll
-    for(int j = 0; j < BV; j++) {
-        const int n = n0 + lrow + RPR * j;
-        b_ok[j] = n < g.Ngemm;
-        b_off[j] = ((b_ok[j] ? n : 0) * ktot + kv) * 2;
-    }
-
-    int ri = 0, si = 0, c0 = 0; // tap counters and channel offset of the NEXT slice to be issued
     const int csteps = (g.Cred + BKT - 1) / BKT;
     const int KT = nr * ns * csteps;
+    int ri = 0, si = 0, c0 = 0; // tap counters and channel offset of the NEXT slice to be issued
+    auto advance = [&]() {
+        c0 += BKT;
+        if(c0 >= g.Cred) {
+            c0 = 0;
+            if(++si == ns) {
+                si = 0;
+                ++ri;
+            }
+        }
+    };
+
+    // With PROD > 0 the block has PROD extra wavefronts that do nothing but issue the loads:
+    // a load-to-LDS instruction holds its wavefront at issue until the memory pipeline takes
+    // it, and in a wavefront that also feeds the matrix unit that wait is lost matrix time.
+    // Producers and consumers meet at one barrier per reduction slice: after barrier kt
+    // slice kt is in LDS and the stage of slice kt-1 is free for slice kt+STAGES-1.
+    if constexpr(PROD > 0) {
+        static_assert(BKT == 32 && (BM / 16) % PROD == 0 && (BN / 16) % PROD == 0, "producer split");
+        if(wave >= NW) {
+            constexpr int PA = BM / 16 / PROD, PB = BN / 16 / PROD; // 16-row pieces per producer
+            const int pw = wave - NW;
+            const int prow = lane >> 2;
+            const int pkv = ((lane & 3) ^ swz_of(prow)) * 8;
+            int ro[PA], bo[PB];
+            unsigned long long mk[PA];
+            bool bok[PB];
+#pragma unroll
+            for(int i = 0; i < PA; i++)
+                row_setup(m0 + (pw * PA + i) * 16 + prow, pkv, ro[i], mk[i]);
+#pragma unroll
+            for(int i = 0; i < PB; i++) {
+                const int n = n0 + (pw * PB + i) * 16 + prow;
+                bok[i] = n < g.Ngemm;
+                bo[i] = ((bok[i] ? n : 0) * ktot + pkv) * 2;
+            }
+            auto produce = [&](int stage) {
+                char *sa = smem + stage * STAGE_BYTES + pw * PA * 16 * ROWB;
+                char *sb = smem + stage * STAGE_BYTES + BM * ROWB + pw * PB * 16 * ROWB;
+                const bool cok = c0 + pkv < g.Cred;
+                const int tapoff = ((ri * g.IW + si) * sy * g.lda + c0) * 2; // same for all lanes
+                const int tap = ri * ns + si;
+#pragma unroll
+                for(int i = 0; i < PA; i++) {
+                    const bool ok = cok && ((mk[i] >> tap) & 1);
+                    const unsigned off = ok ? (unsigned)(ro[i] + tapoff) : OOB;
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(sa + i * 16 * ROWB), 16, off, 0, 0, 0);
+                }
+                const int r = r0 + ri * rstep, s = s0 + si * rstep;
+                const int kb = ((r * g.S + s) * g.Cred + c0) * 2;
+#pragma unroll
+                for(int i = 0; i < PB; i++) {
+                    const unsigned off = (bok[i] && cok) ? (unsigned)(bo[i] + kb) : OOB;
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(sb + i * 16 * ROWB), 16, off, 0, 0, 0);
+                }
+                advance();
+            };
+#pragma unroll
+            for(int st = 0; st < STAGES - 1; st++)
+                if(st < KT)
+                    produce(st);
+            for(int kt = 0; kt < KT; kt++) {
+                if(kt + STAGES - 2 < KT)
+                    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((PA + PB) * (STAGES - 2)) : "memory");
+                else
+                    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+                if(kt + STAGES - 1 < KT)
+                    produce((kt + STAGES - 1) % STAGES);
+            }
+            if constexpr(!BWD) {
+                if(g.stats) { // the two barriers of the statistics epilogue
+                    __syncthreads();
+                    __syncthreads();
+                }
+            }
+            return;
+        }
+    }
+
+    // (PROD == 0) this lane fills slot (tid % SLOTS) of row lrow (+RPR per round) and fetches
+    // the logical channel vector that the swizzle assigns to that slot
+    const int lrow = tid / SLOTS;
+    const int kv = ((tid % SLOTS) ^ swz_of(lrow)) * 8;
+    int rowoff[AV];
+    unsigned long long amask[AV];
+    int b_off[BV];
+    bool b_ok[BV];
+    if constexpr(PROD == 0) {
+#pragma unroll
+        for(int j = 0; j < AV; j++)
+            row_setup(m0 + lrow + RPR * j, kv, rowoff[j], amask[j]);
+#pragma unroll
+        for(int j = 0; j < BV; j++) {
+            const int n = n0 + lrow + RPR * j;
+            b_ok[j] = n < g.Ngemm;
+            b_off[j] = ((b_ok[j] ? n : 0) * ktot + kv) * 2;
+        }
+    }
 
     // one slice = AV + BV load instructions ("pieces"); issue_piece(stage, p) emits piece p of
     // the next slice, advance() steps the slice cursor once all its pieces are out
@@ -430,16 +509,6 @@ __global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArg
             const int kb = ((r * g.S + s) * g.Cred + c0) * 2;
             const unsigned off = (b_ok[j] && cok) ? (unsigned)(b_off[j] + kb) : OOB;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(sb + (j * RPR + wave * RPI) * ROWB), 16, off, 0, 0, 0);
-        }
-    };
-    auto advance = [&]() {
-        c0 += BKT;
-        if(c0 >= g.Cred) {
-            c0 = 0;
-            if(++si == ns) {
-                si = 0;
-                ++ri;
-            }
         }
     };
     auto issue = [&](int stage) {
@@ -468,20 +537,24 @@ __global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArg
     for(int kk = 0; kk < KS; kk++)
         fo[kk] = ((2 * kk + (lane >> 5)) ^ swz) * 16;
 
+    if constexpr(PROD == 0) {
 #pragma unroll
-    for(int st = 0; st < STAGES - 1; st++)
-        if(st < KT)
-            issue(st);
+        for(int st = 0; st < STAGES - 1; st++)
+            if(st < KT)
+                issue(st);
+    }
 
-    constexpr int NP = AV + BV, NQ = KS * TM * TN; // load pieces and MFMAs per iteration
+    constexpr int NP = PROD ? 0 : AV + BV, NQ = KS * TM * TN; // load pieces and MFMAs per iteration
     for(int kt = 0; kt < KT; kt++) {
         // oldest outstanding slice = kt; newer ones may stay in flight
         // (a plain __syncthreads() would make the compiler drain every outstanding load)
-        if(kt + STAGES - 2 < KT)
+        if constexpr(PROD > 0)
+            asm volatile("s_barrier" ::: "memory");
+        else if(kt + STAGES - 2 < KT)
             asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(NP * (STAGES - 2)) : "memory");
         else
             asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-        const bool more = kt + STAGES - 1 < KT;
+        const bool more = !PROD && kt + STAGES - 1 < KT;
         const int nst = (kt + STAGES - 1) % STAGES;
         const char *sa = smem + (kt % STAGES) * STAGE_BYTES;
         const char *sb = sa + BM * ROWB;
@@ -503,7 +576,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) conv_gather_gemm_dma(GatherArg
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk][j], fa[kk][i], acc[i][j], 0, 0, 0);
 #pragma unroll
             for(int p = 0; p < NP; p++)
-                if(q == (p * NQ) / NP) {
+                if(q == (p * NQ) / (NP ? NP : 1)) {
                     __builtin_amdgcn_sched_barrier(0);
                     if(more)
                         issue_piece(nst, p);
@@ -1352,11 +1425,17 @@ template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
         // wavefronts on nearly every ResNet-50 layer, and faster than the same tiles with
         // 64-wide reduction slices (which leave room for one block per CU only)
         int tile = tile_override();
-        if(tile < 0)
+        if(tile < 0) {
             tile = g.Ngemm <= 64 ? 3 : 5;
-#define LAUNCH(BM, BN, WGM, WGN, BKT)                                                                  \
+            // at most one block per CU: nothing else on the CU hides the time a wavefront spends
+            // issuing its loads, so four extra wavefronts per block do the issuing (measured
+            // 5-15 % faster on the 7x7-pixel layers of ResNet-50, slower once CUs hold two blocks)
+            if(tile == 5 && (int64_t)((g.Mc + 255) / 256) * ((g.Ngemm + 127) / 128) * active <= 256)
+                tile = 12;
+        }
+#define LAUNCH(BM, BN, WGM, WGN, BKT, PROD)                                                            \
     do {                                                                                               \
-        auto kern = conv_gather_gemm_dma<BM, BN, WGM, WGN, ST, BKT, BWD>;                               \
+        auto kern = conv_gather_gemm_dma<BM, BN, WGM, WGN, ST, BKT, BWD, PROD>;                         \
         constexpr int lds = ST * (BM + BN) * BKT * 2;                                                  \
         static bool once = false;                                                                      \
         if(lds > 64 * 1024 && !once) {                                                                 \
@@ -1370,12 +1449,13 @@ template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
         g.nblocks = g.blocks_per_class * active;                                                       \
         g.nactive = active;                                                                            \
         g.stats_rows = (g.Mc + BM - 1) / BM;                                                           \
-        kern<<<g.nblocks, 64 * WGM * WGN, lds, st>>>(g);                                               \
+        kern<<<g.nblocks, 64 * (WGM * WGN + PROD), lds, st>>>(g);                                      \
     } while(0)
         switch(tile) {
-        case 2: LAUNCH(128, 128, 2, 2, 32); break;
-        case 5: LAUNCH(256, 128, 4, 2, 32); break;
-        default: LAUNCH(256, 64, 4, 1, 32); break;
+        case 2: LAUNCH(128, 128, 2, 2, 32, 0); break;
+        case 5: LAUNCH(256, 128, 4, 2, 32, 0); break;
+        case 12: LAUNCH(256, 128, 4, 2, 32, 4); break;
+        default: LAUNCH(256, 64, 4, 1, 32, 0); break;
         }
 #undef LAUNCH
         SAGA_CHECK_LAUNCH();
