@@ -62,6 +62,8 @@ int saga_tensor_write(saga_tensor_t t, const void *data, size_t bytes);
 int saga_tensor_read(saga_tensor_t t, void *data, size_t bytes);
 int saga_tensor_save(saga_tensor_t t, const char *path);
 saga_tensor_t saga_tensor_load(const char *path, const char *name);
+/* a file holding one ONNX TensorProto (Tensor::loadProtoBuf, reference src/onnx.cpp:777-790); NULL on failure */
+saga_tensor_t saga_tensor_load_protobuf(const char *path);
 double saga_tensor_sse(saga_tensor_t a, saga_tensor_t b);
 
 saga_graph_t saga_graph_create(void);
@@ -71,6 +73,14 @@ saga_node_t saga_graph_add_node(saga_graph_t g, const char *type, int n_inputs, 
 saga_node_t saga_graph_add_resnet_bottleneck(saga_graph_t g, saga_tensor_t input, int squeeze, int output,
                                              int downsample, const char *name);
 saga_node_t saga_graph_add_resnet(saga_graph_t g, saga_tensor_t input, int output, int downsample, const char *name);
+/* ONNX model file -> graph (Graph::load, reference saga.hpp / src/onnx.cpp:750-775); NULL on failure */
+saga_graph_t saga_graph_load(const char *path);
+/* graph inputs (outputs != 0: outputs) in name order */
+int saga_graph_io_count(saga_graph_t g, int outputs);
+saga_tensor_t saga_graph_io(saga_graph_t g, int outputs, int index);
+/* one text line per node: "type | slot=name:dtype[dims] ... | attr=value ... | slot=name:dtype[dims]";
+   returns the length of the full text, writes at most capacity-1 characters plus a terminator */
+int saga_graph_describe(saga_graph_t g, char *buf, size_t capacity);
 int saga_graph_node_count(saga_graph_t g);
 int saga_graph_save_tensors(saga_graph_t g, const char *path, saga_context_t ctx);
 int saga_graph_load_tensors(saga_graph_t g, const char *path);

@@ -64,6 +64,11 @@ SIGNATURES = {
     "saga_graph_add_resnet_bottleneck": (_VP, [_VP, _VP, C.c_int, C.c_int, C.c_int, C.c_char_p]),
     "saga_graph_add_resnet": (_VP, [_VP, _VP, C.c_int, C.c_int, C.c_char_p]),
     "saga_graph_node_count": (C.c_int, [_VP]),
+    "saga_graph_load": (_VP, [C.c_char_p]),
+    "saga_graph_io_count": (C.c_int, [_VP, C.c_int]),
+    "saga_graph_io": (_VP, [_VP, C.c_int, C.c_int]),
+    "saga_graph_describe": (C.c_int, [_VP, C.c_char_p, C.c_size_t]),
+    "saga_tensor_load_protobuf": (_VP, [C.c_char_p]),
     "saga_graph_save_tensors": (C.c_int, [_VP, C.c_char_p, _VP]),
     "saga_graph_load_tensors": (C.c_int, [_VP, C.c_char_p]),
     "saga_graph_named_tensor": (_VP, [_VP, C.c_char_p]),
@@ -174,6 +179,14 @@ class Tensor:
     def load(cls, path, name=None):
         return cls(lib().saga_tensor_load(path.encode(), _name(name)))
 
+    @classmethod
+    def load_protobuf(cls, path):
+        """Tensor::loadProtoBuf: a file holding one ONNX TensorProto."""
+        h = lib().saga_tensor_load_protobuf(path.encode())
+        if not h:
+            raise _err("loadProtoBuf")
+        return cls(h)
+
     def sse(self, other):
         return lib().saga_tensor_sse(self._h, other._h)
 
@@ -232,8 +245,30 @@ class Dims(list):
 
 
 class Graph:
-    def __init__(self):
-        self._h = lib().saga_graph_create()
+    def __init__(self, handle=None):
+        self._h = handle or lib().saga_graph_create()
+
+    @classmethod
+    def load(cls, path):
+        """Graph::load: an ONNX model file."""
+        h = lib().saga_graph_load(path.encode())
+        if not h:
+            raise _err("Graph::load")
+        return cls(h)
+
+    def inputs(self):
+        """Graph inputs (tensors no node produces and no initializer fills), in name order."""
+        return [Tensor(lib().saga_graph_io(self._h, 0, i)) for i in range(lib().saga_graph_io_count(self._h, 0))]
+
+    def outputs(self):
+        return [Tensor(lib().saga_graph_io(self._h, 1, i)) for i in range(lib().saga_graph_io_count(self._h, 1))]
+
+    def describe(self):
+        """One line per node: type | inputs | attributes | outputs."""
+        n = lib().saga_graph_describe(self._h, None, 0)
+        buf = C.create_string_buffer(n + 1)
+        lib().saga_graph_describe(self._h, buf, n + 1)
+        return buf.value.decode().splitlines()
 
     def __del__(self):
         try:

@@ -2,6 +2,7 @@
 // (the Python tests and bench.py bind it with ctypes).  Declarations: include/saga_capi.h.
 #include <string.h>
 
+#include <algorithm>
 #include <mutex>
 
 #include "saga.hpp"
@@ -236,6 +237,78 @@ saga_node_t saga_graph_add_resnet(saga_graph_t g, saga_tensor_t input, int outpu
     saga_node_t r = nullptr;
     guard([&] { r = new NodeBox{((GraphBox *)g)->g.addResNet(((TensorBox *)input)->t, output, downsample != 0, name)}; });
     return r;
+}
+
+saga_graph_t saga_graph_load(const char *path)
+{
+    auto g = Graph::load(path);
+    if(!g) {
+        g_error = std::string("unable to load ") + path;
+        return nullptr;
+    }
+    return new GraphBox{*g};
+}
+
+saga_tensor_t saga_tensor_load_protobuf(const char *path)
+{
+    auto t = Tensor::loadProtoBuf(path);
+    if(!t) {
+        g_error = std::string("unable to load ") + path;
+        return nullptr;
+    }
+    return box(t);
+}
+
+// graph inputs / outputs in name order (the sets themselves have no order)
+static std::vector<std::shared_ptr<Tensor>> sorted_io(saga_graph_t g, int outputs)
+{
+    auto &set = outputs ? ((GraphBox *)g)->g.m_outputs : ((GraphBox *)g)->g.m_inputs;
+    std::vector<std::shared_ptr<Tensor>> v(set.begin(), set.end());
+    std::sort(v.begin(), v.end(), [](const std::shared_ptr<Tensor> &a, const std::shared_ptr<Tensor> &b) {
+        return a->m_name.value_or("") < b->m_name.value_or("");
+    });
+    return v;
+}
+
+int saga_graph_io_count(saga_graph_t g, int outputs) { return (int)sorted_io(g, outputs).size(); }
+
+saga_tensor_t saga_graph_io(saga_graph_t g, int outputs, int index)
+{
+    const auto v = sorted_io(g, outputs);
+    return index >= 0 && index < (int)v.size() ? box(v[index]) : nullptr;
+}
+
+int saga_graph_describe(saga_graph_t g, char *buf, size_t capacity)
+{
+    std::string out;
+    auto slots = [&](const Tensors &ts) {
+        std::vector<std::string> names;
+        for(const auto &t : ts)
+            names.push_back(t.first);
+        std::sort(names.begin(), names.end());
+        std::string r;
+        for(const auto &n : names) {
+            const auto &t = ts.find(n)->second;
+            r += (r.empty() ? "" : " ") + n + "=" + (t ? t->m_name.value_or("?") + ":" + Tensor::DataTypeStr(t->m_data_type) + t->m_dims.to_string() : "null");
+        }
+        return r;
+    };
+    for(const auto &n : ((GraphBox *)g)->g.m_nodes) {
+        std::vector<std::string> an;
+        for(const auto &a : n->m_attributes)
+            an.push_back(a.first);
+        std::sort(an.begin(), an.end());
+        std::string attrs;
+        for(const auto &a : an)
+            attrs += (attrs.empty() ? "" : " ") + a + "=" + n->m_attributes.find(a)->second.to_string();
+        out += n->m_type + " | " + slots(n->m_inputs) + " | " + attrs + " | " + slots(n->m_outputs) + "\n";
+    }
+    if(buf && capacity) {
+        const size_t c = std::min(capacity - 1, out.size());
+        memcpy(buf, out.data(), c);
+        buf[c] = 0;
+    }
+    return (int)out.size();
 }
 
 int saga_graph_node_count(saga_graph_t g) { return (int)((GraphBox *)g)->g.m_nodes.size(); }

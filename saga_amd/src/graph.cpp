@@ -93,12 +93,6 @@ std::shared_ptr<Node> Graph::addNode(const std::string &type, Loader loader, con
     return m_nodes.empty() ? nullptr : m_nodes.back();
 }
 
-std::shared_ptr<Graph> Graph::load(const char *path)
-{
-    fprintf(stderr, "Unable to load %s -- the ONNX loader is not part of this build\n", path);
-    return nullptr;
-}
-
 // tensors consumed but never produced / produced but never consumed
 std::unordered_set<std::shared_ptr<Tensor>> Graph::inputTensors() const
 {

@@ -946,17 +946,29 @@ struct Transform : public HipOperation {
     double bytes() const override { return (beta_ != 0 ? 3 : 2) * nbytes(b_); }
 };
 
+// y = x0 + x1 (+ x2 ...).  The reference reads x0 and x1 only (cuda_dnn.cpp:1883-1890) although
+// its ONNX loader attaches every input of an n-ary Sum (onnx.cpp:540-553); here all of them are added.
 void sum_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
 {
-    auto x0 = p.lower(pu, n.m_inputs["x0"]);
-    auto x1 = p.lower(pu, n.m_inputs["x1"]);
-    auto y = p.lowerLike(pu, n.m_outputs["y"], *x0);
-    pu.fwd(std::make_shared<AddOp>(x0, x1, y));
+    const auto xh = n.m_inputs.getv("x");
+    if(xh.empty())
+        throw std::runtime_error("sum without inputs");
+    std::vector<T> xs;
+    for(const auto &h : xh)
+        xs.push_back(p.lower(pu, h));
+    auto y = p.lowerLike(pu, n.m_outputs["y"], *xs[0]);
+    if(xs.size() == 1)
+        pu.fwd(std::make_shared<Transform>(xs[0], y));
+    else
+        pu.fwd(std::make_shared<AddOp>(xs[0], xs[1], y));
+    // further writers of y: the program gives every writer after the first beta = 1 (y += x)
+    for(size_t i = 2; i < xs.size(); i++)
+        pu.fwd(std::make_shared<Transform>(xs[i], y));
     if(p.m_pt == ProgramType::INFERENCE)
         return;
     auto dy = p.lowerGrad(pu, n.m_outputs["y"]);
-    pu.bwd(std::make_shared<Transform>(dy, p.lowerGrad(pu, n.m_inputs["x0"])));
-    pu.bwd(std::make_shared<Transform>(dy, p.lowerGrad(pu, n.m_inputs["x1"])));
+    for(const auto &h : xh)
+        pu.bwd(std::make_shared<Transform>(dy, p.lowerGrad(pu, h)));
 }
 REGISTER_HIP_OP("sum", sum_setup);
 

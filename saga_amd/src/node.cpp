@@ -231,13 +231,19 @@ void loss_prepare(std::shared_ptr<Node> n, std::shared_ptr<Tensor> x, Tensors &,
 // ---- sum: operands must agree in type and shape (reference: src/node.cpp:372-389)
 std::shared_ptr<Tensor> sum_infer(const Node &n, const Name &name)
 {
-    auto a = n.m_inputs["x0"], b = n.m_inputs["x1"];
-    if(a->m_data_type != b->m_data_type)
-        throw std::runtime_error(fmt("x0 datatype %s != x1 datatype %s", Tensor::DataTypeStr(a->m_data_type),
-                                     Tensor::DataTypeStr(b->m_data_type)));
-    if(a->m_dims != b->m_dims)
-        throw std::runtime_error(fmt("x0 dimensions %s != x1 dimensions %s", a->m_dims.to_string().c_str(),
-                                     b->m_dims.to_string().c_str()));
+    const auto xs = n.m_inputs.getv("x");
+    if(xs.empty())
+        throw std::runtime_error("sum without inputs");
+    auto a = xs[0];
+    for(size_t i = 1; i < xs.size(); i++) {
+        auto b = xs[i];
+        if(a->m_data_type != b->m_data_type)
+            throw std::runtime_error(fmt("x0 datatype %s != x%zu datatype %s", Tensor::DataTypeStr(a->m_data_type), i,
+                                         Tensor::DataTypeStr(b->m_data_type)));
+        if(a->m_dims != b->m_dims)
+            throw std::runtime_error(fmt("x0 dimensions %s != x%zu dimensions %s", a->m_dims.to_string().c_str(), i,
+                                         b->m_dims.to_string().c_str()));
+    }
     return makeTensor(a->m_data_type, a->m_dims, name);
 }
 

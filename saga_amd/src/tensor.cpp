@@ -327,12 +327,6 @@ void Tensor::printRGB(const char *, std::optional<std::pair<float, float>>)
     throw std::runtime_error("printRGB: image debugging helpers are not part of this build");
 }
 
-std::shared_ptr<Tensor> Tensor::loadProtoBuf(const char *path)
-{
-    fprintf(stderr, "Unable to load %s -- protobuf tensors are not supported by this build\n", path);
-    return nullptr;
-}
-
 // ---------------------------------------------------------------- placeholders + autograd link
 
 static std::mutex g_autograd_mutex;
