@@ -10,7 +10,8 @@
 //
 // Differences from the reference: malformed files, unknown operators and unsupported
 // attribute combinations make Graph::load print the reason and return nullptr (the reference
-// asserts or aborts); fp16 / u8 tensors stored in int32_data are accepted as well.
+// asserts or aborts); fp16 / u8 tensors stored in int32_data are accepted as well; FLOAT16
+// BatchNormalization parameters are widened to fp32 (the batchnorm node takes fp32 parameters).
 #include <fcntl.h>
 #include <string.h>
 #include <sys/mman.h>
@@ -527,6 +528,26 @@ struct Builder {
         return finish(n);
     }
 
+    // The batchnorm node takes fp32 scale / bias / mean / variance whatever the type of x (as
+    // cuDNN does for the reference's backend); fp16 models store them as FLOAT16, so those
+    // initializers are widened once, here, on the host.
+    static std::shared_ptr<Tensor> widened(std::shared_ptr<Tensor> t)
+    {
+        if(t->m_data_type != Tensor::DataType::HALF)
+            return t;
+        auto src = t->access();
+        if(!src)
+            return t;
+        auto w = makeCPUTensor(Tensor::DataType::FLOAT, t->m_dims, t->m_name);
+        auto dst = w->access();
+        const int n = (int)t->m_dims.elements();
+        if(t->m_dims.size() != 1)
+            throw std::runtime_error("ONNX BatchNormalization: parameters must be vectors");
+        for(int i = 0; i < n; i++)
+            dst->set({i}, src->get({i}));
+        return w;
+    }
+
     // reference: make_batchnorm, src/onnx.cpp:424-443
     std::shared_ptr<Node> batchnorm() const
     {
@@ -534,7 +555,7 @@ struct Builder {
         auto n = std::make_shared<Node>("batchnorm");
         static const char *slots[] = {"x", "s", "b", "m", "v"};
         for(int i = 0; i < 5; i++)
-            n->m_inputs[slots[i]] = in(i);
+            n->m_inputs[slots[i]] = i ? widened(in(i)) : in(i);
         n->m_attributes["epsilon"] = np.attribs.get("epsilon", 1e-05f);
         return finish(n);
     }

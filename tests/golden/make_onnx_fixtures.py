@@ -241,6 +241,44 @@ class MiniVGG(nn.Module):
         return self.classifier(torch.flatten(self.features(x), 1))
 
 
+class Bottleneck(nn.Module):
+    def __init__(self, cin, mid, cout, stride):
+        super().__init__()
+        self.c1, self.b1 = nn.Conv2d(cin, mid, 1, bias=False), nn.BatchNorm2d(mid)
+        self.c2, self.b2 = nn.Conv2d(mid, mid, 3, stride, 1, bias=False), nn.BatchNorm2d(mid)  # v1.5: stride here
+        self.c3, self.b3 = nn.Conv2d(mid, cout, 1, bias=False), nn.BatchNorm2d(cout)
+        self.proj = None
+        if stride != 1 or cin != cout:
+            self.proj = nn.Sequential(nn.Conv2d(cin, cout, 1, stride, bias=False), nn.BatchNorm2d(cout))
+
+    def forward(self, x):
+        y = F.relu(self.b1(self.c1(x)))
+        y = F.relu(self.b2(self.c2(y)))
+        y = self.b3(self.c3(y))
+        return F.relu(y + (x if self.proj is None else self.proj(x)))
+
+
+class ResNet50(nn.Module):
+    """ResNet-50 v1.5 with the operator sequence of the model zoo's resnet50-v1-12.onnx; used at full
+    size by the GPU test, which exports it into a temporary directory (too large for a fixture)."""
+
+    def __init__(self, classes=1000):
+        super().__init__()
+        self.stem = nn.Sequential(nn.Conv2d(3, 64, 7, 2, 3, bias=False), nn.BatchNorm2d(64), nn.ReLU(),
+                                  nn.MaxPool2d(3, 2, 1))
+        layers, cin = [], 64
+        for mid, n, stride in [(64, 3, 1), (128, 4, 2), (256, 6, 2), (512, 3, 2)]:
+            for i in range(n):
+                layers.append(Bottleneck(cin, mid, mid * 4, stride if i == 0 else 1))
+                cin = mid * 4
+        self.layers = nn.Sequential(*layers)
+        self.pool = nn.AdaptiveAvgPool2d(1)
+        self.fc = nn.Linear(2048, classes)
+
+    def forward(self, x):
+        return self.fc(torch.flatten(self.pool(self.layers(self.stem(x))), 1))
+
+
 def torch_cases():
     cases = [("mini_resnet", MiniResNet, (2, 3, 16, 16)), ("mini_squeezenet", MiniSqueezeNet, (2, 3, 35, 35)),
              ("mini_vgg", MiniVGG, (2, 3, 16, 16))]
