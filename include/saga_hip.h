@@ -203,6 +203,13 @@ int saga_hip_convert(const SagaTensorView *src, const SagaTensorView *dst, float
 /* softmax over C at every (n,h,w): cudnnSoftmaxForward ACCURATE / MODE_CHANNEL (src/cuda/cuda_dnn.cpp:1937-1945). */
 int saga_hip_softmax(const SagaTensorView *x, const SagaTensorView *y, saga_stream_t stream);
 
+/* y[n,c,h,w] = bilinear sample of x[n,c] at theta[n] (2x3, row major, fp32 [N,2,3] on the device) applied to
+ * the normalised output coordinate; samples outside x count as zero.  Forward only.
+ * cudnnSpatialTfGridGeneratorForward + cudnnSpatialTfSamplerForward, CUDNN_SAMPLER_BILINEAR
+ * (src/cuda/cuda_dnn.cpp:2372-2425). */
+int saga_hip_spatial_transform(const SagaTensorView *x, const float *theta, const SagaTensorView *y,
+                               saga_stream_t stream);
+
 /* ---- classifier head: catclassifier_fwd / catclassifier_bwd (src/cuda/cuda_kernels.cu:11-96).
  *      x is [N,C] with contiguous rows; pred/labels are int32 [N]; loss fp32 [N] (may be NULL). */
 int saga_hip_catclassifier_fwd(const SagaTensorView *x, int32_t *pred, saga_stream_t stream);

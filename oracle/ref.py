@@ -243,6 +243,16 @@ def softmax(x):
     return y
 
 
+def spatial_transform(x, theta, oh, ow):
+    """x [N,C,H,W], theta [N,2,3] -> [N,C,oh,ow]"""
+    x, theta = _f(x), _f(theta)
+    N, Cc, H, W = x.shape
+    assert theta.shape == (N, 2, 3)
+    y = np.empty((N, Cc, oh, ow), np.float32)
+    lib().so_spatial_transform(_p(x), _p(theta), _p(y), _i(N), _i(Cc), _i(H), _i(W), _i(oh), _i(ow))
+    return y
+
+
 def catclassifier_fwd(x):
     x = _f(x)
     N, Cc = x.shape

@@ -26,6 +26,11 @@
  *   so_catclassifier_*             in-tree kernel src/cuda/cuda_kernels.cu:11-64 is the spec; closed forms
  *   so_adam_*                      in-tree kernel src/cuda/cuda_kernels.cu:159-230 is the spec; t=1 closed form
  *   so_softmax                     closed form, rows sum to one
+ *   so_spatial_transform           cuDNN's spatial transformer is third-party code outside the reference tree and
+ *                                  the reference holds no vectors for it; restated from cuDNN's published rule
+ *                                  (normalised coordinates, -1 / 1 = centres of the border pixels, zeros outside)
+ *                                  and pinned against torch's affine_grid + grid_sample(align_corners=True) on
+ *                                  the CPU, identity = copy, and the closed form for resizing a linear ramp
  */
 #include <math.h>
 #include <stdint.h>
@@ -597,6 +602,38 @@ void so_avgpool_bwd(const float *dy, float *dx, int N, int C, int H, int W, int 
         for(int i = 0; i < H * W; i++)
             o[i] = (float)(acc[i] + (beta != 0.0f ? (double)beta * o[i] : 0.0));
         free(acc);
+    }
+}
+
+/* ---------------------------------------------------------------- spatial transformer */
+
+/* affine grid + bilinear sampler, zeros outside (cudnnSpatialTfGridGeneratorForward +
+ * cudnnSpatialTfSamplerForward as called at src/cuda/cuda_dnn.cpp:2407-2416); theta is [N,2,3] */
+void so_spatial_transform(const float *x, const float *theta, float *y, int N, int C, int IH, int IW, int OH, int OW)
+{
+    for(int n = 0; n < N; n++) {
+        const float *t = theta + (size_t)n * 6;
+        for(int h = 0; h < OH; h++)
+            for(int w = 0; w < OW; w++) {
+                const double xt = OW > 1 ? -1.0 + 2.0 * w / (OW - 1) : -1.0;
+                const double yt = OH > 1 ? -1.0 + 2.0 * h / (OH - 1) : -1.0;
+                const double xs = t[0] * xt + t[1] * yt + t[2];
+                const double ys = t[3] * xt + t[4] * yt + t[5];
+                const double px = (xs + 1.0) * 0.5 * (IW - 1), py = (ys + 1.0) * 0.5 * (IH - 1);
+                const double fx = floor(px), fy = floor(py);
+                const double ax = px - fx, ay = py - fy;
+                for(int c = 0; c < C; c++) {
+                    double v = 0;
+                    for(int dy = 0; dy < 2; dy++)
+                        for(int dx = 0; dx < 2; dx++) {
+                            const double yy = fy + dy, xx = fx + dx;
+                            if(yy < 0 || yy >= IH || xx < 0 || xx >= IW)
+                                continue;
+                            v += (dx ? ax : 1.0 - ax) * (dy ? ay : 1.0 - ay) * x[IDX4(n, c, (int)yy, (int)xx, C, IH, IW)];
+                        }
+                    y[IDX4(n, c, h, w, C, OH, OW)] = (float)v;
+                }
+            }
     }
 }
 

@@ -64,6 +64,7 @@ SIGNATURES = {
     "saga_hip_axpby": (_I, [_TV, _TV, _F, _F, _VP]),
     "saga_hip_convert": (_I, [_TV, _TV, _F, _VP]),
     "saga_hip_softmax": (_I, [_TV, _TV, _VP]),
+    "saga_hip_spatial_transform": (_I, [_TV, _VP, _TV, _VP]),
     "saga_hip_catclassifier_fwd": (_I, [_TV, _VP, _VP]),
     "saga_hip_catclassifier_bwd": (_I, [_TV, _TV, _VP, _VP, _VP, _F, _VP]),
     "saga_hip_adam_f32": (_I, [_SZ, _VP, _VP, _VP, _VP, _F, _F, _F, _F, _VP, _VP]),

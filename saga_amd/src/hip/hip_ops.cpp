@@ -601,7 +601,7 @@ void catclassifier_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
         loss = std::make_shared<HipTensor>(Tensor::DataType::FLOAT, ld, HipLayout::NCHW, p.m_ctx.get(), lh->m_name);
         p.m_ctx->m_tensors[lh] = loss;
     }
-    if((int)loss->m_dims.elements() < (int)x->m_dims[0])
+    if(std::max<size_t>(loss->m_dims.elements(), loss->m_storage->m_elements) < (size_t)(int)x->m_dims[0])
         throw std::runtime_error("catclassifier: loss tensor smaller than the batch");
     pu.bwd(std::make_shared<CatClassifierBwd>(x, y, dx, dy, loss));
 }
@@ -1026,6 +1026,56 @@ void softmax_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
     pu.fwd(std::make_shared<Softmax>(x, y));
 }
 REGISTER_HIP_OP("softmax", softmax_setup);
+
+// ---------------------------------------------------------------- spatial transform
+// Affine grid + bilinear sampler, forward only (reference: CudnnSpatialTransformFwd and
+// spatialtransform_setup, :2372-2460).  The kernel samples fp16 and fp32 tensors directly, so the
+// convert -> transform -> convert sandwich the reference builds for non-float inputs (:2462-2500)
+// is not needed: the arithmetic (fp32 mix of exactly converted inputs, rounded once) is the same.
+
+struct SpatialTransform : public HipOperation {
+    const T x_, theta_, y_;
+    SpatialTransform(T x, T theta, T y) : HipOperation("spatialtransform"), x_(x), theta_(theta), y_(y) {}
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vx = x_->view(), vy = y_->view();
+        chkSaga(saga_hip_spatial_transform(&vx, (const float *)theta_->deviceMem(), &vy, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"x", x_}, {"theta", theta_}}; }
+    HipOpArgs listOutputs() const override { return {{"y", y_}}; }
+    double bytes() const override { return nbytes(x_) + nbytes(y_); }
+};
+
+void spatialtransform_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
+{
+    auto x = p.lower(pu, n.m_inputs["x"]);
+    auto y = p.lower(pu, n.m_outputs["y"]);
+    // during inference the transform is a plain resize unless the node asks otherwise
+    const bool disable = p.m_pt == ProgramType::INFERENCE && !n.m_attributes.get("inference", false);
+    if(disable && x->m_dims == y->m_dims) {
+        pu.fwd(std::make_shared<Transform>(x, y));
+        return;
+    }
+    auto th = n.m_inputs.has("theta") ? n.m_inputs["theta"] : nullptr;
+    if(disable || !th) {
+        th = makeCPUTensor(Tensor::DataType::FLOAT, Dims{(int64_t)pu.m_batch_size, (int64_t)2, (int64_t)3},
+                           "theta.identity");
+        auto ta = th->access();
+        for(int i = 0; i < pu.m_batch_size; i++) {
+            ta->set({i, 0, 0}, 1);
+            ta->set({i, 1, 1}, 1);
+        }
+    }
+    auto theta = p.lower(pu, th);
+    if(theta->m_data_type != Tensor::DataType::FLOAT || theta->m_dims.elements() != (size_t)(int)x->m_dims[0] * 6 ||
+       !theta->rowMajor())
+        throw std::runtime_error("spatialtransform: theta must be an fp32 [N,2,3] tensor");
+    if(x->m_data_type != y->m_data_type ||
+       (x->m_data_type != Tensor::DataType::FLOAT && x->m_data_type != Tensor::DataType::HALF))
+        throw std::runtime_error("spatialtransform: x and y must both be fp32 or both fp16");
+    pu.fwd(std::make_shared<SpatialTransform>(x, theta, y));
+}
+REGISTER_HIP_OP("spatialtransform", spatialtransform_setup);
 
 // ---------------------------------------------------------------- dropout
 // Inference: identity (the reference aliases it away, :1576-1616).  Training needs a random

@@ -470,7 +470,12 @@ void HipProgram::addBatchedTensors(const ProgramSource &ps)
                 m_batched_tensors[src] = existing->second;
             } else {
                 const Dims dims = src->m_dims.batch(ps.batch_size);
-                auto st = std::make_shared<HipDoubleBuffer>(src->m_data_type, dims.elements(), m_ctx.get());
+                // The reference front end declares the classifier's loss as {1,1} although one value
+                // per sample is written and read (src/node.cpp:336-337, test/test_classifier.cpp:711-716;
+                // there the page granularity of managed memory absorbs it): a batched tensor's buffers
+                // hold at least one element per sample.
+                const size_t elements = std::max<size_t>(dims.elements(), (size_t)std::max(ps.batch_size, 1));
+                auto st = std::make_shared<HipDoubleBuffer>(src->m_data_type, elements, m_ctx.get());
                 auto t = std::make_shared<HipTensor>(st, dims, hip_strides(dims, layoutFor(src->m_data_type)), 0,
                                                      src->m_name);
                 t->copyFromHost(*src);

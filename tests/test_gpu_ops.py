@@ -464,6 +464,24 @@ def test_softmax(dtype):
 
 
 @pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("shape,out", [((3, 1, 28, 28), (224, 224)), ((2, 3, 32, 32), (32, 32)), ((2, 5, 9, 7), (4, 13))])
+def test_spatial_transform(shape, out, dtype):
+    """Resize with the identity matrix (what the classifier harness does in front of ResNet-50) and
+    random affine maps that reach outside the image."""
+    rng = np.random.default_rng(shape[2] + out[0])
+    x = rnd(rng, *shape, dtype=dtype)
+    ident = np.tile(np.array([[1, 0, 0], [0, 1, 0]], np.float32), (shape[0], 1, 1))
+    for theta in (ident, ident + rng.normal(0, 0.3, ident.shape).astype(np.float32)):
+        want = ref.spatial_transform(x, theta, *out)
+        td = torch.from_numpy(theta).cuda()
+        for layout in ("nchw", "nhwc"):
+            xd = dev(x, dtype, layout)
+            yd = dev(np.zeros((shape[0], shape[1]) + out, np.float32), dtype, layout)
+            K.check(K.lib().saga_hip_spatial_transform(C.byref(K.view(xd)), K.ptr(td), C.byref(K.view(yd)), S()))
+            assert_close(host(yd), want, dtype, "spatial transform")
+
+
+@pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("N,Cc", [(7, 10), (64, 1000), (5, 65)])
 def test_catclassifier(N, Cc, dtype):
     rng = np.random.default_rng(N + Cc)

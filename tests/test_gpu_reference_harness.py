@@ -49,3 +49,59 @@ def test_reference_concat():
     r = run("concat")
     assert r.returncode == 0
     assert "18.0" in r.stdout or "18" in r.stdout
+
+
+def write_idx_dataset(path, n_train=6400, n_test=1280, seed=0):
+    """A stand-in for the MNIST files (idx3-ubyte images, idx1-ubyte labels; big-endian headers:
+    magic, count[, rows, cols]) that the reference's `mnist` command reads (test/mnist.cpp:96-119):
+    ten fixed 7x7 patterns blown up to 28x28, shifted by up to two pixels, with noise."""
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    templates = (rng.random((10, 7, 7)) > 0.5).astype(np.float32).repeat(4, axis=1).repeat(4, axis=2)
+
+    def make(n):
+        labels = rng.integers(0, 10, n).astype(np.uint8)
+        img = templates[labels] * 200.0
+        for i in range(n):
+            img[i] = np.roll(img[i], (int(rng.integers(-2, 3)), int(rng.integers(-2, 3))), axis=(0, 1))
+        img += rng.normal(0, 25, img.shape)
+        return np.clip(img, 0, 255).astype(np.uint8), labels
+
+    for prefix, n in (("train", n_train), ("t10k", n_test)):
+        img, lab = make(n)
+        with open(os.path.join(path, f"{prefix}-images-idx3-ubyte"), "wb") as f:
+            f.write(np.array([2051, n, 28, 28], ">u4").tobytes() + img.tobytes())
+        with open(os.path.join(path, f"{prefix}-labels-idx1-ubyte"), "wb") as f:
+            f.write(np.array([2049, n], ">u4").tobytes() + lab.tobytes())
+
+
+def accuracies(stdout):
+    import re
+    return [float(m) for m in re.findall(r"Accuracy:\s*(\d+\.\d+)%", stdout)]
+
+
+@pytest.mark.parametrize("args,floor", [
+    (["-m", "lecun", "-b", "64"], 99.0),
+    (["-m", "lecun", "-b", "64", "-h", "-c"], 99.0),
+    (["-m", "resnet-50", "-h", "-c", "-b", "256", "-r", "1e-3"], 95.0),
+], ids=["lecun-fp32", "lecun-fp16-nhwc", "resnet50-fp16-nhwc-b256"])
+def test_reference_classifier_harness(tmp_path, args, floor):
+    """The reference's training harness (test/test_classifier.cpp:527-857 behind `saga mnist`):
+    uint8 batches loaded by its pre_ops callback into double-buffered tensors, labels written
+    per batch, loss and predictions read back by post_ops, training and inference programs of
+    one context alternating per epoch, until the test accuracy reaches 99 % or 20 epochs passed.
+    The last case is the command the headline numbers of the reference are quoted for."""
+    write_idx_dataset(str(tmp_path))
+    if not os.path.exists(BIN):
+        pytest.skip("oracle/_ref/saga_refhost not built (make -C oracle -f Makefile.ref)")
+    saved = tmp_path / "weights"
+    saved.mkdir()
+    r = subprocess.run([BIN, "mnist", str(tmp_path), *args, "-s", str(saved)], capture_output=True, text=True,
+                       timeout=300)
+    acc = accuracies(r.stdout)
+    print(r.stdout[-1500:].replace("\033", "<esc>"))
+    print(r.stderr[-2000:])
+    print("accuracy per refresh:", acc[-25:])
+    assert r.returncode == 0
+    assert acc and max(acc) >= floor
+    assert any(os.scandir(saved))  # Graph::saveTensors wrote the trained parameters

@@ -228,3 +228,29 @@ def test_loss_scale_rule():
     assert ref.loss_scale_update(1024, [1, 0, 1]) == 512
     assert ref.loss_scale_update(1000, [1, 0, 0]) == np.float32(1020.0)
     assert ref.loss_scale_update(1000, [2, 0, 0]) == np.float32(900.0)
+
+
+def test_spatial_transform_against_torch_and_closed_forms():
+    """Pins so_spatial_transform: (1) torch's affine_grid + grid_sample with align_corners=True and
+    zero padding is the same published rule, implemented independently; (2) the identity matrix
+    on an equal-sized output is a copy; (3) resizing a linear ramp with the identity matrix gives
+    the same ramp sampled at the new pixel centres; (4) a shift of one input pixel moves the image
+    and fills with zeros."""
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((3, 2, 7, 9)).astype(np.float32)
+    theta = np.tile(np.array([[1, 0, 0], [0, 1, 0]], np.float32), (3, 1, 1))
+    theta += rng.normal(0, 0.25, theta.shape).astype(np.float32)  # rotations, zooms, shifts beyond the border
+    for oh, ow in [(7, 9), (12, 5), (20, 31)]:
+        grid = F.affine_grid(torch.from_numpy(theta), (3, 2, oh, ow), align_corners=True)
+        want = F.grid_sample(torch.from_numpy(x), grid, mode="bilinear", padding_mode="zeros", align_corners=True)
+        np.testing.assert_allclose(ref.spatial_transform(x, theta, oh, ow), want.numpy(), atol=2e-5)  # torch keeps the grid in fp32
+    ident = np.tile(np.array([[1, 0, 0], [0, 1, 0]], np.float32), (3, 1, 1))
+    np.testing.assert_allclose(ref.spatial_transform(x, ident, 7, 9), x, atol=1e-6)
+    ramp = np.broadcast_to(np.arange(8, dtype=np.float32), (1, 1, 4, 8)).copy()
+    up = ref.spatial_transform(ramp, ident[:1], 4, 15)
+    np.testing.assert_allclose(up[0, 0, 2], np.linspace(0, 7, 15), atol=1e-5)
+    shift = ident[:1].copy()
+    shift[0, 0, 2] = 2.0 / (9 - 1)  # one input pixel to the right in normalised units
+    moved = ref.spatial_transform(x[:1], shift, 7, 9)
+    np.testing.assert_allclose(moved[..., :-1], x[:1, ..., 1:], atol=1e-5)
+    np.testing.assert_allclose(moved[..., -1], 0, atol=1e-5)
