@@ -44,6 +44,25 @@ MEASURED_HBM_BYTES_PER_LAUNCH = {
 }
 
 
+def by_kind(rows):
+    """The engine reports one row per operation ("kind#position"); add them up per kind.  `roof_ms` is
+    the time the same launches would take at the roofline: each operation at the larger of its
+    algorithmic flops / MFMA peak and its algorithmic bytes / HBM peak (a 1x1 convolution over
+    56x56 pixels is bound by HBM, a 3x3 one over 14x14 pixels by the matrix cores)."""
+    agg = {}
+    for r in rows:
+        if r["launches"] == 0:
+            continue
+        kind = r["kind"].split("#")[0]
+        a = agg.setdefault(kind, {"kind": kind, "launches": 0, "ms": 0.0, "flops": 0.0, "bytes": 0.0, "roof_ms": 0.0})
+        a["launches"] += r["launches"]
+        a["ms"] += r["ms"]
+        a["flops"] += r["flops"]
+        a["bytes"] += r["bytes"]
+        a["roof_ms"] += max(r["flops"] / (PEAK_FP16_TFLOPS * 1e12), r["bytes"] / (PEAK_HBM_GBS * 1e9)) * 1e3
+    return list(agg.values())
+
+
 def profile_rows(rows):
     out = []
     for r in rows:
@@ -52,7 +71,8 @@ def profile_rows(rows):
         matrix = r["kind"].startswith(MATRIX_KINDS)
         sec = r["ms"] * 1e-3
         row = {"kind": r["kind"], "launches": r["launches"], "ms_total": round(r["ms"], 3),
-               "avg_us": round(r["ms"] * 1e3 / r["launches"], 2)}
+               "avg_us": round(r["ms"] * 1e3 / r["launches"], 2),
+               "frac_of_roofline": round(r["roof_ms"] / r["ms"], 4)}
         if matrix:
             a = r["flops"] / sec / 1e12
             row.update(bound="mfma", achieved=round(a, 2), peak=PEAK_FP16_TFLOPS, unit="TFLOP/s",
@@ -121,6 +141,7 @@ def main():
     if args.copy_calibration:
         return copy_calibration()
 
+    os.environ.setdefault("SAGA_HIP_PROFILE_PER_OP", "1")  # profile rows per operation, see by_kind()
     from saga_amd import api as S
     from saga_amd import networks as N
 
@@ -163,7 +184,7 @@ def main():
     if not args.no_profile:
         train.set_profiling(True)
         train.run(args.steps)
-        rows = train.profile()
+        rows = by_kind(train.profile())
         kernels = profile_rows(rows)
         train.set_profiling(False)
         if kernels:
@@ -178,7 +199,9 @@ def main():
             tf = sum(r["flops"] for r in cr) / (sum(r["ms"] for r in cr) * 1e-3) / 1e12
             conv = {"bound": "mfma", "achieved": round(tf, 1), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(tf / PEAK_FP16_TFLOPS, 4), "mfma_util_pct": round(100 * tf / PEAK_FP16_TFLOPS, 2),
-                    "ms_per_step": round(sum(r["ms"] for r in cr) / args.steps, 3)}
+                    "ms_per_step": round(sum(r["ms"] for r in cr) / args.steps, 3),
+                    # against each layer's own bound (HBM for the wide 1x1 layers, MFMA for the others)
+                    "frac_of_roofline": round(sum(r["roof_ms"] for r in cr) / sum(r["ms"] for r in cr), 4)}
 
     flops_step = 3 * net.flops_fwd * args.batch  # fwd + bwd-data + bwd-filter (the stem has no bwd-data)
     ips = args.batch * args.steps / t_train
