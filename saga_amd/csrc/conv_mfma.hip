@@ -993,11 +993,11 @@ __global__ void __launch_bounds__(64 * NW) conv_bwd_filter_dma(FilterArgs g, uns
     constexpr int RA = BK / (NW * RPA), RB = BK / (NW * RPB);
     constexpr int ROWA = BM * 2, ROWB = BN * 2;
     constexpr int STAGE_BYTES = BK * (ROWA + ROWB);
-    constexpr int WGM = BM >= 128 ? 2 : 1, WGN = NW / WGM;
+    constexpr int WGM = NW == 16 ? 4 : (BM >= 128 ? 2 : 1), WGN = NW / WGM;
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
     constexpr unsigned OOB = 0x7fffff00u;
-    static_assert(RA >= 1 && RB >= 1 && (GA == 8 || GA == 16 || GA == 32) && (GB == 8 || GB == 16), "tile");
+    static_assert(RA >= 1 && RB >= 1 && (GA == 8 || GA == 16 || GA == 32) && (GB == 8 || GB == 16 || GB == 32), "tile");
 
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
@@ -1027,7 +1027,7 @@ __global__ void __launch_bounds__(64 * NW) conv_bwd_filter_dma(FilterArgs g, uns
     const bool ka_ok = ka < g.K;
     // B (x): likewise; the logical granule fixes this lane's (tap, c)
     const int pb0 = wave * RPB + lane / GB;
-    const int swb = GB == 16 ? (pb0 & 3) << 2 : ((pb0 >> 1) & 1) << 2;
+    const int swb = GB >= 16 ? (pb0 & 3) << 2 : ((pb0 >> 1) & 1) << 2;
     const int col = j0 + (((lane % GB) ^ swb) << 3);
     const bool cb_ok = col < g.RSC;
     const int tap = cb_ok ? col / g.C : 0;
@@ -1091,7 +1091,7 @@ __global__ void __launch_bounds__(64 * NW) conv_bwd_filter_dma(FilterArgs g, uns
     const int fp = 8 * (lane >> 5) + ((lane & 15) >> 2);
     const int fc = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
     const int fswa = GA >= 16 ? (fp & 3) << 2 : ((fp >> 1) & 1) << 2;
-    const int fswb = GB == 16 ? (fp & 3) << 2 : ((fp >> 1) & 1) << 2;
+    const int fswb = GB >= 16 ? (fp & 3) << 2 : ((fp >> 1) & 1) << 2;
     int foa[TM], fob[TN];
 #pragma unroll
     for(int i = 0; i < TM; i++) {
@@ -1226,18 +1226,38 @@ struct FilterPlan {
     int bm, bn, tiles_k, tiles_c, splits, m_per_split;
 };
 
-static FilterPlan plan_filter(const ConvGeom &g)
+// big_ok: the caller will run the pipelined kernel, the only one that has the large tiles
+static FilterPlan plan_filter(const ConvGeom &g, bool big_ok = true)
 {
     FilterPlan p;
     const int RSC = g.R * g.S * g.C;
     const int64_t M = (int64_t)g.N * g.P * g.Q;
     p.bm = g.K > 64 ? 128 : 64; // 256x128 tiles were measured slower on every ResNet-50 layer
     p.bn = 128;
+    // SAGA_HIP_FILTER_TILE=128 keeps the small tiles everywhere, =256 takes the large one wherever it fits
+    static const char *env = getenv("SAGA_HIP_FILTER_TILE");
+    static const int forced = env ? atoi(env) : 0;
+    int target = 768; // three blocks fit a CU: 768 blocks are one full round of the chip (measured best of 512..2048)
+    // 256x256 on sixteen wavefronts, one block per CU: half the LDS fill traffic per flop.  Measured
+    // 25-35 % faster where the reduction per tile is long enough to pay for the smaller grid (3x3
+    // filters, or 1x1 with >= 1024 input and >= 512 output channels), slower on the other 1x1 layers.
+    const bool fits = big_ok && g.K > 128 && RSC > 128;
+    const bool pays = RSC >= 1024 && (g.R * g.S > 1 || g.K >= 512);
+    if(fits && forced != 128 && (pays || forced == 256)) {
+        p.bm = p.bn = 256;
+        target = 256;
+    } else if(big_ok && g.K > 64 && g.K <= 128 && RSC >= 1024 && g.R * g.S > 1 && forced != 128) {
+        p.bn = 256; // 128x256 on eight wavefronts, two blocks per CU
+        target = 512;
+    } else if(big_ok && g.K <= 64 && RSC >= 512 && g.R * g.S > 1 && forced != 128) {
+        p.bn = 256; // 64x256 on four wavefronts with two stages, four blocks per CU (measured 17 % faster)
+        target = 1024;
+    }
     p.tiles_k = (g.K + p.bm - 1) / p.bm;
     p.tiles_c = (RSC + p.bn - 1) / p.bn;
     const int tiles = p.tiles_k * p.tiles_c;
-    // three blocks fit a CU: 768 blocks are one full round of the chip (measured best of 512..2048)
-    int64_t want = (768 + tiles - 1) / tiles;
+    // with one block per CU a grid just above the CU count would take two rounds: round down there
+    int64_t want = p.bn == 256 ? target / tiles : (target + tiles - 1) / tiles;
     const int64_t maxs = (M + 255) / 256; // at least 256 pixels per split
     if(want > maxs)
         want = maxs;
@@ -1561,8 +1581,9 @@ size_t conv_mfma_workspace(int kind, const SagaTensorView *x, const SagaTensorVi
     if(kind == SAGA_CONV_BWD_FILTER) {
         ConvGeom gp = g;
         gp.C = (int)Cp;
-        const FilterPlan p = plan_filter(gp);
-        size_t need = xpad + (size_t)p.splits * g.K * g.R * g.S * Cp * sizeof(float);
+        // the launcher falls back to the small tiles for tensors beyond the buffer-load range
+        const FilterPlan p = plan_filter(gp), ps = plan_filter(gp, false);
+        size_t need = xpad + (size_t)std::max(p.splits, ps.splits) * g.K * g.R * g.S * Cp * sizeof(float);
         if(thin) {
             ConvGeom gv = g;
             gv.C = 32;
@@ -1755,7 +1776,9 @@ int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, cons
     const int Cp = pad ? round8(g.C) : g.C;
     ConvGeom gp = g;
     gp.C = Cp;
-    const FilterPlan p = plan_filter(gp);
+    const int64_t xb = ((lx.rows - 1) * (int64_t)(pad ? Cp : lx.pitch) + Cp) * 2, yb = ((ldy.rows - 1) * ldy.pitch + ldy.C) * 2;
+    const bool pipelined = dma_stages() >= 2 && xb < 0x7fffff00 && yb < 0x7fffff00;
+    const FilterPlan p = plan_filter(gp, pipelined);
     const size_t xpad = pad ? (((size_t)lx.rows * Cp * sizeof(half_t) + 255) & ~(size_t)255) : 0;
     const size_t need = xpad + (size_t)p.splits * g.K * g.R * g.S * Cp * sizeof(float);
     if(!ws || ws_bytes < need || !aligned16(ws))
@@ -1780,10 +1803,33 @@ int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, cons
     a.tiles_k = p.tiles_k; a.tiles_c = p.tiles_c;
     a.splits = p.splits; a.m_per_split = p.m_per_split;
     const int blocks = p.tiles_k * p.tiles_c * p.splits;
-    const int64_t xb = ((lx.rows - 1) * (int64_t)a.ldx + Cp) * 2, yb = ((ldy.rows - 1) * ldy.pitch + ldy.C) * 2;
-    if(dma_stages() >= 2 && xb < 0x7fffff00 && yb < 0x7fffff00) {
+    if(pipelined) {
         constexpr int ST = 3, FNW = 8;
-        if(p.bm == 128)
+        if(p.bm == 256) {
+            auto kern = conv_bwd_filter_dma<256, 256, ST, 16>;
+            constexpr int lds = ST * BK * 1024;
+            static bool once = false;
+            if(!once) {
+                const hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+                if(e != hipSuccess)
+                    return (int)e;
+                once = true;
+            }
+            kern<<<blocks, 1024, lds, st>>>(a, (unsigned)xb, (unsigned)yb);
+        } else if(p.bm == 128 && p.bn == 256) {
+            auto kern = conv_bwd_filter_dma<128, 256, ST, FNW>;
+            constexpr int lds = ST * BK * 768;
+            static bool once = false;
+            if(!once) {
+                const hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+                if(e != hipSuccess)
+                    return (int)e;
+                once = true;
+            }
+            kern<<<blocks, 64 * FNW, lds, st>>>(a, (unsigned)xb, (unsigned)yb);
+        } else if(p.bm == 64 && p.bn == 256) {
+            conv_bwd_filter_dma<64, 256, 2, 4><<<blocks, 256, 2 * BK * 640, st>>>(a, (unsigned)xb, (unsigned)yb);
+        } else if(p.bm == 128)
             conv_bwd_filter_dma<128, 128, ST, FNW><<<blocks, 64 * FNW, ST * BK * 512, st>>>(a, (unsigned)xb, (unsigned)yb);
         else
             conv_bwd_filter_dma<64, 128, ST, 4><<<blocks, 256, ST * BK * 384, st>>>(a, (unsigned)xb, (unsigned)yb);
