@@ -38,9 +38,9 @@ CONV_KINDS = ("convfwd", "convbwddata", "convbwdfilter")
 MEASURED_HBM_BYTES_PER_LAUNCH = {
     # the counters cannot tell fused from plain batch-norm launches (same kernels): both kinds carry
     # the average over all 53 batch-norm launches of a step
-    "bnbwd.fused": 666484230, "bnbwd": 666484230,
-    "bntrain.fused": 275035172, "bntrain": 275035172,
-    "convfwd": 229309974, "convbwddata": 290906476, "convbwdfilter": 302333026,
+    "bnbwd.fused": 666482496, "bnbwd": 666482496,
+    "bntrain.fused": 275032221, "bntrain": 275032221,
+    "convfwd": 268755817, "convbwddata": 290992982, "convbwdfilter": 308649991,
 }
 
 
