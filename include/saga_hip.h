@@ -192,6 +192,16 @@ int saga_hip_pool_fwd(int mode, const SagaTensorView *x, const SagaTensorView *y
                       int size, int pad, int stride, saga_stream_t stream);
 int saga_hip_pool_bwd(int mode, const SagaTensorView *x, const SagaTensorView *y, const SagaTensorView *dy,
                       const SagaTensorView *dx, int size, int pad, int stride, float beta, saga_stream_t stream);
+/* Max pooling for training that remembers where each maximum came from.  No single counterpart in the
+ * reference: cudnnPoolingBackward re-derives the maximum from x and y (src/cuda/cuda_dnn.cpp:873-899); here
+ * the forward pass leaves one byte per output element (window position r*size + s of the first maximum,
+ * dense N,P,Q,C order, 8-byte aligned buffer of N*C*P*Q bytes) and the backward pass reads only those and
+ * dy - same result, less than half the traffic.  Channels-last tensors with whole 16-byte channel vectors,
+ * size 2 or 3; SAGA_HIP_EUNSUPPORTED otherwise (use saga_hip_pool_fwd / saga_hip_pool_bwd). */
+int saga_hip_maxpool_fwd_codes(const SagaTensorView *x, const SagaTensorView *y, uint8_t *codes, int size, int pad,
+                               int stride, saga_stream_t stream);
+int saga_hip_maxpool_bwd_codes(const uint8_t *codes, const SagaTensorView *dy, const SagaTensorView *dx, int size,
+                               int pad, int stride, float beta, saga_stream_t stream);
 
 /* y = a + b : cudnnOpTensor ADD (src/cuda/cuda_dnn.cpp:1866-1875). */
 int saga_hip_add(const SagaTensorView *a, const SagaTensorView *b, const SagaTensorView *y, saga_stream_t stream);

@@ -310,6 +310,139 @@ __global__ void __launch_bounds__(256) maxpool_bwd_tiled(DView x, DView y, DView
     }
 }
 
+// ---------------------------------------------------------------- max pooling with position codes
+//
+// Training variant for channels-last tensors: the forward pass also leaves, per output element,
+// one byte naming the window position (r*K + s) of its first maximum; the backward pass then
+// needs neither x nor y - an input position receives dy of every window whose code names it.
+// All loads of a thread are issued before the first is consumed (addresses of positions outside
+// the image are clamped and their values ignored).
+
+template <int VN> struct CodeVec;
+template <> struct CodeVec<8> {
+    typedef unsigned type __attribute__((ext_vector_type(2)));
+};
+template <> struct CodeVec<4> {
+    typedef unsigned type;
+};
+
+template <typename T, int VN, int K>
+__global__ void __launch_bounds__(256)
+    maxpool_fwd_codes_k(DView x, DView y, uint8_t *__restrict__ codes, int pad, int stride, unsigned total)
+{
+    const int C = y.d[1], P = y.d[2], Q = y.d[3], H = x.d[2], W = x.d[3];
+    const unsigned cv = C / VN;
+    for(unsigned i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
+        const int c = (int)(i % cv) * VN;
+        unsigned t = i / cv;
+        const int q = (int)(t % (unsigned)Q);
+        t /= (unsigned)Q;
+        const int p = (int)(t % (unsigned)P), n = (int)(t / (unsigned)P);
+        const int h0 = p * stride - pad, w0 = q * stride - pad;
+        float v[K * K][VN];
+        bool ok[K * K];
+#pragma unroll
+        for(int r = 0; r < K; r++)
+#pragma unroll
+            for(int s = 0; s < K; s++) {
+                const int h = h0 + r, w = w0 + s;
+                ok[r * K + s] = h >= 0 && h < H && w >= 0 && w < W;
+                const int hc = h < 0 ? 0 : (h >= H ? H - 1 : h), wc = w < 0 ? 0 : (w >= W ? W - 1 : w);
+                PV<T, VN>::load((const T *)x.ptr + off4(x, n, c, hc, wc), v[r * K + s]);
+            }
+        float acc[VN];
+        unsigned code[VN];
+#pragma unroll
+        for(int j = 0; j < VN; j++) {
+            acc[j] = -INFINITY;
+            code[j] = 0;
+        }
+        bool first = true; // the first position inside the image seeds the maximum of every channel
+#pragma unroll
+        for(int k = 0; k < K * K; k++) {
+#pragma unroll
+            for(int j = 0; j < VN; j++) {
+                const bool take = ok[k] && (first || better(v[k][j], acc[j]));
+                acc[j] = take ? v[k][j] : acc[j];
+                code[j] = take ? (unsigned)k : code[j];
+            }
+            first = first && !ok[k];
+        }
+        PV<T, VN>::store((T *)y.ptr + off4(y, n, c, p, q), acc);
+        typename CodeVec<VN>::type packed;
+        if constexpr(VN == 8) {
+            packed[0] = code[0] | code[1] << 8 | code[2] << 16 | code[3] << 24;
+            packed[1] = code[4] | code[5] << 8 | code[6] << 16 | code[7] << 24;
+        } else {
+            packed = code[0] | code[1] << 8 | code[2] << 16 | code[3] << 24;
+        }
+        *(typename CodeVec<VN>::type *)(codes + (size_t)i * VN) = packed;
+    }
+}
+
+// MAXW = the most windows that can cover one input position along one axis, ceil(K / stride)
+template <typename T, int VN, int K, int MAXW>
+__global__ void __launch_bounds__(256)
+    maxpool_bwd_codes_k(const uint8_t *__restrict__ codes, DView dy, DView dx, int pad, int stride, float beta, unsigned total)
+{
+    const int C = dx.d[1], H = dx.d[2], W = dx.d[3], P = dy.d[2], Q = dy.d[3];
+    const unsigned cv = C / VN;
+    for(unsigned i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
+        const int c = (int)(i % cv) * VN;
+        unsigned t = i / cv;
+        const int w = (int)(t % (unsigned)W);
+        t /= (unsigned)W;
+        const int h = (int)(t % (unsigned)H), n = (int)(t / (unsigned)H);
+        // windows p with p*stride - pad <= h <= p*stride - pad + K - 1
+        int p0 = cdiv_floor(h + pad - K + stride, stride), p1 = cdiv_floor(h + pad, stride);
+        int q0 = cdiv_floor(w + pad - K + stride, stride), q1 = cdiv_floor(w + pad, stride);
+        p0 = p0 < 0 ? 0 : p0;
+        q0 = q0 < 0 ? 0 : q0;
+        p1 = p1 > P - 1 ? P - 1 : p1;
+        q1 = q1 > Q - 1 ? Q - 1 : q1;
+        float g[MAXW * MAXW][VN];
+        typename CodeVec<VN>::type cd[MAXW * MAXW];
+        bool ok[MAXW * MAXW];
+        unsigned expect[MAXW * MAXW];
+#pragma unroll
+        for(int a = 0; a < MAXW; a++)
+#pragma unroll
+            for(int b = 0; b < MAXW; b++) {
+                const int p = p0 + a, q = q0 + b;
+                const int e = a * MAXW + b;
+                ok[e] = p <= p1 && q <= q1;
+                const int pc = p <= p1 ? p : p0 > p1 ? 0 : p1, qc = q <= q1 ? q : q0 > q1 ? 0 : q1;
+                expect[e] = (unsigned)((h + pad - pc * stride) * K + (w + pad - qc * stride));
+                PV<T, VN>::load((const T *)dy.ptr + off4(dy, n, c, pc, qc), g[e]);
+                cd[e] = *(const typename CodeVec<VN>::type *)(codes + ((((size_t)n * P + pc) * Q + qc) * C + c));
+            }
+        float acc[VN];
+#pragma unroll
+        for(int j = 0; j < VN; j++)
+            acc[j] = 0.0f;
+#pragma unroll
+        for(int e = 0; e < MAXW * MAXW; e++)
+#pragma unroll
+            for(int j = 0; j < VN; j++) {
+                unsigned cj;
+                if constexpr(VN == 8)
+                    cj = (cd[e][j >> 2] >> (8 * (j & 3))) & 255u;
+                else
+                    cj = (cd[e] >> (8 * j)) & 255u;
+                acc[j] += (ok[e] && cj == expect[e]) ? g[e][j] : 0.0f;
+            }
+        T *out = (T *)dx.ptr + off4(dx, n, c, h, w);
+        if(beta != 0.0f) {
+            float old[VN];
+            PV<T, VN>::load(out, old);
+#pragma unroll
+            for(int j = 0; j < VN; j++)
+                acc[j] += beta * old[j];
+        }
+        PV<T, VN>::store(out, acc);
+    }
+}
+
 static int vec_for(int dtype, std::initializer_list<const SagaTensorView *> vs)
 {
     const int vn = dtype == SAGA_HALF ? 8 : 4;
@@ -420,4 +553,90 @@ int saga_hip_pool_bwd(int mode, const SagaTensorView *x, const SagaTensorView *y
     return 0;
 }
 
+// Max pooling that records where each maximum came from (one byte per output element, dense
+// N,P,Q,C order); only channels-last tensors whose channels fill whole 16-byte vectors, 2x2 or
+// 3x3 windows.  SAGA_HIP_EUNSUPPORTED otherwise: the caller then uses saga_hip_pool_fwd/bwd.
+static bool codes_ok(const SagaTensorView *a, const SagaTensorView *b, int size, int pad, int stride)
+{
+    if(size < 2 || size > 3 || stride < 1 || stride > size || pad < 0 || pad >= size)
+        return false;
+    if(a->dtype != b->dtype || (a->dtype != SAGA_HALF && a->dtype != SAGA_FLOAT))
+        return false;
+    if(vec_for(a->dtype, {a, b}) == 1)
+        return false;
+    return view_elements(a) < (int64_t)1 << 31 && view_elements(b) < (int64_t)1 << 31;
+}
+
+int saga_hip_maxpool_fwd_codes(const SagaTensorView *x, const SagaTensorView *y, uint8_t *codes, int size, int pad,
+                               int stride, saga_stream_t stream)
+{
+    if(!valid_view(x) || !valid_view(y) || !codes)
+        return SAGA_HIP_EINVAL;
+    if(x->dims[0] != y->dims[0] || x->dims[1] != y->dims[1] || y->dims[2] != pool_dim(x->dims[2], size, pad, stride) ||
+       y->dims[3] != pool_dim(x->dims[3], size, pad, stride))
+        return SAGA_HIP_ESHAPE;
+    if(!codes_ok(x, y, size, pad, stride) || ((uintptr_t)codes & 7))
+        return SAGA_HIP_EUNSUPPORTED;
+    const int vn = x->dtype == SAGA_HALF ? 8 : 4;
+    const unsigned total = (unsigned)(view_elements(y) / vn);
+    const int g = grid_for(total, 256, 256 * 256);
+    hipStream_t st = as_stream(stream);
+    const DView dvx = dview(x), dvy = dview(y);
+#define GO(T, VN)                                                                                              \
+    do {                                                                                                       \
+        if(size == 3)                                                                                          \
+            maxpool_fwd_codes_k<T, VN, 3><<<g, 256, 0, st>>>(dvx, dvy, codes, pad, stride, total);              \
+        else                                                                                                   \
+            maxpool_fwd_codes_k<T, VN, 2><<<g, 256, 0, st>>>(dvx, dvy, codes, pad, stride, total);              \
+    } while(0)
+    if(x->dtype == SAGA_HALF)
+        GO(half_t, 8);
+    else
+        GO(float, 4);
+#undef GO
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
+int saga_hip_maxpool_bwd_codes(const uint8_t *codes, const SagaTensorView *dy, const SagaTensorView *dx, int size, int pad,
+                               int stride, float beta, saga_stream_t stream)
+{
+    if(!valid_view(dy) || !valid_view(dx) || !codes)
+        return SAGA_HIP_EINVAL;
+    if(dy->dims[0] != dx->dims[0] || dy->dims[1] != dx->dims[1] ||
+       dy->dims[2] != pool_dim(dx->dims[2], size, pad, stride) || dy->dims[3] != pool_dim(dx->dims[3], size, pad, stride))
+        return SAGA_HIP_ESHAPE;
+    if(!codes_ok(dx, dy, size, pad, stride) || ((uintptr_t)codes & 7))
+        return SAGA_HIP_EUNSUPPORTED;
+    const int vn = dx->dtype == SAGA_HALF ? 8 : 4;
+    const unsigned total = (unsigned)(view_elements(dx) / vn);
+    const int g = grid_for(total, 256, 256 * 256);
+    const int maxw = (size + stride - 1) / stride;
+    hipStream_t st = as_stream(stream);
+    const DView dvdy = dview(dy), dvdx = dview(dx);
+#define GO2(T, VN, K, MW) maxpool_bwd_codes_k<T, VN, K, MW><<<g, 256, 0, st>>>(codes, dvdy, dvdx, pad, stride, beta, total)
+#define GO(T, VN)                                                                                              \
+    do {                                                                                                       \
+        if(size == 3 && maxw == 3)                                                                             \
+            GO2(T, VN, 3, 3);                                                                                  \
+        else if(size == 3 && maxw == 2)                                                                        \
+            GO2(T, VN, 3, 2);                                                                                  \
+        else if(size == 3)                                                                                     \
+            GO2(T, VN, 3, 1);                                                                                  \
+        else if(maxw == 2)                                                                                     \
+            GO2(T, VN, 2, 2);                                                                                  \
+        else                                                                                                   \
+            GO2(T, VN, 2, 1);                                                                                  \
+    } while(0)
+    if(dx->dtype == SAGA_HALF)
+        GO(half_t, 8);
+    else
+        GO(float, 4);
+#undef GO
+#undef GO2
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
 } // extern "C"
+

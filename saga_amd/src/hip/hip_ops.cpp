@@ -386,6 +386,67 @@ struct PoolBwd : public HipOperation {
     }
 };
 
+// Max pooling in a training program, channels-last: the forward pass records the position of every
+// maximum in a byte tensor of y's shape and the backward pass reads that instead of x and y.
+struct MaxPoolFwdCodes : public HipOperation {
+    const T x_, y_, codes_;
+    const int size_, pad_, stride_;
+    MaxPoolFwdCodes(T x, T y, T codes, int size, int pad, int stride)
+      : HipOperation("poolfwd"), x_(x), y_(y), codes_(codes), size_(size), pad_(pad), stride_(stride)
+    {
+    }
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vx = x_->view(), vy = y_->view();
+        chkSaga(saga_hip_maxpool_fwd_codes(&vx, &vy, (uint8_t *)codes_->deviceMem(), size_, pad_, stride_, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"x", x_}}; }
+    HipOpArgs listOutputs() const override { return {{"y", y_}, {"codes", codes_}}; }
+    std::string info() const override { return "max+codes"; }
+    double bytes() const override { return nbytes(x_) + nbytes(y_) + nbytes(codes_); }
+};
+
+struct MaxPoolBwdCodes : public HipOperation {
+    const T codes_, dy_, dx_;
+    const int size_, pad_, stride_;
+    float beta_ = 0;
+    MaxPoolBwdCodes(T codes, T dy, T dx, int size, int pad, int stride)
+      : HipOperation("poolbwd"), codes_(codes), dy_(dy), dx_(dx), size_(size), pad_(pad), stride_(stride)
+    {
+    }
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vdy = dy_->view(), vdx = dx_->view();
+        chkSaga(saga_hip_maxpool_bwd_codes((const uint8_t *)codes_->deviceMem(), &vdy, &vdx, size_, pad_, stride_, beta_,
+                                           S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"codes", codes_}, {"dy", dy_}}; }
+    HipOpArgs listOutputs() const override { return {{"dx", dx_}}; }
+    float *getBeta(const T &t) override { return t == dx_ ? &beta_ : nullptr; }
+    double bytes() const override { return nbytes(dx_) * (beta_ != 0 ? 2 : 1) + nbytes(dy_) + nbytes(codes_); }
+};
+
+// what saga_hip_maxpool_*_codes accept (anything else takes the x / y based kernels)
+static bool maxpool_codes_fit(const HipTensor &x, const HipTensor &y, const HipTensor *dx, const HipTensor *dy, int size,
+                              int pad, int stride)
+{
+    if(getenv("SAGA_HIP_NO_POOL_CODES"))
+        return false;
+    if(size < 2 || size > 3 || stride < 1 || stride > size || pad >= size)
+        return false;
+    const int vn = x.m_data_type == Tensor::DataType::HALF ? 8 : x.m_data_type == Tensor::DataType::FLOAT ? 4 : 0;
+    if(!vn || x.m_dims.size() != 4 || (int)x.m_dims[1] % vn)
+        return false;
+    for(const HipTensor *t : {&x, &y, dx, dy}) {
+        if(!t || !t->cpacked() || t->m_data_type != x.m_data_type || t->m_dims.elements() >= ((size_t)1 << 31))
+            return false;
+        for(int i : {0, 2, 3})
+            if((int)t->m_dims[i] > 1 && t->m_strides[i] % vn)
+                return false;
+    }
+    return true;
+}
+
 void pooling_setup(HipProgram &p, HipProgramUnit &pu, const Node &n, int mode)
 {
     auto x = p.lower(pu, n.m_inputs["x"]);
@@ -393,11 +454,21 @@ void pooling_setup(HipProgram &p, HipProgramUnit &pu, const Node &n, int mode)
     const int size = n.m_attributes.get("global", false) ? (int)x->m_dims[2] : n.m_attributes.get("size", 1);
     const int pad = n.m_attributes.get("pad", 0);
     const int stride = n.m_attributes.get("stride", 1);
-    pu.fwd(std::make_shared<PoolFwd>(x, y, mode, size, pad, stride));
-    if(p.m_pt == ProgramType::INFERENCE)
+    if(p.m_pt == ProgramType::INFERENCE) {
+        pu.fwd(std::make_shared<PoolFwd>(x, y, mode, size, pad, stride));
         return;
+    }
     auto dx = p.lowerGrad(pu, n.m_inputs["x"]);
     auto dy = p.lowerGrad(pu, n.m_outputs["y"]);
+    if(mode == SAGA_POOL_MAX && dx && dy && maxpool_codes_fit(*x, *y, dx.get(), dy.get(), size, pad, stride)) {
+        // dense N,H,W,C bytes whatever pitch y has
+        auto codes = std::make_shared<HipTensor>(Tensor::DataType::U8, y->m_dims, HipLayout::NHWC, p.m_ctx.get(),
+                                                 n.m_outputs["y"]->namePostfix("maxpos"));
+        pu.fwd(std::make_shared<MaxPoolFwdCodes>(x, y, codes, size, pad, stride));
+        pu.bwd(std::make_shared<MaxPoolBwdCodes>(codes, dy, dx, size, pad, stride));
+        return;
+    }
+    pu.fwd(std::make_shared<PoolFwd>(x, y, mode, size, pad, stride));
     pu.bwd(std::make_shared<PoolBwd>(x, y, dx, dy, mode, size, pad, stride));
 }
 void maxpool_setup(HipProgram &p, HipProgramUnit &pu, const Node &n) { pooling_setup(p, pu, n, SAGA_POOL_MAX); }

@@ -409,6 +409,48 @@ def test_pooling(k, pad, stride, H, layout, padc, dtype):
         assert_close(host(dxd), dx_ref + 1, dtype, mode + "pool bwd")
 
 
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("padc", [0, 8])
+@pytest.mark.parametrize("k,pad,stride,H", [(2, 0, 2, 8), (3, 1, 2, 9), (3, 1, 2, 12), (3, 1, 1, 6), (3, 0, 3, 10), (2, 1, 1, 5)])
+def test_maxpool_with_position_codes(k, pad, stride, H, padc, dtype):
+    """The training pair saga_hip_maxpool_fwd_codes / _bwd_codes on channels-last tensors (dense and
+    with a wider channel pitch): y and the recorded first-maximum positions bit-exact against the
+    oracle's indices, dx against the oracle's backward - on post-relu data full of exact ties, with
+    a NaN and with rows of -inf."""
+    rng = np.random.default_rng(k * 100 + H + pad)
+    shape = (3, 16, H, H + 1)
+    x = np.maximum(rnd(rng, *shape, dtype=dtype), 0)
+    x[0, 3, 1, 2] = np.nan
+    x[1, 5] = -np.inf
+    P, Q = ref.pool_out(H, k, pad, stride), ref.pool_out(H + 1, k, pad, stride)
+    oshape = (3, 16, P, Q)
+    dy = rnd(rng, *oshape, dtype=dtype)
+    y_ref, idx_ref = ref.maxpool_fwd(x, k, pad, stride, with_idx=True)
+    L = K.lib()
+    xd = dev(x, dtype, "nhwc", padc)
+    yd = dev(np.zeros(oshape, np.float32), dtype, "nhwc", padc)
+    codes = torch.full((3, P, Q, 16), 255, dtype=torch.uint8, device="cuda")
+    K.check(L.saga_hip_maxpool_fwd_codes(C.byref(K.view(xd)), C.byref(K.view(yd)), K.ptr(codes), k, pad, stride, S()))
+    np.testing.assert_array_equal(host(yd), y_ref)
+    # code r*k+s -> input position (p*stride-pad+r)*W + (q*stride-pad+s), the oracle's index
+    cd = codes.cpu().numpy().astype(np.int64).transpose(0, 3, 1, 2)
+    pp, qq = np.meshgrid(np.arange(P), np.arange(Q), indexing="ij")
+    pos = (pp * stride - pad + cd // k) * (H + 1) + (qq * stride - pad + cd % k)
+    np.testing.assert_array_equal(pos, idx_ref)
+    dx_ref = ref.maxpool_bwd(x, dy, k, pad, stride)
+    dyd = dev(dy, dtype, "nhwc", padc)
+    for beta in (0.0, 1.0):
+        dxd = dev(np.ones(shape, np.float32), dtype, "nhwc", padc)
+        K.check(L.saga_hip_maxpool_bwd_codes(K.ptr(codes), C.byref(K.view(dyd)), C.byref(K.view(dxd)), k, pad, stride,
+                                             beta, S()))
+        assert_close(host(dxd), dx_ref + beta, dtype, "maxpool bwd from codes")
+    # what the pair does not take is refused, not computed wrongly
+    xn = dev(x, dtype, "nchw")
+    yn = dev(np.zeros(oshape, np.float32), dtype, "nchw")
+    rc = L.saga_hip_maxpool_fwd_codes(C.byref(K.view(xn)), C.byref(K.view(yn)), K.ptr(codes), k, pad, stride, S())
+    assert rc == -3  # SAGA_HIP_EUNSUPPORTED
+
+
 def test_pooling_golden(golden):
     g = golden["ops"]
     x = T(g, "pooling_input")
