@@ -326,121 +326,122 @@ template <> struct CodeVec<4> {
     typedef unsigned type;
 };
 
-template <typename T, int VN, int K>
-__global__ void __launch_bounds__(256)
-    maxpool_fwd_codes_k(DView x, DView y, uint8_t *__restrict__ codes, int pad, int stride, unsigned total)
+// Work mapping without integer division (a thread handles 16 bytes; eight divisions by run-time
+// values cost more than its memory traffic): blockIdx.z = sample, blockIdx.y = output row,
+// threadIdx.x = channel vector, threadIdx.y (+ blockIdx.x) = output column.  K and the stride
+// are template parameters so that the window arithmetic folds to shifts and constants.
+template <typename T, int VN, int K, int S>
+__global__ void __launch_bounds__(256) maxpool_fwd_codes_k(DView x, DView y, uint8_t *__restrict__ codes, int pad)
 {
     const int C = y.d[1], P = y.d[2], Q = y.d[3], H = x.d[2], W = x.d[3];
-    const unsigned cv = C / VN;
-    for(unsigned i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
-        const int c = (int)(i % cv) * VN;
-        unsigned t = i / cv;
-        const int q = (int)(t % (unsigned)Q);
-        t /= (unsigned)Q;
-        const int p = (int)(t % (unsigned)P), n = (int)(t / (unsigned)P);
-        const int h0 = p * stride - pad, w0 = q * stride - pad;
-        float v[K * K][VN];
-        bool ok[K * K];
+    const int n = blockIdx.z, p = blockIdx.y;
+    const int q = blockIdx.x * blockDim.y + threadIdx.y;
+    const int c = threadIdx.x * VN;
+    if(q >= Q || c >= C)
+        return;
+    const int h0 = p * S - pad, w0 = q * S - pad;
+    float v[K * K][VN];
+    bool ok[K * K];
 #pragma unroll
-        for(int r = 0; r < K; r++)
+    for(int r = 0; r < K; r++)
 #pragma unroll
-            for(int s = 0; s < K; s++) {
-                const int h = h0 + r, w = w0 + s;
-                ok[r * K + s] = h >= 0 && h < H && w >= 0 && w < W;
-                const int hc = h < 0 ? 0 : (h >= H ? H - 1 : h), wc = w < 0 ? 0 : (w >= W ? W - 1 : w);
-                PV<T, VN>::load((const T *)x.ptr + off4(x, n, c, hc, wc), v[r * K + s]);
-            }
-        float acc[VN];
-        unsigned code[VN];
+        for(int s = 0; s < K; s++) {
+            const int h = h0 + r, w = w0 + s;
+            ok[r * K + s] = h >= 0 && h < H && w >= 0 && w < W;
+            const int hc = h < 0 ? 0 : (h >= H ? H - 1 : h), wc = w < 0 ? 0 : (w >= W ? W - 1 : w);
+            PV<T, VN>::load((const T *)x.ptr + off4(x, n, c, hc, wc), v[r * K + s]);
+        }
+    float acc[VN];
+    unsigned code[VN];
+#pragma unroll
+    for(int j = 0; j < VN; j++) {
+        acc[j] = -INFINITY;
+        code[j] = 0;
+    }
+    bool first = true; // the first position inside the image seeds the maximum of every channel
+#pragma unroll
+    for(int k = 0; k < K * K; k++) {
 #pragma unroll
         for(int j = 0; j < VN; j++) {
-            acc[j] = -INFINITY;
-            code[j] = 0;
+            const bool take = ok[k] && (first || better(v[k][j], acc[j]));
+            acc[j] = take ? v[k][j] : acc[j];
+            code[j] = take ? (unsigned)k : code[j];
         }
-        bool first = true; // the first position inside the image seeds the maximum of every channel
-#pragma unroll
-        for(int k = 0; k < K * K; k++) {
-#pragma unroll
-            for(int j = 0; j < VN; j++) {
-                const bool take = ok[k] && (first || better(v[k][j], acc[j]));
-                acc[j] = take ? v[k][j] : acc[j];
-                code[j] = take ? (unsigned)k : code[j];
-            }
-            first = first && !ok[k];
-        }
-        PV<T, VN>::store((T *)y.ptr + off4(y, n, c, p, q), acc);
-        typename CodeVec<VN>::type packed;
-        if constexpr(VN == 8) {
-            packed[0] = code[0] | code[1] << 8 | code[2] << 16 | code[3] << 24;
-            packed[1] = code[4] | code[5] << 8 | code[6] << 16 | code[7] << 24;
-        } else {
-            packed = code[0] | code[1] << 8 | code[2] << 16 | code[3] << 24;
-        }
-        *(typename CodeVec<VN>::type *)(codes + (size_t)i * VN) = packed;
+        first = first && !ok[k];
     }
+    PV<T, VN>::store((T *)y.ptr + off4(y, n, c, p, q), acc);
+    typename CodeVec<VN>::type packed;
+    if constexpr(VN == 8) {
+        packed[0] = code[0] | code[1] << 8 | code[2] << 16 | code[3] << 24;
+        packed[1] = code[4] | code[5] << 8 | code[6] << 16 | code[7] << 24;
+    } else {
+        packed = code[0] | code[1] << 8 | code[2] << 16 | code[3] << 24;
+    }
+    *(typename CodeVec<VN>::type *)(codes + ((((size_t)n * P + p) * Q + q) * C + c)) = packed;
 }
 
-// MAXW = the most windows that can cover one input position along one axis, ceil(K / stride)
-template <typename T, int VN, int K, int MAXW>
+// floor(a / S) for a that may be negative, S a compile-time constant
+template <int S> __device__ __forceinline__ int floor_div(int a) { return a >= 0 ? a / S : -((-a + S - 1) / S); }
+
+// blockIdx.z = sample, blockIdx.y = input row, threadIdx.x = channel vector, threadIdx.y = input column
+template <typename T, int VN, int K, int S>
 __global__ void __launch_bounds__(256)
-    maxpool_bwd_codes_k(const uint8_t *__restrict__ codes, DView dy, DView dx, int pad, int stride, float beta, unsigned total)
+    maxpool_bwd_codes_k(const uint8_t *__restrict__ codes, DView dy, DView dx, int pad, float beta)
 {
-    const int C = dx.d[1], H = dx.d[2], W = dx.d[3], P = dy.d[2], Q = dy.d[3];
-    const unsigned cv = C / VN;
-    for(unsigned i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
-        const int c = (int)(i % cv) * VN;
-        unsigned t = i / cv;
-        const int w = (int)(t % (unsigned)W);
-        t /= (unsigned)W;
-        const int h = (int)(t % (unsigned)H), n = (int)(t / (unsigned)H);
-        // windows p with p*stride - pad <= h <= p*stride - pad + K - 1
-        int p0 = cdiv_floor(h + pad - K + stride, stride), p1 = cdiv_floor(h + pad, stride);
-        int q0 = cdiv_floor(w + pad - K + stride, stride), q1 = cdiv_floor(w + pad, stride);
-        p0 = p0 < 0 ? 0 : p0;
-        q0 = q0 < 0 ? 0 : q0;
-        p1 = p1 > P - 1 ? P - 1 : p1;
-        q1 = q1 > Q - 1 ? Q - 1 : q1;
-        float g[MAXW * MAXW][VN];
-        typename CodeVec<VN>::type cd[MAXW * MAXW];
-        bool ok[MAXW * MAXW];
-        unsigned expect[MAXW * MAXW];
+    constexpr int MAXW = (K + S - 1) / S; // the most windows that cover one input position along one axis
+    const int C = dx.d[1], W = dx.d[3], P = dy.d[2], Q = dy.d[3];
+    const int n = blockIdx.z, h = blockIdx.y;
+    const int w = blockIdx.x * blockDim.y + threadIdx.y;
+    const int c = threadIdx.x * VN;
+    if(w >= W || c >= C)
+        return;
+    // windows p with p*S - pad <= h <= p*S - pad + K - 1
+    int p0 = floor_div<S>(h + pad - K + S), p1 = floor_div<S>(h + pad);
+    int q0 = floor_div<S>(w + pad - K + S), q1 = floor_div<S>(w + pad);
+    p0 = p0 < 0 ? 0 : p0;
+    q0 = q0 < 0 ? 0 : q0;
+    p1 = p1 > P - 1 ? P - 1 : p1;
+    q1 = q1 > Q - 1 ? Q - 1 : q1;
+    float g[MAXW * MAXW][VN];
+    typename CodeVec<VN>::type cd[MAXW * MAXW];
+    bool ok[MAXW * MAXW];
+    unsigned expect[MAXW * MAXW];
 #pragma unroll
-        for(int a = 0; a < MAXW; a++)
+    for(int a = 0; a < MAXW; a++)
 #pragma unroll
-            for(int b = 0; b < MAXW; b++) {
-                const int p = p0 + a, q = q0 + b;
-                const int e = a * MAXW + b;
-                ok[e] = p <= p1 && q <= q1;
-                const int pc = p <= p1 ? p : p0 > p1 ? 0 : p1, qc = q <= q1 ? q : q0 > q1 ? 0 : q1;
-                expect[e] = (unsigned)((h + pad - pc * stride) * K + (w + pad - qc * stride));
-                PV<T, VN>::load((const T *)dy.ptr + off4(dy, n, c, pc, qc), g[e]);
-                cd[e] = *(const typename CodeVec<VN>::type *)(codes + ((((size_t)n * P + pc) * Q + qc) * C + c));
-            }
-        float acc[VN];
+        for(int b = 0; b < MAXW; b++) {
+            const int p = p0 + a, q = q0 + b;
+            const int e = a * MAXW + b;
+            ok[e] = p <= p1 && q <= q1;
+            const int pc = p <= p1 ? p : p0 > p1 ? 0 : p1, qc = q <= q1 ? q : q0 > q1 ? 0 : q1;
+            expect[e] = (unsigned)((h + pad - pc * S) * K + (w + pad - qc * S));
+            PV<T, VN>::load((const T *)dy.ptr + off4(dy, n, c, pc, qc), g[e]);
+            cd[e] = *(const typename CodeVec<VN>::type *)(codes + ((((size_t)n * P + pc) * Q + qc) * C + c));
+        }
+    float acc[VN];
+#pragma unroll
+    for(int j = 0; j < VN; j++)
+        acc[j] = 0.0f;
+#pragma unroll
+    for(int e = 0; e < MAXW * MAXW; e++)
+#pragma unroll
+        for(int j = 0; j < VN; j++) {
+            unsigned cj;
+            if constexpr(VN == 8)
+                cj = (cd[e][j >> 2] >> (8 * (j & 3))) & 255u;
+            else
+                cj = (cd[e] >> (8 * j)) & 255u;
+            acc[j] += (ok[e] && cj == expect[e]) ? g[e][j] : 0.0f;
+        }
+    T *out = (T *)dx.ptr + off4(dx, n, c, h, w);
+    if(beta != 0.0f) {
+        float old[VN];
+        PV<T, VN>::load(out, old);
 #pragma unroll
         for(int j = 0; j < VN; j++)
-            acc[j] = 0.0f;
-#pragma unroll
-        for(int e = 0; e < MAXW * MAXW; e++)
-#pragma unroll
-            for(int j = 0; j < VN; j++) {
-                unsigned cj;
-                if constexpr(VN == 8)
-                    cj = (cd[e][j >> 2] >> (8 * (j & 3))) & 255u;
-                else
-                    cj = (cd[e] >> (8 * j)) & 255u;
-                acc[j] += (ok[e] && cj == expect[e]) ? g[e][j] : 0.0f;
-            }
-        T *out = (T *)dx.ptr + off4(dx, n, c, h, w);
-        if(beta != 0.0f) {
-            float old[VN];
-            PV<T, VN>::load(out, old);
-#pragma unroll
-            for(int j = 0; j < VN; j++)
-                acc[j] += beta * old[j];
-        }
-        PV<T, VN>::store(out, acc);
+            acc[j] += beta * old[j];
     }
+    PV<T, VN>::store(out, acc);
 }
 
 static int vec_for(int dtype, std::initializer_list<const SagaTensorView *> vs)
@@ -564,7 +565,20 @@ static bool codes_ok(const SagaTensorView *a, const SagaTensorView *b, int size,
         return false;
     if(vec_for(a->dtype, {a, b}) == 1)
         return false;
-    return view_elements(a) < (int64_t)1 << 31 && view_elements(b) < (int64_t)1 << 31;
+    const int vn = a->dtype == SAGA_HALF ? 8 : 4;
+    // one block spans all channel vectors of a pixel; rows and samples are grid dimensions
+    return a->dims[1] / vn <= 256 && a->dims[0] <= 65535 && a->dims[2] <= 65535 && b->dims[2] <= 65535;
+}
+
+// block = (channel vectors rounded up to a power of two) x (columns to fill 256 threads)
+static void codes_launch_shape(int cv, int cols, int rows, int n, dim3 &grid, dim3 &block)
+{
+    int bx = 1;
+    while(bx < cv)
+        bx <<= 1;
+    const int by = 256 / bx;
+    block = dim3(bx, by, 1);
+    grid = dim3((cols + by - 1) / by, rows, n);
 }
 
 int saga_hip_maxpool_fwd_codes(const SagaTensorView *x, const SagaTensorView *y, uint8_t *codes, int size, int pad,
@@ -578,22 +592,27 @@ int saga_hip_maxpool_fwd_codes(const SagaTensorView *x, const SagaTensorView *y,
     if(!codes_ok(x, y, size, pad, stride) || ((uintptr_t)codes & 7))
         return SAGA_HIP_EUNSUPPORTED;
     const int vn = x->dtype == SAGA_HALF ? 8 : 4;
-    const unsigned total = (unsigned)(view_elements(y) / vn);
-    const int g = grid_for(total, 256, 256 * 256);
+    dim3 grid, block;
+    codes_launch_shape(y->dims[1] / vn, y->dims[3], y->dims[2], y->dims[0], grid, block);
     hipStream_t st = as_stream(stream);
     const DView dvx = dview(x), dvy = dview(y);
+#define GO2(T, VN, K, S) maxpool_fwd_codes_k<T, VN, K, S><<<grid, block, 0, st>>>(dvx, dvy, codes, pad)
 #define GO(T, VN)                                                                                              \
     do {                                                                                                       \
-        if(size == 3)                                                                                          \
-            maxpool_fwd_codes_k<T, VN, 3><<<g, 256, 0, st>>>(dvx, dvy, codes, pad, stride, total);              \
-        else                                                                                                   \
-            maxpool_fwd_codes_k<T, VN, 2><<<g, 256, 0, st>>>(dvx, dvy, codes, pad, stride, total);              \
+        switch(size * 4 + stride) {                                                                            \
+        case 13: GO2(T, VN, 3, 1); break;                                                                      \
+        case 14: GO2(T, VN, 3, 2); break;                                                                      \
+        case 15: GO2(T, VN, 3, 3); break;                                                                      \
+        case 9: GO2(T, VN, 2, 1); break;                                                                       \
+        default: GO2(T, VN, 2, 2); break;                                                                      \
+        }                                                                                                      \
     } while(0)
     if(x->dtype == SAGA_HALF)
         GO(half_t, 8);
     else
         GO(float, 4);
 #undef GO
+#undef GO2
     SAGA_CHECK_LAUNCH();
     return 0;
 }
@@ -609,24 +628,20 @@ int saga_hip_maxpool_bwd_codes(const uint8_t *codes, const SagaTensorView *dy, c
     if(!codes_ok(dx, dy, size, pad, stride) || ((uintptr_t)codes & 7))
         return SAGA_HIP_EUNSUPPORTED;
     const int vn = dx->dtype == SAGA_HALF ? 8 : 4;
-    const unsigned total = (unsigned)(view_elements(dx) / vn);
-    const int g = grid_for(total, 256, 256 * 256);
-    const int maxw = (size + stride - 1) / stride;
+    dim3 grid, block;
+    codes_launch_shape(dx->dims[1] / vn, dx->dims[3], dx->dims[2], dx->dims[0], grid, block);
     hipStream_t st = as_stream(stream);
     const DView dvdy = dview(dy), dvdx = dview(dx);
-#define GO2(T, VN, K, MW) maxpool_bwd_codes_k<T, VN, K, MW><<<g, 256, 0, st>>>(codes, dvdy, dvdx, pad, stride, beta, total)
+#define GO2(T, VN, K, S) maxpool_bwd_codes_k<T, VN, K, S><<<grid, block, 0, st>>>(codes, dvdy, dvdx, pad, beta)
 #define GO(T, VN)                                                                                              \
     do {                                                                                                       \
-        if(size == 3 && maxw == 3)                                                                             \
-            GO2(T, VN, 3, 3);                                                                                  \
-        else if(size == 3 && maxw == 2)                                                                        \
-            GO2(T, VN, 3, 2);                                                                                  \
-        else if(size == 3)                                                                                     \
-            GO2(T, VN, 3, 1);                                                                                  \
-        else if(maxw == 2)                                                                                     \
-            GO2(T, VN, 2, 2);                                                                                  \
-        else                                                                                                   \
-            GO2(T, VN, 2, 1);                                                                                  \
+        switch(size * 4 + stride) {                                                                            \
+        case 13: GO2(T, VN, 3, 1); break;                                                                      \
+        case 14: GO2(T, VN, 3, 2); break;                                                                      \
+        case 15: GO2(T, VN, 3, 3); break;                                                                      \
+        case 9: GO2(T, VN, 2, 1); break;                                                                       \
+        default: GO2(T, VN, 2, 2); break;                                                                      \
+        }                                                                                                      \
     } while(0)
     if(dx->dtype == SAGA_HALF)
         GO(half_t, 8);
