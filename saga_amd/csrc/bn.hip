@@ -219,55 +219,73 @@ __device__ __forceinline__ double wave_sum_f64(double v)
     return v;
 }
 
-// Adds the gx per-block partial pairs of channel c over one wavefront, in a fixed order.
-// The loads of a lane are independent: eight are issued before any is consumed, so the
-// wavefront pays the memory latency a few times, not once per partial.
-__device__ __forceinline__ void sum_partials(const float *__restrict__ partial, int gx, int C, int c, int lane,
-                                             double &s0, double &s1)
+// Adds the gx per-block partial pairs of channel c over the four wavefronts of a block, in a
+// fixed order.  The loads of a thread are independent: eight are issued before any is consumed,
+// and with 256 threads on one channel even 2048 partials are one such batch per thread, so the
+// block pays the memory latency about once (these kernels are nothing but latency).
+// The totals are valid in thread 0 only.
+__device__ __forceinline__ void sum_partials(const float *__restrict__ partial, int gx, int C, int c, double &s0,
+                                             double &s1)
 {
     typedef float float2_t __attribute__((ext_vector_type(2)));
+    __shared__ double red[4][2];
     const float2_t *p = (const float2_t *)partial + c;
+    const int tid = threadIdx.x;
     double a0 = 0, a1 = 0;
-    int g = lane;
-    for(; g + 7 * 64 < gx; g += 8 * 64) {
+    int g = tid;
+    for(; g + 7 * 256 < gx; g += 8 * 256) {
         float2_t v[8];
 #pragma unroll
         for(int u = 0; u < 8; u++)
-            v[u] = p[(int64_t)(g + u * 64) * C];
+            v[u] = p[(int64_t)(g + u * 256) * C];
 #pragma unroll
         for(int u = 0; u < 8; u++) {
             a0 += v[u][0];
             a1 += v[u][1];
         }
     }
-    for(; g < gx; g += 64) {
-        const float2_t v = p[(int64_t)g * C];
-        a0 += v[0];
-        a1 += v[1];
+    {
+        // the remainder, again as one batch: out-of-range slots read row 0 and are not added
+        float2_t v[8];
+#pragma unroll
+        for(int u = 0; u < 8; u++) {
+            const int r = g + u * 256;
+            v[u] = p[(int64_t)(r < gx ? r : 0) * C];
+        }
+#pragma unroll
+        for(int u = 0; u < 8; u++)
+            if(g + u * 256 < gx) {
+                a0 += v[u][0];
+                a1 += v[u][1];
+            }
     }
-    s0 = wave_sum_f64(a0);
-    s1 = wave_sum_f64(a1);
+    a0 = wave_sum_f64(a0);
+    a1 = wave_sum_f64(a1);
+    if((tid & 63) == 0) {
+        red[tid >> 6][0] = a0;
+        red[tid >> 6][1] = a1;
+    }
+    __syncthreads();
+    s0 = red[0][0] + red[1][0] + red[2][0] + red[3][0];
+    s1 = red[0][1] + red[1][1] + red[2][1] + red[3][1];
 }
 
 // Finalize: mean, biased variance, invstd, running statistics, fused scale/shift.
-// One wavefront per channel adds the per-block partials (lanes stride over the blocks).
+// One block per channel adds the per-block partials (threads stride over the blocks).
 template <typename T>
 __global__ void __launch_bounds__(256)
     bn_stats_finalize(const float *__restrict__ partial, int gx, const T *__restrict__ xrow0, int64_t kstride,
                       const float *__restrict__ s, const float *__restrict__ b, float *run_m, float *run_v,
                       float *save_mean, float *save_invstd, float *ss, double M, int C, float eps, float expavg)
 {
-    const int lane = threadIdx.x & 63;
-    const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if(c >= C)
-        return;
+    const int c = blockIdx.x;
     // parameter loads first: they overlap the partial-sum loads instead of following them
     const double k = xrow0 ? (double)(float)xrow0[c * kstride] : 0.0;
     const float sv = s[c], bv = b[c];
     const float rm_old = run_m ? run_m[c] : 0.0f, rv_old = run_v ? run_v[c] : 0.0f;
     double s0, s1;
-    sum_partials(partial, gx, C, c, lane, s0, s1);
-    if(lane != 0)
+    sum_partials(partial, gx, C, c, s0, s1);
+    if(threadIdx.x != 0)
         return;
     const double dm = s0 / M;
     double var = s1 / M - dm * dm;
@@ -378,22 +396,19 @@ __global__ void __launch_bounds__(256)
 }
 
 // coef[0..C) = s*invstd ; coef[C..2C) = db/M ; coef[2C..3C) = ds*invstd/M ; writes ds, db.
-// One wavefront per channel, as above.
+// One block per channel, as above.
 __global__ void __launch_bounds__(256)
     bn_bwd_finalize(const float *__restrict__ partial, int gx, const float *__restrict__ s,
                     const float *__restrict__ save_invstd, float *ds, float *db, float *coef, double M, int C,
                     float beta_p)
 {
-    const int lane = threadIdx.x & 63;
-    const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if(c >= C)
-        return;
+    const int c = blockIdx.x;
     const double inv = save_invstd[c];
     const float sv = s[c];
     const float ds_old = beta_p != 0.0f ? ds[c] : 0.0f, db_old = beta_p != 0.0f ? db[c] : 0.0f;
     double s0, s1;
-    sum_partials(partial, gx, C, c, lane, s0, s1);
-    if(lane != 0)
+    sum_partials(partial, gx, C, c, s0, s1);
+    if(threadIdx.x != 0)
         return;
     const double dsv = s1 * inv;
     ds[c] = (float)(beta_p != 0.0f ? dsv + (double)beta_p * ds_old : dsv);
@@ -753,7 +768,7 @@ int saga_hip_bn_train_fwd(const SagaTensorView *x, const SagaTensorView *z, cons
 #define GO(T, VN)                                                                                                   \
     do {                                                                                                            \
         bn_stats_cl<T, VN><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, partial, lx.rows, C, sh.cvb);           \
-        bn_stats_finalize<T><<<(C + 3) / 4, 256, 0, st>>>(partial, sh.gx, (const T *)x->ptr, 1, s, b, run_m,      \
+        bn_stats_finalize<T><<<C, 256, 0, st>>>(partial, sh.gx, (const T *)x->ptr, 1, s, b, run_m,      \
                                                               run_v, save_mean, save_invstd, ss, (double)lx.rows, C, \
                                                               eps, expavg);                                         \
         bn_apply_cl<T, VN, 1><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, add ? (const T *)z->ptr : nullptr,   \
@@ -815,7 +830,7 @@ int saga_hip_bn_train_fwd_partials(const SagaTensorView *x, const SagaTensorView
     dim3 grid(sh.gx, sh.gy);
 #define GO(T, VN)                                                                                                   \
     do {                                                                                                            \
-        bn_stats_finalize<T><<<(C + 3) / 4, 256, 0, st>>>(partial, partial_rows, (const T *)nullptr, 1, s, b, run_m, \
+        bn_stats_finalize<T><<<C, 256, 0, st>>>(partial, partial_rows, (const T *)nullptr, 1, s, b, run_m, \
                                                           run_v, save_mean, save_invstd, ss, (double)lx.rows, C,    \
                                                           eps, expavg);                                             \
         bn_apply_cl<T, VN, 1><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, add ? (const T *)z->ptr : nullptr,   \
@@ -899,7 +914,7 @@ int saga_hip_bn_bwd_ex(const SagaTensorView *x, const SagaTensorView *y, const S
                                                      lx.rows, C, sh.cvb, flags, recompute ? s : nullptr,             \
                                                      recompute ? b : nullptr, recompute ? save_invstd : nullptr,     \
                                                      early_dz ? (T *)dz->ptr : nullptr, ldz.pitch);                  \
-        bn_bwd_finalize<<<(C + 3) / 4, 256, 0, st>>>(partial, sh.gx, s, save_invstd, ds, db, coef,                \
+        bn_bwd_finalize<<<C, 256, 0, st>>>(partial, sh.gx, s, save_invstd, ds, db, coef,                \
                                                          (double)lx.rows, C, beta_p);                                \
         if(early_dz)                                                                                                 \
             bn_bwd_apply_cl<T, VN, false><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, nullptr, 0,              \
