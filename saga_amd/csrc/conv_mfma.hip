@@ -285,6 +285,33 @@ __device__ __forceinline__ unsigned pack2(float a, float b)
     return __builtin_bit_cast(unsigned, v);
 }
 
+// Reads the 32 channels nb .. nb+31 of this lane's pixel row the way the epilogue stores them
+// (16 contiguous bytes per lane: the lower half-wave channels 16q .. 16q+7, the upper one
+// 16q+8 .. 16q+15) and hands every lane the values of ITS accumulator elements: the same
+// half-wave swap as on the way out undoes the regrouping.  All lanes must call it.
+// f[v] belongs to channel nb + 8*(v/4) + 4*hi + v%4.
+__device__ __forceinline__ void load_row32(const half_t *row, bool ok, int nb, int ncols, int hi, float (&f)[16])
+{
+    typedef unsigned u4 __attribute__((ext_vector_type(4)));
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for(int q = 0; q < 2; q++) {
+        const int n = nb + 16 * q + 8 * hi;
+        u4 o = {0, 0, 0, 0};
+        if(ok && n < ncols)
+            o = *(const u4 *)(row + n);
+        const auto s0 = __builtin_amdgcn_permlane32_swap(o[0], o[2], false, false);
+        const auto s1 = __builtin_amdgcn_permlane32_swap(o[1], o[3], false, false);
+        const unsigned w[4] = {s0[0], s1[0], s0[1], s1[1]}; // elements 8q .. 8q+7, two per word
+#pragma unroll
+        for(int e = 0; e < 4; e++) {
+            const h2 v = __builtin_bit_cast(h2, w[e]);
+            f[8 * q + 2 * e] = (float)v[0];
+            f[8 * q + 2 * e + 1] = (float)v[1];
+        }
+    }
+}
+
 // One step of a halving exchange over n live values per lane: the lane with bit m set keeps
 // the upper half, its partner (lane ^ m) the lower half, and each adds what the other held of
 // its half.  n is a template parameter so that every array index is a constant and the
@@ -462,6 +489,10 @@ __global__ void __launch_bounds__(64 * (WGM * WGN + PROD), PROD ? (WGM * WGN + P
                     produce((kt + STAGES - 1) % STAGES);
             }
             if constexpr(!BWD) {
+                if(g.bn_s) { // the two barriers around the folded batch norm's parameter table
+                    __syncthreads();
+                    __syncthreads();
+                }
                 if(g.stats) { // the two barriers of the statistics epilogue
                     __syncthreads();
                     __syncthreads();
@@ -587,6 +618,25 @@ __global__ void __launch_bounds__(64 * (WGM * WGN + PROD), PROD ? (WGM * WGN + P
             advance();
     }
 
+    // Inference with a folded batch norm: scale = s/sqrt(v+eps) and shift = b - m*scale of the
+    // block's BN channels go into LDS once (the stage memory is free after the last slice).
+    float *bnp = (float *)smem;
+    if constexpr(!BWD) {
+        if(g.bn_s) {
+            __syncthreads(); // every wavefront is done reading the last slice
+            if(tid < BN) {
+                const int n = n0 + tid;
+                float sc = 0.0f, sh = 0.0f;
+                if(n < g.Ngemm) {
+                    sc = g.bn_s[n] * rsqrtf(g.bn_v[n] + g.bn_eps);
+                    sh = g.bn_b[n] - g.bn_m[n] * sc;
+                }
+                bnp[tid] = sc;
+                bnp[BN + tid] = sh;
+            }
+            __syncthreads();
+        }
+    }
     // acc[i][j][v]: pixel wm + 32*i + lane%32, channel wn + 32*j + 8*(v/4) + 4*(lane/32) + v%4
     const int hi = lane >> 5;
     const bool vec_ok = (g.ldo & 7) == 0 && (g.Ngemm & 7) == 0 && ((uintptr_t)g.out & 15) == 0;
@@ -616,38 +666,30 @@ __global__ void __launch_bounds__(64 * (WGM * WGN + PROD), PROD ? (WGM * WGN + P
                     f[v] = g.alpha * acc[i][j][v];
                 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
                 if(g.beta != 0.0f) {
+                    float old[16];
+                    load_row32(orow, ok, nb, g.Ngemm, hi, old);
 #pragma unroll
-                    for(int q = 0; q < 4; q++) {
-                        const int n = nb + 8 * q + 4 * hi;
-                        if(ok && n < g.Ngemm) {
-                            const half4_t old = *(const half4_t *)(orow + n);
-#pragma unroll
-                            for(int e = 0; e < 4; e++)
-                                f[4 * q + e] += g.beta * (float)old[e];
-                        }
-                    }
+                    for(int v = 0; v < 16; v++)
+                        f[v] += g.beta * old[v];
                 }
                 if constexpr(!BWD) {
                     if(g.bn_s) {
+                        float zz[16];
+                        if(g.bn_flags & SAGA_BN_ADD)
+                            load_row32(g.z + pix * g.ldz, ok, nb, g.Ngemm, hi, zz);
 #pragma unroll
                         for(int q = 0; q < 4; q++) {
-                            const int n = nb + 8 * q + 4 * hi;
-                            if(n < g.Ngemm) {
-                                const float4_t vs = *(const float4_t *)(g.bn_s + n), vb = *(const float4_t *)(g.bn_b + n);
-                                const float4_t vm = *(const float4_t *)(g.bn_m + n), vv = *(const float4_t *)(g.bn_v + n);
-                                half4_t zz = {0, 0, 0, 0};
-                                if((g.bn_flags & SAGA_BN_ADD) && ok)
-                                    zz = *(const half4_t *)(g.z + pix * g.ldz + n);
+                            // scale and shift of the block's channels were put into LDS after the main loop
+                            const int cl = wn + j * 32 + 8 * q + 4 * hi;
+                            const float4_t sc = *(const float4_t *)(bnp + cl), sh = *(const float4_t *)(bnp + BN + cl);
 #pragma unroll
-                                for(int e = 0; e < 4; e++) {
-                                    const float sc = vs[e] * rsqrtf(vv[e] + g.bn_eps);
-                                    float t = __builtin_fmaf(f[4 * q + e], sc, vb[e] - vm[e] * sc);
-                                    if(g.bn_flags & SAGA_BN_ADD)
-                                        t += (float)zz[e];
-                                    if(g.bn_flags & SAGA_BN_RELU)
-                                        t = (t != t) ? t : fmaxf(t, 0.0f);
-                                    f[4 * q + e] = t;
-                                }
+                            for(int e = 0; e < 4; e++) {
+                                float t = __builtin_fmaf(f[4 * q + e], sc[e], sh[e]);
+                                if(g.bn_flags & SAGA_BN_ADD)
+                                    t += zz[4 * q + e];
+                                if(g.bn_flags & SAGA_BN_RELU)
+                                    t = (t != t) ? t : fmaxf(t, 0.0f);
+                                f[4 * q + e] = t;
                             }
                         }
                     }
