@@ -1583,14 +1583,12 @@ static bool set_bn(GatherArgs &a, const ConvBnFold *bn, const SagaTensorView *y,
         CLInfo lz;
         if(!bn->z || bn->z->dtype != SAGA_HALF || !same_dims(bn->z, y) || !as_channels_last(bn->z, &lz) || lz.rows != ly.rows)
             return false;
-        // 8-byte loads of 4 channels
-        if(lz.pitch % 4 || ((uintptr_t)bn->z->ptr & 7) || ((uintptr_t)bn->s & 15) || ((uintptr_t)bn->b & 15) ||
-           ((uintptr_t)bn->m & 15) || ((uintptr_t)bn->v & 15))
+        // where the epilogue stores 16-byte vectors it also reads the residual in 16-byte vectors
+        const bool vec = ly.pitch % 8 == 0 && y->dims[1] % 8 == 0 && aligned16(y->ptr);
+        if(vec && (lz.pitch % 8 || !aligned16(bn->z->ptr)))
             return false;
         a.z = (const half_t *)bn->z->ptr;
         a.ldz = (int)lz.pitch;
-    } else if(((uintptr_t)bn->s & 15) || ((uintptr_t)bn->b & 15) || ((uintptr_t)bn->m & 15) || ((uintptr_t)bn->v & 15)) {
-        return false;
     }
     return true;
 }
