@@ -158,11 +158,15 @@ int saga_hip_bn_train_fwd(const SagaTensorView *x, const SagaTensorView *z, cons
                           size_t ws_bytes, saga_stream_t stream);
 /* training forward from per-channel partial sums of x that already exist (the output of
  * saga_hip_conv2d_fwd_bnstats): finalises the statistics and normalises, without the pass
- * over x that computes them.  workspace: 2*C floats.  Channels-last tensors only. */
+ * over x that computes them.  workspace: 2*C floats.  Channels-last tensors only.
+ * relu_mask (may be NULL; fp16 with C % 8 == 0 and SAGA_BN_RELU only): rows*C/8 bytes, bit j of byte
+ * [row][c/8] set where y[row][c - c%8 + j] > 0 - the role of cuDNN's reserve space for the fused
+ * add + relu operation (src/cuda/cuda_dnn.cpp:2095-2136); saga_hip_bn_bwd_ex reads it in place of y. */
 int saga_hip_bn_train_fwd_partials(const SagaTensorView *x, const SagaTensorView *z, const SagaTensorView *y,
                                    const float *s, const float *b, float *run_m, float *run_v, float *save_mean,
                                    float *save_invstd, float eps, float expavg, int flags, const float *partial,
-                                   int partial_rows, void *workspace, size_t ws_bytes, saga_stream_t stream);
+                                   int partial_rows, uint8_t *relu_mask, void *workspace, size_t ws_bytes,
+                                   saga_stream_t stream);
 int saga_hip_bn_bwd(const SagaTensorView *x, const SagaTensorView *y, const SagaTensorView *dy,
                     const SagaTensorView *dx, const SagaTensorView *dz, const float *s, const float *save_mean,
                     const float *save_invstd, float *ds, float *db, float beta_dx, float beta_dz, float beta_p,
@@ -171,12 +175,14 @@ int saga_hip_bn_bwd(const SagaTensorView *x, const SagaTensorView *y, const Saga
 /* bwd with the bias b at hand, as cudnnBatchNormalizationBackwardEx receives it
  * (src/cuda/cuda_dnn.cpp:2138-2163): for SAGA_BN_RELU without SAGA_BN_ADD on channels-last tensors
  * the relu mask is recomputed from x (the forward's own expression, rounded as it was stored)
- * and y may be NULL - one tensor less to read in each of the two passes.  b NULL: as saga_hip_bn_bwd. */
+ * and y may be NULL - one tensor less to read in each of the two passes.  b NULL: as saga_hip_bn_bwd.
+ * relu_mask (may be NULL): the bytes saga_hip_bn_train_fwd_partials left; where the masked gradient goes
+ * to dz first (SAGA_BN_ADD, beta_dz == 0, fp16 channels-last) they replace the read of y. */
 int saga_hip_bn_bwd_ex(const SagaTensorView *x, const SagaTensorView *y, const SagaTensorView *dy,
                        const SagaTensorView *dx, const SagaTensorView *dz, const float *s, const float *b,
                        const float *save_mean, const float *save_invstd, float *ds, float *db, float beta_dx,
-                       float beta_dz, float beta_p, int flags, void *workspace, size_t ws_bytes,
-                       saga_stream_t stream);
+                       float beta_dz, float beta_p, int flags, const uint8_t *relu_mask, void *workspace,
+                       size_t ws_bytes, saga_stream_t stream);
 
 /* ---- activations: cudnnActivationForward / Backward (src/cuda/cuda_dnn.cpp:631-638, :668-676),
  *      leaky relu kernel (src/cuda/cuda_kernels.cu:478-495).  y = act(x) + beta*y ; dx = dy*act'(x) + beta*dx. */

@@ -93,8 +93,10 @@ __global__ void __launch_bounds__(256)
     bn_apply_cl(const T *__restrict__ x, int64_t px, const T *__restrict__ z, int64_t pz, T *__restrict__ y, int64_t py,
                 const float *__restrict__ s, const float *__restrict__ b, const float *__restrict__ m,
                 const float *__restrict__ v, const float *__restrict__ ss, float eps, int64_t rows, int C, int cvb,
-                int flags)
+                int flags, uint8_t *__restrict__ mask = nullptr)
 {
+    // mask (VN == 8 only): one byte per row and 8-channel vector, bit j set where the stored y is > 0;
+    // the backward pass of a fused add + relu layer reads it instead of y
     const int tx = threadIdx.x % cvb, ty = threadIdx.x / cvb, rb = 256 / cvb;
     const int c0 = (blockIdx.y * cvb + tx) * VN;
     if(c0 >= C)
@@ -130,6 +132,15 @@ __global__ void __launch_bounds__(256)
             o[j] = t;
         }
         L::store(y + r * py + c0, o);
+        if constexpr(VN == 8) {
+            if(mask) {
+                unsigned bits = 0;
+#pragma unroll
+                for(int j = 0; j < VN; j++)
+                    bits |= ((float)(T)o[j] > 0.0f ? 1u : 0u) << j;
+                mask[r * (C / VN) + c0 / VN] = (uint8_t)bits;
+            }
+        }
     };
     int64_t r = (int64_t)blockIdx.x * rb + ty;
     for(; r + 3 * stride < rows; r += 4 * stride) {
@@ -314,8 +325,10 @@ __global__ void __launch_bounds__(256)
     bn_bwd_stats_cl(const T *__restrict__ x, int64_t px, const T *__restrict__ y, int64_t py, const T *__restrict__ dy,
                     int64_t pdy, const float *__restrict__ save_mean, float *__restrict__ partial, int64_t rows, int C,
                     int cvb, int flags, const float *__restrict__ rs, const float *__restrict__ rb_, const float *__restrict__ rinv,
-                    T *__restrict__ dz, int64_t pdz)
+                    T *__restrict__ dz, int64_t pdz, const uint8_t *__restrict__ mask = nullptr)
 {
+    // mask set (VN == 8): the relu mask comes from the byte per row and channel vector that the
+    // forward pass left, and y is not read
     // dz set: the masked gradient dy' is stored there on the way (it is the residual branch's
     // gradient anyway), and the second pass reads it instead of y and dy
     // rs/rb_/rinv (scale, bias, saved 1/std) set: the relu mask is recomputed from x as
@@ -339,12 +352,14 @@ __global__ void __launch_bounds__(256)
         typedef Ld<T, VN> L;
         typedef typename L::V V;
         const int64_t stride = (int64_t)gridDim.x * rb;
-        auto add = [&](const V &xr, const V &gr, const V &yr, int64_t r) {
+        auto add = [&](const V &xr, const V &gr, const V &yr, unsigned mb, int64_t r) {
             float gm[VN];
 #pragma unroll
             for(int j = 0; j < VN; j++) {
                 float g = L::at(gr, j);
-                const float yv = recompute ? (float)(T)__builtin_fmaf(L::at(xr, j), sc[j], sh[j]) : L::at(yr, j);
+                const float yv = recompute ? (float)(T)__builtin_fmaf(L::at(xr, j), sc[j], sh[j])
+                                 : mask    ? (float)((mb >> j) & 1u)
+                                           : L::at(yr, j);
                 if(relu && !(yv > 0.0f))
                     g = 0.0f;
                 a0[j] += g;
@@ -355,21 +370,24 @@ __global__ void __launch_bounds__(256)
                 L::store(dz + r * pdz + c0, gm);
         };
         int64_t r = (int64_t)blockIdx.x * rb + ty;
+        const int mp = C / VN, mc = c0 / VN; // mask row pitch and this thread's byte
         for(; r + 3 * stride < rows; r += 4 * stride) {
             V xr[4], gr[4], yr[4];
+            unsigned mb[4];
 #pragma unroll
             for(int u = 0; u < 4; u++) {
                 xr[u] = L::raw(x + (r + u * stride) * px + c0);
                 gr[u] = L::raw(dy + (r + u * stride) * pdy + c0);
-                yr[u] = relu && !recompute ? L::raw(y + (r + u * stride) * py + c0) : gr[u];
+                yr[u] = relu && !recompute && !mask ? L::raw(y + (r + u * stride) * py + c0) : gr[u];
+                mb[u] = mask ? mask[(r + u * stride) * mp + mc] : 0u;
             }
 #pragma unroll
             for(int u = 0; u < 4; u++)
-                add(xr[u], gr[u], yr[u], r + u * stride);
+                add(xr[u], gr[u], yr[u], mb[u], r + u * stride);
         }
         for(; r < rows; r += stride) {
             const V xr = L::raw(x + r * px + c0), gr = L::raw(dy + r * pdy + c0);
-            add(xr, gr, relu && !recompute ? L::raw(y + r * py + c0) : gr, r);
+            add(xr, gr, relu && !recompute && !mask ? L::raw(y + r * py + c0) : gr, mask ? mask[r * mp + mc] : 0u, r);
         }
     }
 #pragma unroll
@@ -806,7 +824,8 @@ int saga_hip_bn_train_fwd(const SagaTensorView *x, const SagaTensorView *z, cons
 int saga_hip_bn_train_fwd_partials(const SagaTensorView *x, const SagaTensorView *z, const SagaTensorView *y,
                                    const float *s, const float *b, float *run_m, float *run_v, float *save_mean,
                                    float *save_invstd, float eps, float expavg, int flags, const float *partial,
-                                   int partial_rows, void *workspace, size_t ws_bytes, saga_stream_t stream)
+                                   int partial_rows, uint8_t *relu_mask, void *workspace, size_t ws_bytes,
+                                   saga_stream_t stream)
 {
     if(!valid_view(x) || !valid_view(y) || !s || !b || !partial || partial_rows < 1)
         return SAGA_HIP_EINVAL;
@@ -826,6 +845,9 @@ int saga_hip_bn_train_fwd_partials(const SagaTensorView *x, const SagaTensorView
     hipStream_t st = as_stream(stream);
     float *ss = (float *)workspace;
     const int vn = vec_width(x->dtype, C, {x, y, add ? z : nullptr}, {lx.pitch, ly.pitch, add ? lz.pitch : 0});
+    // the mask has one byte per 8 fp16 channels: only the 8-wide fp16 kernel with relu writes it
+    if(relu_mask && !(x->dtype == SAGA_HALF && vn == 8 && (flags & SAGA_BN_RELU)))
+        return SAGA_HIP_EUNSUPPORTED;
     Shape sh = plan(lx.rows, C / vn);
     dim3 grid(sh.gx, sh.gy);
 #define GO(T, VN)                                                                                                   \
@@ -835,7 +857,7 @@ int saga_hip_bn_train_fwd_partials(const SagaTensorView *x, const SagaTensorView
                                                           eps, expavg);                                             \
         bn_apply_cl<T, VN, 1><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, add ? (const T *)z->ptr : nullptr,   \
                                                     lz.pitch, (T *)y->ptr, ly.pitch, nullptr, nullptr, nullptr,     \
-                                                    nullptr, ss, eps, lx.rows, C, sh.cvb, flags);                   \
+                                                    nullptr, ss, eps, lx.rows, C, sh.cvb, flags, relu_mask);        \
     } while(0)
     if(x->dtype == SAGA_HALF) {
         if(vn == 8) GO(half_t, 8); else GO(half_t, 1);
@@ -853,14 +875,14 @@ int saga_hip_bn_bwd(const SagaTensorView *x, const SagaTensorView *y, const Saga
                     int flags, void *workspace, size_t ws_bytes, saga_stream_t stream)
 {
     return saga_hip_bn_bwd_ex(x, y, dy, dx, dz, s, nullptr, save_mean, save_invstd, ds, db, beta_dx, beta_dz, beta_p,
-                              flags, workspace, ws_bytes, stream);
+                              flags, nullptr, workspace, ws_bytes, stream);
 }
 
 int saga_hip_bn_bwd_ex(const SagaTensorView *x, const SagaTensorView *y, const SagaTensorView *dy,
                        const SagaTensorView *dx, const SagaTensorView *dz, const float *s, const float *b,
                        const float *save_mean, const float *save_invstd, float *ds, float *db, float beta_dx,
-                       float beta_dz, float beta_p, int flags, void *workspace, size_t ws_bytes,
-                       saga_stream_t stream)
+                       float beta_dz, float beta_p, int flags, const uint8_t *relu_mask, void *workspace,
+                       size_t ws_bytes, saga_stream_t stream)
 {
     if(!valid_view(x) || !valid_view(dy) || !valid_view(dx) || !s || !save_mean || !save_invstd || !ds || !db)
         return SAGA_HIP_EINVAL;
@@ -900,6 +922,8 @@ int saga_hip_bn_bwd_ex(const SagaTensorView *x, const SagaTensorView *y, const S
         // residual layers: the first pass leaves dy' in dz, the second reads it in place of y and dy
         const bool early_dz = dz && beta_dz == 0.0f && relu && !recompute && dz->ptr != dy->ptr && dz->ptr != x->ptr &&
                               dz->ptr != y->ptr;
+        // the forward pass's relu mask replaces y where only the first pass needs it
+        const uint8_t *mk = relu_mask && early_dz && dt == SAGA_HALF && vn == 8 ? relu_mask : nullptr;
 #define GO(T, VN)                                                                                                    \
     do {                                                                                                             \
         if(recompute)                                                                                                \
@@ -913,7 +937,7 @@ int saga_hip_bn_bwd_ex(const SagaTensorView *x, const SagaTensorView *y, const S
                                                      ly.pitch, (const T *)dy->ptr, ldy.pitch, save_mean, partial,    \
                                                      lx.rows, C, sh.cvb, flags, recompute ? s : nullptr,             \
                                                      recompute ? b : nullptr, recompute ? save_invstd : nullptr,     \
-                                                     early_dz ? (T *)dz->ptr : nullptr, ldz.pitch);                  \
+                                                     early_dz ? (T *)dz->ptr : nullptr, ldz.pitch, mk);              \
         bn_bwd_finalize<<<C, 256, 0, st>>>(partial, sh.gx, s, save_invstd, ds, db, coef,                \
                                                          (double)lx.rows, C, beta_p);                                \
         if(early_dz)                                                                                                 \

@@ -51,10 +51,10 @@ SIGNATURES = {
     "saga_hip_bn_infer": (_I, [_TV, _TV, _TV, _VP, _VP, _VP, _VP, _F, _I, _VP]),
     "saga_hip_bn_workspace_size": (_SZ, [_TV]),
     "saga_hip_bn_train_fwd": (_I, [_TV, _TV, _TV, _VP, _VP, _VP, _VP, _VP, _VP, _F, _F, _I, _VP, _SZ, _VP]),
-    "saga_hip_bn_train_fwd_partials": (_I, [_TV, _TV, _TV, _VP, _VP, _VP, _VP, _VP, _VP, _F, _F, _I, _VP, _I, _VP,
+    "saga_hip_bn_train_fwd_partials": (_I, [_TV, _TV, _TV, _VP, _VP, _VP, _VP, _VP, _VP, _F, _F, _I, _VP, _I, _VP, _VP,
                                             _SZ, _VP]),
     "saga_hip_bn_bwd": (_I, [_TV, _TV, _TV, _TV, _TV, _VP, _VP, _VP, _VP, _VP, _F, _F, _F, _I, _VP, _SZ, _VP]),
-    "saga_hip_bn_bwd_ex": (_I, [_TV, _TV, _TV, _TV, _TV, _VP, _VP, _VP, _VP, _VP, _VP, _F, _F, _F, _I, _VP, _SZ,
+    "saga_hip_bn_bwd_ex": (_I, [_TV, _TV, _TV, _TV, _TV, _VP, _VP, _VP, _VP, _VP, _VP, _F, _F, _F, _I, _VP, _VP, _SZ,
                                 _VP]),
     "saga_hip_act_fwd": (_I, [_I, _F, _TV, _TV, _F, _VP]),
     "saga_hip_act_bwd": (_I, [_I, _F, _TV, _TV, _TV, _TV, _F, _VP]),

@@ -717,6 +717,11 @@ struct BnTrain : public HipOperation {
     float expavg_ = NAN;
     float m_beta_ = 1.0f, v_beta_ = 1.0f; // running statistics are read-modify-write
     std::shared_ptr<ConvStatsLink> stats_; // the producer of x leaves the per-channel sums here
+    // fused add + relu on fp16 channels-last tensors: one bit per element (stored y > 0), which the
+    // backward pass reads instead of y (the role of cuDNN's reserve space, reference :2095-2136);
+    // mask_valid_ says whether the forward pass of this step wrote it
+    T mask_;
+    bool mask_valid_ = false;
     BnTrain(HipProgram &p, T x, T z, T s, T b, T m, T v, T y, T sm, T sv, float eps, int flags)
       : HipOperation(flags ? "bntrain.fused" : "bntrain")
       , x_(x), z_(z), s_(s), b_(b), m_(m), v_(v), y_(y), sm_(sm), sv_(sv), eps_(eps), flags_(flags)
@@ -733,15 +738,18 @@ struct BnTrain : public HipOperation {
         SagaTensorView vz;
         if(z_)
             vz = z_->view();
+        mask_valid_ = false;
         if(stats_ && stats_->valid) {
             stats_->valid = false;
             const int r = saga_hip_bn_train_fwd_partials(
                 &vx, z_ ? &vz : nullptr, &vy, (const float *)s_->deviceMem(), (const float *)b_->deviceMem(),
                 (float *)m_->deviceMem(), (float *)v_->deviceMem(), (float *)sm_->deviceMem(), (float *)sv_->deviceMem(),
-                eps_, expavg_, flags_, (const float *)stats_->partial->m_ptr, stats_->rows, p.m_ctx->m_workspace.ptr(),
-                p.m_ctx->m_workspace.size(), S(p));
+                eps_, expavg_, flags_, (const float *)stats_->partial->m_ptr, stats_->rows,
+                mask_ ? (uint8_t *)mask_->deviceMem() : nullptr, p.m_ctx->m_workspace.ptr(), p.m_ctx->m_workspace.size(),
+                S(p));
             if(r == 0) {
                 expavg_ = p.m_pc.bn_expavg;
+                mask_valid_ = mask_ != nullptr;
                 return;
             }
             if(r != SAGA_HIP_EUNSUPPORTED)
@@ -761,9 +769,15 @@ struct BnTrain : public HipOperation {
             r.push_back({"z", z_});
         return r;
     }
-    HipOpArgs listOutputs() const override { return {{"y", y_}, {"m", m_}, {"v", v_}, {"sm", sm_}, {"sv", sv_}}; }
+    HipOpArgs listOutputs() const override
+    {
+        HipOpArgs r{{"y", y_}, {"m", m_}, {"v", v_}, {"sm", sm_}, {"sv", sv_}};
+        if(mask_)
+            r.push_back({"mask", mask_});
+        return r;
+    }
     // statistics pass reads x (unless the producer supplied the sums), normalise pass reads x (+z), writes y
-    double bytes() const override { return ((z_ ? 4 : 3) - (stats_ ? 1 : 0)) * nbytes(x_); }
+    double bytes() const override { return ((z_ ? 4 : 3) - (stats_ ? 1 : 0) + (mask_ ? 0.0625 : 0)) * nbytes(x_); }
     float *getBeta(const T &t) override
     {
         if(t == m_)
@@ -798,6 +812,7 @@ struct BnBwd : public HipOperation {
                                 (const float *)fwd_->sm_->deviceMem(),
                                 (const float *)fwd_->sv_->deviceMem(), (float *)ds_->deviceMem(),
                                 (float *)db_->deviceMem(), dx_beta_, dz_beta_, ds_beta_, flags_,
+                                fwd_->mask_valid_ ? (const uint8_t *)fwd_->mask_->deviceMem() : nullptr,
                                 p.m_ctx->m_workspace.ptr(), p.m_ctx->m_workspace.size(), S(p)));
     }
     HipOpArgs listInputs() const override
@@ -805,6 +820,8 @@ struct BnBwd : public HipOperation {
         HipOpArgs r{{"x", fwd_->x_}, {"dy", dy_}, {"s", fwd_->s_}, {"sm", fwd_->sm_}, {"sv", fwd_->sv_}};
         if(flags_ & SAGA_BN_RELU)
             r.push_back({"y", fwd_->y_});
+        if(fwd_->mask_)
+            r.push_back({"mask", fwd_->mask_});
         return r;
     }
     HipOpArgs listOutputs() const override
@@ -827,8 +844,8 @@ struct BnBwd : public HipOperation {
     {
         const double e = nbytes(dx_);
         const bool reads_y = (flags_ & SAGA_BN_RELU) && (flags_ & SAGA_BN_ADD);
-        if(reads_y && dz_ && dz_beta_ == 0) // pass 1: x, y, dy -> dz ; pass 2: x, dz -> dx
-            return e * (7 + (dx_beta_ != 0 ? 1 : 0));
+        if(reads_y && dz_ && dz_beta_ == 0) // pass 1: x, y (or its 1-bit mask), dy -> dz ; pass 2: x, dz -> dx
+            return e * ((fwd_->mask_ ? 6.0625 : 7) + (dx_beta_ != 0 ? 1 : 0));
         return e * (4 + (reads_y ? 2 : 0) + 1 + (dz_ ? 1 : 0) + (dx_beta_ != 0 ? 1 : 0) +
                     (dz_ && dz_beta_ != 0 ? 1 : 0));
     }
@@ -893,6 +910,14 @@ void batchnorm_lower(HipProgram &p, HipProgramUnit &pu, const Node &n, std::shar
     // if the op that wrote x last is a convolution and nothing else writes x, take the sums from it
     if(ConvFwd *producer = conv_producer())
         f->stats_ = producer->offerStats();
+    // residual + relu on fp16 channels-last tensors with whole 8-channel vectors, statistics from
+    // the convolution: the forward pass also leaves the relu mask, one bit per element
+    if(f->stats_ && z && (flags & SAGA_BN_RELU) && (flags & SAGA_BN_ADD) && x->m_data_type == Tensor::DataType::HALF &&
+       x->m_dims.size() == 4 && x->cpacked() && y->cpacked() && (int)x->m_dims[1] % 8 == 0 && !getenv("SAGA_HIP_NO_RELU_MASK")) {
+        const Dims md{x->m_dims[0], (int64_t)((int)x->m_dims[1] / 8), x->m_dims[2], x->m_dims[3]};
+        f->mask_ = std::make_shared<HipTensor>(Tensor::DataType::U8, md, HipLayout::NHWC, p.m_ctx.get(),
+                                               n.m_outputs["y"]->namePostfix("relumask"));
+    }
     pu.fwd(f);
 
     auto dx = p.lowerGrad(pu, xh);

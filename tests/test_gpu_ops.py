@@ -160,10 +160,13 @@ def test_conv_bnstats_then_bn_from_partials(case):
     sd, bd, md, vd = (dev(t) for t in (s, b, m, v))
     sm, sv = dev(np.zeros(Kk, np.float32)), dev(np.zeros(Kk, np.float32))
     ws2 = torch.zeros(2 * Kk, dtype=torch.float32, device="cuda")
+    # the relu mask (one bit per element) exists for fp16 tensors with whole 8-channel vectors
+    want_mask = fused and Kk % 8 == 0
+    mask = torch.zeros(max(1, int(np.prod(y_ref.shape)) // 8), dtype=torch.uint8, device="cuda")
     K.check(L.saga_hip_bn_train_fwd_partials(C.byref(K.view(yd)), C.byref(K.view(zd)) if fused else None,
                                              C.byref(K.view(od)), K.ptr(sd), K.ptr(bd), K.ptr(md), K.ptr(vd),
                                              K.ptr(sm), K.ptr(sv), 1e-5, 0.1, flags, K.ptr(partial), rows.value,
-                                             K.ptr(ws2), ws2.numel() * 4, S()))
+                                             K.ptr(mask) if want_mask else None, K.ptr(ws2), ws2.numel() * 4, S()))
     o_ref, rsm, rsv, rm, rv = ref.bn_train_fwd(host(yd), s, b, m, v, 1e-5, 0.1)
     if fused:
         o_ref = ref.act_fwd(o_ref + z)
@@ -172,6 +175,28 @@ def test_conv_bnstats_then_bn_from_partials(case):
     assert_close(host(sv), rsv, torch.float32, "saved invstd", 1e-3)
     assert_close(host(md), rm, torch.float32, "running mean", 1e-3)
     assert_close(host(vd), rv, torch.float32, "running var", 1e-3)
+    if want_mask:
+        # bit j of byte [pixel][c/8] <-> the stored y[pixel][8*(c/8)+j] > 0, bit-exact
+        y_dev = host(od).transpose(0, 2, 3, 1).reshape(-1, Kk // 8, 8)
+        bits = np.unpackbits(mask.cpu().numpy().reshape(-1, Kk // 8, 1), axis=2, bitorder="little")
+        np.testing.assert_array_equal(bits.astype(bool), y_dev > 0)
+        # backward with the mask in place of y: y is passed poisoned, so any read of it would show
+        dy = rnd(rng, *y_ref.shape, dtype=dtype)
+        dyp = dy * (host(od) > 0)
+        dx_ref, ds_ref, db_ref = ref.bn_bwd(host(yd), dyp, s, host(sm), host(sv))
+        dyd = dev(dy, dtype, "nhwc")
+        dxd, dzd = dev(np.zeros_like(y_ref), dtype, "nhwc"), dev(np.zeros_like(y_ref), dtype, "nhwc")
+        poisoned = dev(np.full_like(y_ref, -1.0), dtype, "nhwc")
+        dsd, dbd = dev(np.zeros(Kk, np.float32)), dev(np.zeros(Kk, np.float32))
+        vx = K.view(yd)
+        wsb = torch.zeros(L.saga_hip_bn_workspace_size(C.byref(vx)), dtype=torch.uint8, device="cuda")
+        K.check(L.saga_hip_bn_bwd_ex(C.byref(vx), C.byref(K.view(poisoned)), C.byref(K.view(dyd)), C.byref(K.view(dxd)),
+                                     C.byref(K.view(dzd)), K.ptr(sd), K.ptr(bd), K.ptr(sm), K.ptr(sv), K.ptr(dsd),
+                                     K.ptr(dbd), 0.0, 0.0, 0.0, flags, K.ptr(mask), K.ptr(wsb), wsb.numel(), S()))
+        assert_close(host(dzd), dyp, dtype, "bn dz (mask bits)")
+        assert_close(host(dxd), dx_ref, dtype, "bn dx (mask bits)")
+        assert_close(host(dsd), ds_ref, torch.float32, "bn ds (mask bits)", 5e-3)
+        assert_close(host(dbd), db_ref, torch.float32, "bn db (mask bits)", 5e-3)
 
 
 @pytest.mark.parametrize("dtype", DT)
@@ -324,7 +349,7 @@ def test_batchnorm(shape, flags, layout, padc, dtype):
         y_arg = None if layout.startswith("nhwc") else C.byref(K.view(yd))  # only channels-last can do without y
         K.check(L.saga_hip_bn_bwd_ex(C.byref(K.view(xd)), y_arg, C.byref(K.view(dyd)), C.byref(K.view(dx2)), None,
                                      K.ptr(sd), K.ptr(bd), K.ptr(sm), K.ptr(sv), K.ptr(dsd), K.ptr(dbd), 0.0, 0.0,
-                                     0.0, flags, K.ptr(ws), ws.numel(), S()))
+                                     0.0, flags, None, K.ptr(ws), ws.numel(), S()))
         assert_close(host(dx2), dx2_ref, dtype, "bn dx (mask from x)")
         assert_close(host(dsd), ds2_ref, torch.float32, "bn ds (mask from x)", 1e-4 if dtype == torch.float32 else 5e-3)
         assert_close(host(dbd), db2_ref, torch.float32, "bn db (mask from x)", 1e-4 if dtype == torch.float32 else 5e-3)
