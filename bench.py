@@ -38,9 +38,9 @@ CONV_KINDS = ("convfwd", "convbwddata", "convbwdfilter")
 MEASURED_HBM_BYTES_PER_LAUNCH = {
     # the counters cannot tell fused from plain batch-norm launches (same kernels): both kinds carry
     # the average over all 53 batch-norm launches of a step
-    "bnbwd.fused": 666482496, "bnbwd": 666482496,
-    "bntrain.fused": 275032221, "bntrain": 275032221,
-    "convfwd": 268755817, "convbwddata": 290992982, "convbwdfilter": 308649991,
+    "bnbwd.fused": 635763596, "bnbwd": 635763596,
+    "bntrain.fused": 285295384, "bntrain": 285295384,
+    "convfwd": 263599419, "convbwddata": 287505075, "convbwdfilter": 308654371,
 }
 
 
@@ -61,6 +61,30 @@ def by_kind(rows):
         a["bytes"] += r["bytes"]
         a["roof_ms"] += max(r["flops"] / (PEAK_FP16_TFLOPS * 1e12), r["bytes"] / (PEAK_HBM_GBS * 1e9)) * 1e3
     return list(agg.values())
+
+
+def write_per_op(path, rows, steps):
+    """One line per operation, in program order: average time per launch, achieved rate, the time its
+    algorithmic flops and bytes would take at the MFMA and HBM peaks, and which of the two bounds it."""
+    def pos(r):
+        return int(r["kind"].split("#")[1]) if "#" in r["kind"] else 0
+    with open(path, "w") as f:
+        f.write(f"per-operation profile of one training step (average over {steps} steps, HIP events on the engine's stream)\n")
+        f.write("  #  kind                    us  GFLOP      MB   TFLOP/s    GB/s  bound  roof_us  frac\n")
+        tot = roof = 0.0
+        for r in sorted(rows, key=pos):
+            if r["launches"] == 0:
+                continue
+            us = r["ms"] * 1e3 / r["launches"]
+            fl, by = r["flops"] / r["launches"], r["bytes"] / r["launches"]
+            t_m, t_h = fl / (PEAK_FP16_TFLOPS * 1e12) * 1e6, by / (PEAK_HBM_GBS * 1e9) * 1e6
+            bound = max(t_m, t_h)
+            tot += us
+            roof += bound
+            f.write(f"{pos(r):3d}  {r['kind'].split('#')[0]:18s} {us:8.1f} {fl / 1e9:6.1f} {by / 1e6:7.1f} "
+                    f"{fl / us / 1e6 if us else 0:9.1f} {by / us / 1e3 if us else 0:7.0f}  {'mfma' if t_m >= t_h else 'hbm':5s} "
+                    f"{bound:7.1f}  {bound / us if us else 0:.3f}\n")
+        f.write(f"sum of operations {tot / 1e3:.3f} ms, sum of roofline bounds {roof / 1e3:.3f} ms, fraction {roof / tot:.3f}\n")
 
 
 def profile_rows(rows):
@@ -133,6 +157,8 @@ def main():
     ap.add_argument("--cpu-batch", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-profile", action="store_true")
+    ap.add_argument("--per-op", metavar="FILE",
+                    help="also write one line per operation of the training step (time, rate, own roofline bound)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run a plain 1 GiB device copy five times and exit (reference for the HBM counters)")
     args = ap.parse_args()
@@ -184,7 +210,10 @@ def main():
     if not args.no_profile:
         train.set_profiling(True)
         train.run(args.steps)
-        rows = by_kind(train.profile())
+        raw = train.profile()
+        if args.per_op:
+            write_per_op(args.per_op, raw, args.steps)
+        rows = by_kind(raw)
         kernels = profile_rows(rows)
         train.set_profiling(False)
         if kernels:
