@@ -50,7 +50,7 @@ size_t saga_hip_conv2d_workspace_size(int kind, const SagaTensorView *x, const S
     ConvGeom g;
     if(geometry(x, w, y, p, &g))
         return 0;
-    return conv_mfma_workspace(kind, x, w, y, g);
+    return std::max(conv_mfma_workspace(kind, x, w, y, g), conv_f32_workspace(kind, x, w, y, g));
 }
 
 int saga_hip_conv2d_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y,
@@ -63,6 +63,9 @@ int saga_hip_conv2d_fwd(const SagaTensorView *x, const SagaTensorView *w, const 
         return r;
     if(!force_direct()) {
         r = conv_mfma_fwd(x, w, y, g, alpha, beta, workspace, ws_bytes, as_stream(stream));
+        if(r != SAGA_HIP_EUNSUPPORTED)
+            return r;
+        r = conv_f32_fwd(x, w, y, g, alpha, beta, workspace, ws_bytes, as_stream(stream));
         if(r != SAGA_HIP_EUNSUPPORTED)
             return r;
     }
@@ -123,6 +126,9 @@ int saga_hip_conv2d_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, 
         r = conv_mfma_bwd_data(dy, w, dx, g, alpha, beta, workspace, ws_bytes, as_stream(stream));
         if(r != SAGA_HIP_EUNSUPPORTED)
             return r;
+        r = conv_f32_bwd_data(dy, w, dx, g, alpha, beta, workspace, ws_bytes, as_stream(stream));
+        if(r != SAGA_HIP_EUNSUPPORTED)
+            return r;
     }
     return conv_direct_bwd_data(dy, w, dx, g, alpha, beta, as_stream(stream));
 }
@@ -137,6 +143,9 @@ int saga_hip_conv2d_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy
         return r;
     if(!force_direct()) {
         r = conv_mfma_bwd_filter(x, dy, dw, g, alpha, beta, workspace, ws_bytes, as_stream(stream));
+        if(r != SAGA_HIP_EUNSUPPORTED)
+            return r;
+        r = conv_f32_bwd_filter(x, dy, dw, g, alpha, beta, workspace, ws_bytes, as_stream(stream));
         if(r != SAGA_HIP_EUNSUPPORTED)
             return r;
     }

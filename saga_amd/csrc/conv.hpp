@@ -38,3 +38,13 @@ int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const 
                        const ConvGeom &g, float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st);
 int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, const SagaTensorView *dw,
                          const ConvGeom &g, float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st);
+
+// fp32 MFMA implicit-GEMM kernels (any strides, groups == 1); SAGA_HIP_EUNSUPPORTED otherwise.
+size_t conv_f32_workspace(int kind, const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y,
+                          const ConvGeom &g);
+int conv_f32_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y, const ConvGeom &g, float alpha,
+                 float beta, void *ws, size_t ws_bytes, hipStream_t st);
+int conv_f32_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx, const ConvGeom &g,
+                      float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st);
+int conv_f32_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, const SagaTensorView *dw, const ConvGeom &g,
+                        float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st);
