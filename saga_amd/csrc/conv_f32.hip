@@ -17,17 +17,19 @@
 
 namespace {
 
-struct KTab {
-    long long a_off; // offset of the channel in the gathered tensor (c*sC or k*sC)
-    long long b_off; // offset of the filter element, without the GEMM-column term
-    int dr, ds;      // tap displacement r*dil, s*dil
+struct KTabA {
+    long long off; // generic: offset of the channel in the gathered tensor; linear: that plus the tap's displacement
+    int dr, ds;    // generic: tap displacement r*dil, s*dil; linear: dr = tap number r*S + s
 };
 
 struct TabArgs {
-    KTab *tab;
+    KTabA *ta;
+    long long *tb;            // offset of the filter element, without the GEMM-column term
     int n, RS, S, dil;
     long long a_sc;           // channel stride of the gathered tensor
     long long w_s_red, w_s2, w_s3; // filter strides: reduction channel, r, s
+    long long lin_sh, lin_sw; // linear form: +-dil*sH, +-dil*sW of the gathered tensor; 0,0 selects the generic form
+    int linear;
 };
 
 __global__ void __launch_bounds__(256) f32_build_ktab(TabArgs a)
@@ -37,26 +39,33 @@ __global__ void __launch_bounds__(256) f32_build_ktab(TabArgs a)
         return;
     const int ch = k / a.RS, rs = k - ch * a.RS;
     const int r = rs / a.S, s = rs - r * a.S;
-    KTab t;
-    t.a_off = ch * a.a_sc;
-    t.b_off = ch * a.w_s_red + r * a.w_s2 + s * a.w_s3;
-    t.dr = r * a.dil;
-    t.ds = s * a.dil;
-    a.tab[k] = t;
+    KTabA t;
+    if(a.linear) {
+        t.off = ch * a.a_sc + r * a.lin_sh + s * a.lin_sw;
+        t.dr = rs;
+        t.ds = 0;
+    } else {
+        t.off = ch * a.a_sc;
+        t.dr = r * a.dil;
+        t.ds = s * a.dil;
+    }
+    a.ta[k] = t;
+    a.tb[k] = ch * a.w_s_red + r * a.w_s2 + s * a.w_s3;
 }
 
 struct GatherF32 {
     const float *a; // fwd: x ; bwd-data: dy
     const float *b; // filter
     float *out;     // fwd: y ; bwd-data: dx
-    const KTab *tab;
+    const KTabA *ta;
+    const long long *tb;
     int M, Ngemm, Kred;
     int OH, OW; // spatial dims of the tensor written
     int IH, IW; // spatial dims of the tensor gathered from
     long long a_sn, a_sh, a_sw;
     long long o_sn, o_sc, o_sh, o_sw;
     long long b_sn; // filter stride of the GEMM column (fwd: k, bwd-data: c)
-    int stride, pad;
+    int stride, pad, dil, R, S;
     float alpha, beta;
 };
 
@@ -67,7 +76,10 @@ constexpr int FBM = 128, FBK = 16, FPAD = 8;
 // 256 threads = 4 wavefronts (2 x 2), each a 64 x (BN/2) part of the 128 x BN tile.  The filter is
 // the MFMA's first operand, so a lane ends up with 16 channels of ONE pixel and consecutive lanes
 // with consecutive pixels: contiguous stores for NCHW outputs.
-template <int BN, bool BWD>
+// LIN (stride 1 backward, any forward, at most 64 taps): the address of a tap is linear in the
+// tap's displacement, so the table holds the finished offset, and whether a tap of this thread's
+// pixel lies inside the image is one bit of a mask computed once.
+template <int BN, bool BWD, bool LIN>
 __global__ void __launch_bounds__(256) conv_f32_gather(GatherF32 g)
 {
     constexpr int TN = BN / 64;        // 32-wide column tiles per wavefront
@@ -95,17 +107,48 @@ __global__ void __launch_bounds__(256) conv_f32_gather(GatherF32 g)
         th0 = BWD ? oh + g.pad : oh * g.stride - g.pad;
         tw0 = BWD ? ow + g.pad : ow * g.stride - g.pad;
     }
+    unsigned long long tapmask = 0;
+    if(LIN) {
+        a_base += th0 * g.a_sh + tw0 * g.a_sw; // may point outside the tensor: only valid taps are read
+        if(m_ok)
+            for(int r = 0; r < g.R; r++) {
+                const int ih = BWD ? th0 - r * g.dil : th0 + r * g.dil;
+                if(ih < 0 || ih >= g.IH)
+                    continue;
+                for(int q = 0; q < g.S; q++) {
+                    const int iw = BWD ? tw0 - q * g.dil : tw0 + q * g.dil;
+                    if(iw >= 0 && iw < g.IW)
+                        tapmask |= 1ull << (r * g.S + q);
+                }
+            }
+    }
     // the filter tile: this thread's reduction row is fixed, its columns step by 16
     const int bk = tid & (FBK - 1), bn0 = tid >> 4;
 
+    // The table entries of a slice are fetched one iteration before the data they address, so that
+    // the data loads never wait for a table load (two dependent trips to memory per slice otherwise).
     float ra[FBK / 2], rb[BPT];
+    KTabA ea[FBK / 2];
+    long long eb = 0;
+    auto load_table = [&](int k0) {
+#pragma unroll
+        for(int j = 0; j < FBK / 2; j++) {
+            const int kg = k0 + ak0 + 2 * j;
+            ea[j] = g.ta[kg < g.Kred ? kg : 0];
+        }
+        const int kg = k0 + bk;
+        eb = g.tb[kg < g.Kred ? kg : 0];
+    };
     auto load_slice = [&](int k0) {
 #pragma unroll
         for(int j = 0; j < FBK / 2; j++) {
             const int kg = k0 + ak0 + 2 * j;
+            const KTabA e = ea[j];
             float v = 0.0f;
-            if(m_ok && kg < g.Kred) {
-                const KTab e = g.tab[kg];
+            if(LIN) {
+                if(kg < g.Kred && ((tapmask >> e.dr) & 1))
+                    v = g.a[a_base + e.off];
+            } else if(m_ok && kg < g.Kred) {
                 int ih, iw;
                 bool ok;
                 if(BWD) {
@@ -119,16 +162,15 @@ __global__ void __launch_bounds__(256) conv_f32_gather(GatherF32 g)
                     ok = ih >= 0 && ih < g.IH && iw >= 0 && iw < g.IW;
                 }
                 if(ok)
-                    v = g.a[a_base + e.a_off + ih * g.a_sh + iw * g.a_sw];
+                    v = g.a[a_base + e.off + ih * g.a_sh + iw * g.a_sw];
             }
             ra[j] = v;
         }
         const int kg = k0 + bk;
-        const long long boff = kg < g.Kred ? g.tab[kg].b_off : 0;
 #pragma unroll
         for(int j = 0; j < BPT; j++) {
             const int n = n0 + bn0 + 16 * j;
-            rb[j] = (kg < g.Kred && n < g.Ngemm) ? g.b[n * g.b_sn + boff] : 0.0f;
+            rb[j] = (kg < g.Kred && n < g.Ngemm) ? g.b[n * g.b_sn + eb] : 0.0f;
         }
     };
     auto store_slice = [&](int buf) {
@@ -150,14 +192,18 @@ __global__ void __launch_bounds__(256) conv_f32_gather(GatherF32 g)
                 acc[i][j][v] = 0.0f;
 
     const int KT = (g.Kred + FBK - 1) / FBK;
+    load_table(0);
     load_slice(0);
+    load_table(FBK);
     store_slice(0);
     __syncthreads();
     const int fr = lane & 31, fk = lane >> 5;
     for(int kt = 0; kt < KT; kt++) {
         const int buf = kt & 1;
-        if(kt + 1 < KT)
+        if(kt + 1 < KT) {
             load_slice((kt + 1) * FBK); // in flight during the MFMAs below
+            load_table((kt + 2) * FBK);
+        }
 #pragma unroll
         for(int kk = 0; kk < FBK / 2; kk++) {
             float fa[2], fb[TN];
@@ -207,7 +253,7 @@ __global__ void __launch_bounds__(256) conv_f32_gather(GatherF32 g)
 struct FilterF32 {
     const float *x, *dy;
     float *partial; // [splits][K][CRS]
-    const KTab *tab; // per column (c,r,s): a_off = c*sC(x), dr, ds
+    const KTabA *tab; // per column (c,r,s), generic form: off = c*sC(x), dr, ds
     int M, K, CRS;
     int P, Q, H, W;
     long long x_sn, x_sh, x_sw;
@@ -236,7 +282,7 @@ __global__ void __launch_bounds__(256) conv_f32_bwd_filter(FilterF32 g)
 
     // loads: lanes run along the pixels (contiguous in NCHW), 8 rows / columns per thread
     const int lm = tid & 31, l0 = tid >> 5;
-    KTab cols[8];
+    KTabA cols[8];
     bool col_ok[8];
 #pragma unroll
     for(int j = 0; j < 8; j++) {
@@ -265,7 +311,7 @@ __global__ void __launch_bounds__(256) conv_f32_bwd_filter(FilterF32 g)
             ra[j] = (ok && k < g.K) ? g.dy[dyb + k * g.dy_sc] : 0.0f;
             const int ih = ih0 + cols[j].dr, iw = iw0 + cols[j].ds;
             rb[j] = (ok && col_ok[j] && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W)
-                        ? g.x[xb + cols[j].a_off + ih * g.x_sh + iw * g.x_sw]
+                        ? g.x[xb + cols[j].off + ih * g.x_sh + iw * g.x_sw]
                         : 0.0f;
         }
     };
@@ -302,7 +348,7 @@ __global__ void __launch_bounds__(256) conv_f32_bwd_filter(FilterF32 g)
 }
 
 __global__ void __launch_bounds__(256)
-    conv_f32_filter_reduce(const float *__restrict__ partial, float *__restrict__ dw, const KTab *__restrict__ tab, int K,
+    conv_f32_filter_reduce(const float *__restrict__ partial, float *__restrict__ dw, const long long *__restrict__ tb, int K,
                            int CRS, int splits, long long w_sk, float alpha, float beta)
 {
     const long long total = (long long)K * CRS;
@@ -311,7 +357,7 @@ __global__ void __launch_bounds__(256)
         float s = 0.0f;
         for(int p = 0; p < splits; p++)
             s += partial[(long long)p * total + i];
-        float *o = dw + k * w_sk + tab[col].b_off;
+        float *o = dw + k * w_sk + tb[col];
         *o = beta != 0.0f ? alpha * s + beta * *o : alpha * s;
     }
 }
@@ -353,7 +399,7 @@ static bool f32_ok(const SagaTensorView *a, const SagaTensorView *b, const SagaT
            (long long)g.C * g.R * g.S < big;
 }
 
-static size_t tab_bytes(int n) { return (((size_t)n * sizeof(KTab)) + 255) & ~(size_t)255; }
+static size_t tab_bytes(int n) { return (((size_t)n * (sizeof(KTabA) + sizeof(long long))) + 255) & ~(size_t)255; }
 
 } // namespace
 
@@ -378,9 +424,12 @@ static int gather_launch(bool bwd, const SagaTensorView *a, const SagaTensorView
     const int Kred = red_ch * g.R * g.S;
     if(!ws || ws_bytes < tab_bytes(Kred) || !aligned16(ws))
         return SAGA_HIP_EWORKSPACE;
-    KTab *tab = (KTab *)ws;
+    KTabA *ta = (KTabA *)ws;
+    long long *tb = (long long *)(ta + Kred);
+    const bool lin = (!bwd || g.stride == 1) && g.R * g.S <= 64;
     TabArgs t;
-    t.tab = tab;
+    t.ta = ta;
+    t.tb = tb;
     t.n = Kred;
     t.RS = g.R * g.S;
     t.S = g.S;
@@ -389,12 +438,16 @@ static int gather_launch(bool bwd, const SagaTensorView *a, const SagaTensorView
     t.w_s_red = bwd ? w->strides[0] : w->strides[1];
     t.w_s2 = w->strides[2];
     t.w_s3 = w->strides[3];
+    t.linear = lin;
+    t.lin_sh = (bwd ? -1 : 1) * g.dil * a->strides[2];
+    t.lin_sw = (bwd ? -1 : 1) * g.dil * a->strides[3];
     f32_build_ktab<<<(Kred + 255) / 256, 256, 0, st>>>(t);
     GatherF32 k;
     k.a = (const float *)a->ptr;
     k.b = (const float *)w->ptr;
     k.out = (float *)out->ptr;
-    k.tab = tab;
+    k.ta = ta;
+    k.tb = tb;
     k.M = out->dims[0] * out->dims[2] * out->dims[3];
     k.Ngemm = out->dims[1];
     k.Kred = Kred;
@@ -412,21 +465,28 @@ static int gather_launch(bool bwd, const SagaTensorView *a, const SagaTensorView
     k.b_sn = bwd ? w->strides[1] : w->strides[0];
     k.stride = g.stride;
     k.pad = g.pad;
+    k.dil = g.dil;
+    k.R = g.R;
+    k.S = g.S;
     k.alpha = alpha;
     k.beta = beta;
     const int bm = (k.M + FBM - 1) / FBM;
-    if(k.Ngemm > 64) {
-        const int blocks = bm * ((k.Ngemm + 127) / 128);
-        if(bwd)
-            conv_f32_gather<128, true><<<blocks, 256, 0, st>>>(k);
-        else
-            conv_f32_gather<128, false><<<blocks, 256, 0, st>>>(k);
-    } else {
-        if(bwd)
-            conv_f32_gather<64, true><<<bm, 256, 0, st>>>(k);
-        else
-            conv_f32_gather<64, false><<<bm, 256, 0, st>>>(k);
-    }
+#define GO(BN, BLOCKS)                                                                  \
+    do {                                                                                \
+        if(bwd && lin)                                                                  \
+            conv_f32_gather<BN, true, true><<<BLOCKS, 256, 0, st>>>(k);                 \
+        else if(bwd)                                                                    \
+            conv_f32_gather<BN, true, false><<<BLOCKS, 256, 0, st>>>(k);                \
+        else if(lin)                                                                    \
+            conv_f32_gather<BN, false, true><<<BLOCKS, 256, 0, st>>>(k);                \
+        else                                                                            \
+            conv_f32_gather<BN, false, false><<<BLOCKS, 256, 0, st>>>(k);               \
+    } while(0)
+    if(k.Ngemm > 64)
+        GO(128, bm * ((k.Ngemm + 127) / 128));
+    else
+        GO(64, bm);
+#undef GO
     SAGA_CHECK_LAUNCH();
     return 0;
 }
@@ -457,9 +517,11 @@ int conv_f32_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, const
     const size_t need = tab_bytes(CRS) + (size_t)p.splits * g.K * CRS * sizeof(float);
     if(!ws || ws_bytes < need || !aligned16(ws))
         return SAGA_HIP_EWORKSPACE;
-    KTab *tab = (KTab *)ws;
+    KTabA *tab = (KTabA *)ws;
+    long long *tb = (long long *)(tab + CRS);
     TabArgs t;
-    t.tab = tab;
+    t.ta = tab;
+    t.tb = tb;
     t.n = CRS;
     t.RS = g.R * g.S;
     t.S = g.S;
@@ -468,6 +530,8 @@ int conv_f32_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, const
     t.w_s_red = dw->strides[1];
     t.w_s2 = dw->strides[2];
     t.w_s3 = dw->strides[3];
+    t.linear = 0;
+    t.lin_sh = t.lin_sw = 0;
     f32_build_ktab<<<(CRS + 255) / 256, 256, 0, st>>>(t);
     FilterF32 k;
     k.x = (const float *)x->ptr;
@@ -496,7 +560,7 @@ int conv_f32_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, const
     conv_f32_bwd_filter<<<p.tiles_k * p.tiles_c * p.splits, 256, 0, st>>>(k);
     SAGA_CHECK_LAUNCH();
     const long long total = (long long)g.K * CRS;
-    conv_f32_filter_reduce<<<grid_for(total, 256, 4096), 256, 0, st>>>(k.partial, (float *)dw->ptr, tab, g.K, CRS, p.splits,
+    conv_f32_filter_reduce<<<grid_for(total, 256, 4096), 256, 0, st>>>(k.partial, (float *)dw->ptr, tb, g.K, CRS, p.splits,
                                                                      dw->strides[0], alpha, beta);
     SAGA_CHECK_LAUNCH();
     return 0;
