@@ -3,7 +3,8 @@
 //  * fp16: gemm_mfma_f16, 64x64x32 block tiles on v_mfma_f32_32x32x16_f16 (one 32x32 tile per
 //    wave), operands staged through LDS with the reduction index contiguous; an operand
 //    stored with the other index contiguous is transposed on its way into LDS.
-//  * fp32: gemm_tiled, LDS-tiled 64x64x16 with a 4x4 register block per lane.
+//  * fp32: gemm_mfma_f32, the same 64x64x16 LDS tiles on v_mfma_f32_32x32x2_f32 (gemm_tiled, a 4x4
+//    register block per lane, is kept as the non-matrix-core reference of the same tiling).
 #include "common.hpp"
 
 namespace {
@@ -71,6 +72,65 @@ __global__ void __launch_bounds__(256)
             const float v = alpha * acc[i][j];
             *o = (T)(beta != 0.0f ? v + beta * (float)*o : v);
         }
+    }
+}
+
+// fp32 on the matrix cores: the tiles of gemm_tiled, multiplied with v_mfma_f32_32x32x2_f32 (one
+// 32x32 tile per wavefront, 8 instructions per 16-deep slice) instead of a 4x4 register block per
+// lane.  A lane feeds A[m = lane%32][k = lane/32] and B[k][n = lane%32] and ends up with column
+// n = lane%32, rows 8*(v/4) + 4*(lane/32) + v%4 of the tile.
+__global__ void __launch_bounds__(256)
+    gemm_mfma_f32(int tA, int tB, int M, int N, int K, float alpha, const float *__restrict__ A, int lda,
+                  const float *__restrict__ B, int ldb, float beta, float *__restrict__ C, int ldc)
+{
+    typedef float float16_t __attribute__((ext_vector_type(16)));
+    constexpr int BM = 64, BN = 64, BK = 16;
+    __shared__ float As[BK][BM + 4];
+    __shared__ float Bs[BK][BN + 4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int wr = (wave >> 1) * 32, wc = (wave & 1) * 32;
+    const int fr = lane & 31, fk = lane >> 5;
+    float16_t acc;
+#pragma unroll
+    for(int v = 0; v < 16; v++)
+        acc[v] = 0.0f;
+    for(int k0 = 0; k0 < K; k0 += BK) {
+        for(int e = tid; e < BM * BK; e += 256) {
+            int mm, kk;
+            if(tA) { mm = e % BM; kk = e / BM; } else { kk = e % BK; mm = e / BK; }
+            const int gm = m0 + mm, gk = k0 + kk;
+            float v = 0;
+            if(gm < M && gk < K)
+                v = tA ? A[(int64_t)gk * lda + gm] : A[(int64_t)gm * lda + gk];
+            As[kk][mm] = v;
+        }
+        for(int e = tid; e < BN * BK; e += 256) {
+            int nn, kk;
+            if(tB) { kk = e % BK; nn = e / BK; } else { nn = e % BN; kk = e / BN; }
+            const int gn = n0 + nn, gk = k0 + kk;
+            float v = 0;
+            if(gn < N && gk < K)
+                v = tB ? B[(int64_t)gn * ldb + gk] : B[(int64_t)gk * ldb + gn];
+            Bs[kk][nn] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for(int kk = 0; kk < BK / 2; kk++)
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(As[2 * kk + fk][wr + fr], Bs[2 * kk + fk][wc + fr], acc, 0, 0, 0);
+        __syncthreads();
+    }
+    const int gn = n0 + wc + fr;
+    if(gn >= N)
+        return;
+#pragma unroll
+    for(int v = 0; v < 16; v++) {
+        const int gm = m0 + wr + 8 * (v >> 2) + 4 * fk + (v & 3);
+        if(gm >= M)
+            continue;
+        float *o = C + (int64_t)gm * ldc + gn;
+        const float r = alpha * acc[v];
+        *o = beta != 0.0f ? r + beta * *o : r;
     }
 }
 
@@ -175,8 +235,8 @@ extern "C" int saga_hip_gemm(int transA, int transB, int M, int N, int K, float 
         gemm_mfma_f16<<<grid, 256, 0, st>>>(transA, transB, M, N, K, alpha, (const half_t *)A, lda, (const half_t *)B,
                                             ldb, beta, (half_t *)C, ldc, a_vec, b_vec);
     } else if(dtype == SAGA_FLOAT)
-        gemm_tiled<float><<<grid, 256, 0, st>>>(transA, transB, M, N, K, alpha, (const float *)A, lda,
-                                                (const float *)B, ldb, beta, (float *)C, ldc);
+        gemm_mfma_f32<<<grid, 256, 0, st>>>(transA, transB, M, N, K, alpha, (const float *)A, lda, (const float *)B, ldb,
+                                            beta, (float *)C, ldc);
     else
         return SAGA_HIP_EUNSUPPORTED;
     SAGA_CHECK_LAUNCH();
