@@ -133,7 +133,9 @@ int saga_hip_conv2d_fwd_bn_infer(const SagaTensorView *x, const SagaTensorView *
 /* y[n,c,:,:] += b[c] : cudnnAddTensor of a {1,C,1,1} bias (src/cuda/cuda_dnn.cpp:39-68). b is fp32 or y's type. */
 int saga_hip_bias_add(const SagaTensorView *y, const SagaTensorView *b, saga_stream_t stream);
 /* db[c] = beta*db + sum_{n,h,w} dy : cudnnConvolutionBackwardBias (src/cuda/cuda_dnn.cpp:378-385). */
-int saga_hip_bias_bwd(const SagaTensorView *dy, const SagaTensorView *db, float beta, saga_stream_t stream);
+size_t saga_hip_bias_bwd_workspace_size(const SagaTensorView *dy);
+int saga_hip_bias_bwd(const SagaTensorView *dy, const SagaTensorView *db, float beta, void *workspace, size_t ws_bytes,
+                      saga_stream_t stream);
 
 /* ---- GEMM: cublasSgemm / cublasHgemm as used by the fc node (src/cuda/cuda_dnn.cpp:1001-1025).
  *      Row-major: C[M,N] = alpha * op(A) * op(B) + beta * C, op(A) is MxK, op(B) is KxN;

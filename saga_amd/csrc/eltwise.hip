@@ -297,6 +297,130 @@ __global__ void __launch_bounds__(256) bias_bwd_cl(const T *dy, int64_t pitch, T
     }
 }
 
+// Large channels-last tensors: the rows are split over gridDim.x blocks, each leaving one fp32
+// partial per channel; bias_bwd_final adds them in block order (deterministic, no atomics).
+// Block = 64 channels x 4 row lanes, as above.
+template <typename T>
+__global__ void __launch_bounds__(256)
+    bias_bwd_partial_cl(const T *__restrict__ dy, int64_t pitch, float *__restrict__ partial, int64_t rows, int C)
+{
+    __shared__ float part[4][64];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int c = blockIdx.y * 64 + lane;
+    float acc = 0;
+    if(c < C) {
+        const int64_t stride = (int64_t)gridDim.x * 4;
+        int64_t r = (int64_t)blockIdx.x * 4 + wv;
+        for(; r + 7 * stride < rows; r += 8 * stride) {
+            float v[8];
+#pragma unroll
+            for(int u = 0; u < 8; u++)
+                v[u] = (float)dy[(r + u * stride) * pitch + c];
+#pragma unroll
+            for(int u = 0; u < 8; u++)
+                acc += v[u];
+        }
+        for(; r < rows; r += stride)
+            acc += (float)dy[r * pitch + c];
+    }
+    part[wv][lane] = acc;
+    __syncthreads();
+    if(wv == 0 && c < C)
+        partial[(int64_t)blockIdx.x * C + c] = part[0][lane] + part[1][lane] + part[2][lane] + part[3][lane];
+}
+
+// The same with 16-byte loads along C (C, the pitch and the base address multiples of the vector):
+// cvp (a power of two, at most 256) threads cover the channel vectors of one row, 256 / cvp rows at a time.
+template <typename T>
+__global__ void __launch_bounds__(256) bias_bwd_partial_vec(const T *__restrict__ dy, int64_t pitch,
+                                                            float *__restrict__ partial, int64_t rows, int C, int cvp)
+{
+    typedef typename Vec<T>::type V;
+    constexpr int VN = Vec<T>::n;
+    __shared__ float part[256][VN + 1];
+    const int cv = C / VN;
+    const int ci = blockIdx.y * cvp + (threadIdx.x & (cvp - 1));
+    const int rl = threadIdx.x / cvp, nrl = 256 / cvp;
+    float acc[VN];
+#pragma unroll
+    for(int j = 0; j < VN; j++)
+        acc[j] = 0.0f;
+    if(ci < cv) {
+        const int64_t stride = (int64_t)gridDim.x * nrl;
+        int64_t r = (int64_t)blockIdx.x * nrl + rl;
+        const T *base = dy + (int64_t)ci * VN;
+        for(; r + 3 * stride < rows; r += 4 * stride) {
+            V v[4];
+#pragma unroll
+            for(int u = 0; u < 4; u++)
+                v[u] = *(const V *)(base + (r + u * stride) * pitch);
+#pragma unroll
+            for(int u = 0; u < 4; u++)
+#pragma unroll
+                for(int j = 0; j < VN; j++)
+                    acc[j] += (float)v[u][j];
+        }
+        for(; r < rows; r += stride) {
+            const V v = *(const V *)(base + r * pitch);
+#pragma unroll
+            for(int j = 0; j < VN; j++)
+                acc[j] += (float)v[j];
+        }
+    }
+#pragma unroll
+    for(int j = 0; j < VN; j++)
+        part[threadIdx.x][j] = acc[j];
+    __syncthreads();
+    if(rl == 0 && ci < cv) {
+        for(int k = 1; k < nrl; k++)
+#pragma unroll
+            for(int j = 0; j < VN; j++)
+                acc[j] += part[threadIdx.x + k * cvp][j];
+#pragma unroll
+        for(int j = 0; j < VN; j++)
+            partial[(int64_t)blockIdx.x * C + ci * VN + j] = acc[j];
+    }
+}
+
+// One block per 32 channels: 8 lanes per channel each add every 8th partial (four loads in flight),
+// then lane 0 adds the 8 lane sums in order.
+template <typename TB>
+__global__ void __launch_bounds__(256) bias_bwd_final(const float *__restrict__ partial, int gx, TB *db, int C, float beta)
+{
+    __shared__ float part[8][32];
+    const int cl = threadIdx.x & 31, gl = threadIdx.x >> 5;
+    const int c = blockIdx.x * 32 + cl;
+    float s = 0;
+    if(c < C) {
+        int g = gl;
+        for(; g + 24 < gx; g += 32) {
+            const float v0 = partial[(int64_t)g * C + c], v1 = partial[(int64_t)(g + 8) * C + c];
+            const float v2 = partial[(int64_t)(g + 16) * C + c], v3 = partial[(int64_t)(g + 24) * C + c];
+            s += (v0 + v1) + (v2 + v3);
+        }
+        for(; g < gx; g += 8)
+            s += partial[(int64_t)g * C + c];
+    }
+    part[gl][cl] = s;
+    __syncthreads();
+    if(gl == 0 && c < C) {
+        for(int k = 1; k < 8; k++)
+            s += part[k][cl];
+        db[c] = (TB)(beta != 0.0f ? s + beta * (float)db[c] : s);
+    }
+}
+
+// blocks along the rows for the two-pass form; 1 = the single-pass kernel is enough
+static int bias_bwd_splits(int64_t rows, int C)
+{
+    if(rows * C < (int64_t)1 << 20)
+        return 1;
+    int64_t gx = C >= 512 ? 512 : 1024; // at least four blocks of the vector kernel per CU
+    if(gx > rows / 64)
+        gx = rows / 64;
+    return gx < 2 ? 1 : (int)gx;
+}
+
 template <typename T, typename TB>
 __global__ void __launch_bounds__(256) bias_bwd_cf(const T *dy, int64_t npitch, TB *db, int N, int C, int64_t HW, float beta)
 {
@@ -419,7 +543,17 @@ int saga_hip_bias_add(const SagaTensorView *y, const SagaTensorView *b, saga_str
     return 0;
 }
 
-int saga_hip_bias_bwd(const SagaTensorView *dy, const SagaTensorView *db, float beta, saga_stream_t stream)
+size_t saga_hip_bias_bwd_workspace_size(const SagaTensorView *dy)
+{
+    CLInfo cl;
+    if(!valid_view(dy) || !as_channels_last(dy, &cl))
+        return 0;
+    const int gx = bias_bwd_splits(cl.rows, cl.C);
+    return gx > 1 ? (size_t)gx * cl.C * sizeof(float) : 0;
+}
+
+int saga_hip_bias_bwd(const SagaTensorView *dy, const SagaTensorView *db, float beta, void *workspace, size_t ws_bytes,
+                      saga_stream_t stream)
 {
     if(!valid_view(dy) || !valid_view(db))
         return SAGA_HIP_EINVAL;
@@ -428,8 +562,25 @@ int saga_hip_bias_bwd(const SagaTensorView *dy, const SagaTensorView *db, float 
     hipStream_t st = as_stream(stream);
     CLInfo cl;
     CFInfo cf;
+    const size_t need = saga_hip_bias_bwd_workspace_size(dy);
+    if(need && (!workspace || ws_bytes < need))
+        return SAGA_HIP_EWORKSPACE;
 #define BIAS_BWD(T, TB)                                                                                     \
-    if(as_channels_last(dy, &cl))                                                                           \
+    if(as_channels_last(dy, &cl) && need) {                                                                 \
+        const int gx = bias_bwd_splits(cl.rows, cl.C);                                                      \
+        constexpr int VN = Vec<T>::n;                                                                       \
+        if(cl.C % VN == 0 && cl.pitch % VN == 0 && (uintptr_t)dy->ptr % 16 == 0) {                          \
+            int cvp = 1;                                                                                    \
+            while(cvp < cl.C / VN && cvp < 256)                                                             \
+                cvp *= 2;                                                                                   \
+            bias_bwd_partial_vec<T><<<dim3(gx, (cl.C / VN + cvp - 1) / cvp), 256, 0, st>>>(                  \
+                (const T *)dy->ptr, cl.pitch, (float *)workspace, cl.rows, cl.C, cvp);                      \
+        } else                                                                                              \
+            bias_bwd_partial_cl<T><<<dim3(gx, (cl.C + 63) / 64), 256, 0, st>>>(                             \
+                (const T *)dy->ptr, cl.pitch, (float *)workspace, cl.rows, cl.C);                           \
+        bias_bwd_final<TB><<<(cl.C + 31) / 32, 256, 0, st>>>((const float *)workspace, gx, (TB *)db->ptr,  \
+                                                               cl.C, beta);                                 \
+    } else if(as_channels_last(dy, &cl))                                                                    \
         bias_bwd_cl<T, TB><<<(cl.C + 63) / 64, 256, 0, st>>>((const T *)dy->ptr, cl.pitch, (TB *)db->ptr,     \
                                                              cl.rows, cl.C, beta);                          \
     else if(as_channels_first(dy, &cf))                                                                     \

@@ -130,6 +130,50 @@ __global__ void __launch_bounds__(256)
     }
 }
 
+// Average pooling over windows of 1024 positions or more (global pooling of a large image): one
+// block per output vector, the window positions striped over its 256 threads, then a tree sum in LDS.
+template <typename T, int VN>
+__global__ void __launch_bounds__(256) avgpool_fwd_wide_k(DView x, DView y, int k, int pad, int stride)
+{
+    __shared__ float part[256][VN];
+    const int C = y.d[1], P = y.d[2], Q = y.d[3], H = x.d[2], W = x.d[3];
+    int n, c, p, q;
+    decode<VN>(blockIdx.x, C, P, Q, n, c, p, q);
+    float acc[VN];
+#pragma unroll
+    for(int j = 0; j < VN; j++)
+        acc[j] = 0.0f;
+    for(int t = threadIdx.x; t < k * k; t += 256) {
+        const int h = p * stride - pad + t / k, w = q * stride - pad + t % k;
+        if(h < 0 || h >= H || w < 0 || w >= W)
+            continue;
+        float v[VN];
+        PV<T, VN>::load((const T *)x.ptr + off4(x, n, c, h, w), v);
+#pragma unroll
+        for(int j = 0; j < VN; j++)
+            acc[j] += v[j];
+    }
+#pragma unroll
+    for(int j = 0; j < VN; j++)
+        part[threadIdx.x][j] = acc[j];
+    __syncthreads();
+    for(int w = 128; w > 0; w >>= 1) {
+        if((int)threadIdx.x < w) {
+#pragma unroll
+            for(int j = 0; j < VN; j++)
+                part[threadIdx.x][j] += part[threadIdx.x + w][j];
+        }
+        __syncthreads();
+    }
+    if(threadIdx.x == 0) {
+        const float inv = 1.0f / (float)(k * k);
+#pragma unroll
+        for(int j = 0; j < VN; j++)
+            acc[j] = part[0][j] * inv;
+        PV<T, VN>::store((T *)y.ptr + off4(y, n, c, p, q), acc);
+    }
+}
+
 static __device__ __forceinline__ int cdiv_floor(int a, int b) { return a >= 0 ? a / b : -((-a + b - 1) / b); }
 
 template <typename T, int VN, int MODE>
@@ -487,6 +531,8 @@ int saga_hip_pool_fwd(int mode, const SagaTensorView *x, const SagaTensorView *y
         if(mode == SAGA_POOL_MAX)                                                                        \
             pool_fwd_k<T, VN, SAGA_POOL_MAX><<<g, 256, 0, st>>>(dvx, dvy, dvi, idx != nullptr, size, pad, \
                                                                 stride, total);                          \
+        else if(size >= 32 && total < ((int64_t)1 << 30))                                                \
+            avgpool_fwd_wide_k<T, VN><<<(int)total, 256, 0, st>>>(dvx, dvy, size, pad, stride);           \
         else                                                                                             \
             pool_fwd_k<T, VN, SAGA_POOL_AVG><<<g, 256, 0, st>>>(dvx, dvy, dvi, 0, size, pad, stride, total); \
     } while(0)

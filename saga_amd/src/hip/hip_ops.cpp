@@ -206,11 +206,15 @@ struct BiasAdd : public HipOperation {
 struct BiasBwd : public HipOperation {
     const T dy_, db_;
     float beta_ = 0;
-    BiasBwd(T dy, T db) : HipOperation("biasbwd"), dy_(dy), db_(db) {}
+    BiasBwd(HipProgram &p, T dy, T db) : HipOperation("biasbwd"), dy_(dy), db_(db)
+    {
+        const SagaTensorView vdy = dy->shapeView();
+        p.m_ctx->m_workspace.request(saga_hip_bias_bwd_workspace_size(&vdy));
+    }
     void exec(HipProgram &p) override
     {
         const SagaTensorView vdy = dy_->view(), vdb = db_->view();
-        chkSaga(saga_hip_bias_bwd(&vdy, &vdb, beta_, S(p)));
+        chkSaga(saga_hip_bias_bwd(&vdy, &vdb, beta_, p.m_ctx->m_workspace.ptr(), p.m_ctx->m_workspace.size(), S(p)));
     }
     HipOpArgs listInputs() const override { return {{"dy", dy_}}; }
     HipOpArgs listOutputs() const override { return {{"db", db_}}; }
@@ -241,7 +245,7 @@ void conv_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
         auto dy = p.lowerGrad(pu, n.m_outputs["y"]);
         if(b) {
             auto db = p.lowerGrad(pu, n.m_inputs["b"], y->m_dims.size());
-            pu.bwd(std::make_shared<BiasBwd>(dy, db));
+            pu.bwd(std::make_shared<BiasBwd>(p, dy, db));
             p.upd(n.m_inputs["b"], b, db);
         }
         auto dw = p.lowerGrad(pu, n.m_inputs["w"]);
@@ -259,7 +263,7 @@ void conv_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
         auto dy = p.lowerGrad(pu, n.m_outputs["y"]);
         if(b) {
             auto db = p.lowerGrad(pu, n.m_inputs["b"], y->m_dims.size());
-            pu.bwd(std::make_shared<BiasBwd>(dy, db));
+            pu.bwd(std::make_shared<BiasBwd>(p, dy, db));
             p.upd(n.m_inputs["b"], b, db);
         }
         auto dw = p.lowerGrad(pu, n.m_inputs["w"]);
@@ -531,7 +535,7 @@ void fc_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
     p.upd(n.m_inputs["w"], w, dw);
     if(b) {
         auto db = p.lowerGrad(pu, n.m_inputs["b"], 2);
-        pu.bwd(std::make_shared<BiasBwd>(dy, db)); // column sums of dy
+        pu.bwd(std::make_shared<BiasBwd>(p, dy, db)); // column sums of dy
         p.upd(n.m_inputs["b"], b, db);
     }
     if(dx) // dx[batch,in] = dy * W^T

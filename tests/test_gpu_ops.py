@@ -236,8 +236,30 @@ def test_bias(layout, padc, dtype):
     assert_close(host(yd), ref.bias_add(y, b), dtype, "bias add")
     db = dev(np.ones(16, np.float32), torch.float32)
     dyd = dev(y, dtype, layout, padc)
-    K.check(K.lib().saga_hip_bias_bwd(C.byref(K.view(dyd)), C.byref(K.view(db.view(1, 16, 1, 1))), 1.0, S()))
+    K.check(K.lib().saga_hip_bias_bwd(C.byref(K.view(dyd)), C.byref(K.view(db.view(1, 16, 1, 1))), 1.0, None, 0, S()))
     assert_close(host(db), ref.bias_bwd(y) + 1, dtype, "bias bwd")
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("padc", [0, 8, 3])
+@pytest.mark.parametrize("shape", [(4, 64, 96, 96), (2, 20, 200, 150), (64, 1000, 5, 5), (1, 4104, 16, 16)])
+def test_bias_bwd_large(shape, padc, dtype):
+    """Tensors large enough for the two-pass reduction over row blocks (needs the workspace)."""
+    rng = np.random.default_rng(6)
+    y = rnd(rng, *shape, dtype=dtype)
+    c = shape[1]
+    dyd = dev(y, dtype, "nhwc", padc)
+    vdy = K.view(dyd)
+    need = K.lib().saga_hip_bias_bwd_workspace_size(C.byref(vdy))
+    assert need > 0
+    db = dev(np.ones(c, np.float32), torch.float32)
+    vdb = K.view(db.view(1, c, 1, 1))
+    assert K.lib().saga_hip_bias_bwd(C.byref(vdy), C.byref(vdb), 1.0, None, 0, S()) == -4
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    K.check(K.lib().saga_hip_bias_bwd(C.byref(vdy), C.byref(vdb), 1.0, K.ptr(ws), need, S()))
+    got, want = host(db), ref.bias_bwd(y) + 1
+    scale = np.abs(y.astype(np.float64)).sum(axis=(0, 2, 3)).max()
+    assert np.abs(got - want).max() <= 2e-6 * scale, "bias bwd large"
 
 
 @pytest.mark.parametrize("dtype", DT)
@@ -403,7 +425,8 @@ def test_relu_golden_and_nan(golden):
 
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("layout,padc", LAYOUTS)
-@pytest.mark.parametrize("k,pad,stride,H", [(2, 0, 2, 8), (3, 1, 2, 9), (3, 1, 1, 6), (7, 0, 1, 7)])
+@pytest.mark.parametrize("k,pad,stride,H", [(2, 0, 2, 8), (3, 1, 2, 9), (3, 1, 1, 6), (7, 0, 1, 7), (40, 0, 1, 40),
+                                            (32, 2, 4, 44)])
 def test_pooling(k, pad, stride, H, layout, padc, dtype):
     rng = np.random.default_rng(k * 10 + H)
     shape = (2, 16, H, H)
