@@ -45,6 +45,8 @@ CONV_CASES = [
     (2, 4, 12, 12, 16, 5, 2, 2, 1),
     (2, 1, 10, 11, 8, 3, 1, 2, 1),
     (1, 3, 21, 21, 72, 8, 3, 4, 1),
+    (2, 32, 12, 11, 72, 5, 2, 2, 1),
+    (5, 96, 10, 10, 40, 3, 1, 1, 1),
 ]
 
 
