@@ -178,6 +178,9 @@ struct HipOperation {
     // must cross HBM (memory-bound ops); used for roofline accounting only
     virtual double flops() const { return 0; }
     virtual double bytes() const { return 0; }
+    // false for an operation whose launches take host values that change from step to step
+    // (loss scale, Adam's bias corrections): it is never recorded into a HIP graph
+    virtual bool graphSafe() const { return true; }
 
     // inputs plus the outputs that are accumulated into
     HipOpArgs getInputs();
@@ -224,6 +227,8 @@ public:
     int m_program_index_gen = 0;
 
     HipScratch m_workspace;
+    // bumped whenever a storage gets a new device address; recorded HIP graphs of older epochs are dropped
+    uint64_t m_mem_epoch = 0;
 
     // front-end tensor -> device tensor, shared by all programs of this context so that
     // inference and training programs see the same weights
@@ -314,6 +319,22 @@ public:
     std::vector<hipEvent_t> m_events;          // one per op boundary (ops + 1)
     std::map<std::string, ProfileRow> m_profile;
     void collectProfile();
+
+    // ---- HIP graphs: runs of graph-safe operations of the step are recorded once per combination of
+    // front buffers (batched tensors alternate between two device buffers) and replayed with one launch each
+    struct GraphSegment {
+        size_t begin = 0, end = 0; // [begin, end) of m_ops
+        bool graph = false;        // false: run operation by operation
+        std::map<unsigned, hipGraphExec_t> exec; // by front-buffer key
+    };
+    std::vector<GraphSegment> m_segments;
+    std::vector<HipDoubleBuffer *> m_graph_dbufs; // every double-buffered storage the operations touch
+    uint64_t m_graph_epoch = ~(uint64_t)0;
+    void *m_graph_ws = nullptr;
+    long m_steps_run = 0; // executions of m_ops so far
+    bool graphsEnabled() const;
+    void dropGraphs();
+    void runOpsGraphed();
 
     SagaAux *m_aux = nullptr; // pinned host memory the optimizer kernels write their flags to
     float m_mp_scaling = 1.0f;

@@ -636,6 +636,8 @@ struct CatClassifierBwd : public HipOperation {
                                            (const int32_t *)dy_->deviceMem(),
                                            loss_ ? (float *)loss_->deviceMem() : nullptr, scale, S(p)));
     }
+    // the loss scale is a launch argument and changes every step
+    bool graphSafe() const override { return x_->m_data_type != Tensor::DataType::HALF; }
     HipOpArgs listInputs() const override { return {{"x", x_}, {"y", y_}, {"dy", dy_}}; }
     HipOpArgs listOutputs() const override
     {

@@ -27,6 +27,8 @@ struct Optimizer : public HipOperation {
     HipOpArgs listInputs() const override { return m_inputs; }
     HipOpArgs listOutputs() const override { return m_outputs; }
     std::string info() const override { return fmt("%zd elements", m_elements); }
+    // bias corrections and the loss scale are launch arguments that change every step
+    bool graphSafe() const override { return false; }
     // w, g, m, v read and w, m, v written in fp32: 28 bytes per element; the mixed flavour moves
     // fp16 w/g and an extra fp32 master copy: also 28
     double bytes() const override { return 28.0 * m_elements; }

@@ -47,6 +47,8 @@ void HipStorage::rehome(const std::shared_ptr<HipMemory> &mem, void *ptr)
     m_memory = mem;
     m_data = ptr;
     m_in_arena = false;
+    if(m_ctx)
+        m_ctx->m_mem_epoch++;
 }
 
 void HipStorage::allocOwn()

@@ -80,24 +80,30 @@ def accuracies(stdout):
     return [float(m) for m in re.findall(r"Accuracy:\s*(\d+\.\d+)%", stdout)]
 
 
-@pytest.mark.parametrize("args,floor", [
-    (["-m", "lecun", "-b", "64"], 99.0),
-    (["-m", "lecun", "-b", "64", "-h", "-c"], 99.0),
-    (["-m", "resnet-50", "-h", "-c", "-b", "256", "-r", "1e-3"], 95.0),
-], ids=["lecun-fp32", "lecun-fp16-nhwc", "resnet50-fp16-nhwc-b256"])
-def test_reference_classifier_harness(tmp_path, args, floor):
+@pytest.mark.parametrize("args,floor,graphs", [
+    (["-m", "lecun", "-b", "64"], 99.0, False),
+    (["-m", "lecun", "-b", "64", "-h", "-c"], 99.0, False),
+    (["-m", "resnet-50", "-h", "-c", "-b", "256", "-r", "1e-3"], 95.0, False),
+    (["-m", "lecun", "-b", "64", "-h", "-c"], 99.0, True),
+], ids=["lecun-fp32", "lecun-fp16-nhwc", "resnet50-fp16-nhwc-b256", "lecun-fp16-nhwc-hip-graphs"])
+def test_reference_classifier_harness(tmp_path, args, floor, graphs):
     """The reference's training harness (test/test_classifier.cpp:527-857 behind `saga mnist`):
     uint8 batches loaded by its pre_ops callback into double-buffered tensors, labels written
     per batch, loss and predictions read back by post_ops, training and inference programs of
     one context alternating per epoch, until the test accuracy reaches 99 % or 20 epochs passed.
-    The last case is the command the headline numbers of the reference are quoted for."""
+    The resnet-50 case is the command the headline numbers of the reference are quoted for; the last case
+    replays the steps from HIP graphs (SAGA_HIP_GRAPH=1), with the double-buffered batch tensors
+    alternating underneath the recordings."""
     write_idx_dataset(str(tmp_path))
     if not os.path.exists(BIN):
         pytest.skip("oracle/_ref/saga_refhost not built (make -C oracle -f Makefile.ref)")
     saved = tmp_path / "weights"
     saved.mkdir()
+    env = dict(os.environ, SAGA_HIP_GRAPH="1", SAGA_HIP_GRAPH_VERBOSE="1") if graphs else None
     r = subprocess.run([BIN, "mnist", str(tmp_path), *args, "-s", str(saved)], capture_output=True, text=True,
-                       timeout=300)
+                       timeout=300, env=env)
+    if graphs:
+        assert "into a graph" in r.stderr
     acc = accuracies(r.stdout)
     print(r.stdout[-1500:].replace("\033", "<esc>"))
     print(r.stderr[-2000:])
