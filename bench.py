@@ -38,9 +38,9 @@ CONV_KINDS = ("convfwd", "convbwddata", "convbwdfilter")
 MEASURED_HBM_BYTES_PER_LAUNCH = {
     # the counters cannot tell fused from plain batch-norm launches (same kernels): both kinds carry
     # the average over all 53 batch-norm launches of a step
-    "bnbwd.fused": 635763596, "bnbwd": 635763596,
-    "bntrain.fused": 285295384, "bntrain": 285295384,
-    "convfwd": 263599419, "convbwddata": 287505075, "convbwdfilter": 308654371,
+    "bnbwd.fused": 635805665, "bnbwd": 635805665,
+    "bntrain.fused": 285298731, "bntrain": 285298731,
+    "convfwd": 263642790, "convbwddata": 287438380, "convbwdfilter": 308631930,
 }
 
 
