@@ -1377,19 +1377,36 @@ __global__ void __launch_bounds__(256)
 }
 
 // dw[k][r][s][c] = alpha * sum_p partial[p][k][r][s*4 + c] + beta * dw
+// 16 outputs per block, 16 threads per output that each add every 16th split (four loads in flight),
+// then a fixed-order sum of the 16: hundreds of splits would otherwise be one long dependent chain.
 __global__ void __launch_bounds__(256)
     thin_filter_reduce(const float *__restrict__ partial, half_t *__restrict__ dw, int64_t n, int C, int S, int splits,
                        float alpha, float beta)
 {
+    __shared__ float part[16][17];
     const int64_t np = n / (S * C) * 32;
-    for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    const int o = threadIdx.x & 15, q = threadIdx.x >> 4;
+    const int64_t i = (int64_t)blockIdx.x * 16 + o;
+    float acc = 0;
+    if(i < n) {
         const int c = (int)(i % C);
         const int64_t t = i / C;
         const int s = (int)(t % S);
-        const int64_t j = (t / S) * 32 + s * 4 + c;
-        float acc = 0;
-        for(int p = 0; p < splits; p++)
-            acc += partial[(int64_t)p * np + j];
+        const float *src = partial + (t / S) * 32 + s * 4 + c;
+        int p = q;
+        for(; p + 48 < splits; p += 64) {
+            const float v0 = src[(int64_t)p * np], v1 = src[(int64_t)(p + 16) * np];
+            const float v2 = src[(int64_t)(p + 32) * np], v3 = src[(int64_t)(p + 48) * np];
+            acc += (v0 + v1) + (v2 + v3);
+        }
+        for(; p < splits; p += 16)
+            acc += src[(int64_t)p * np];
+    }
+    part[q][o] = acc;
+    __syncthreads();
+    if(q == 0 && i < n) {
+        for(int k = 1; k < 16; k++)
+            acc += part[k][o];
         acc *= alpha;
         if(beta != 0.0f)
             acc += beta * (float)dw[i];
@@ -1811,7 +1828,7 @@ int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, cons
         else
             conv_bwd_filter_dma<64, 128, ST, 4><<<blocks, 256, ST * BK * 384, st>>>(a, (unsigned)(px * 8), (unsigned)yb);
         SAGA_CHECK_LAUNCH();
-        thin_filter_reduce<<<grid_for(n, 256, 256 * 8), 256, 0, st>>>(a.partial, (half_t *)dw->ptr, n, g.C, g.S, p.splits,
+        thin_filter_reduce<<<(int)((n + 15) / 16), 256, 0, st>>>(a.partial, (half_t *)dw->ptr, n, g.C, g.S, p.splits,
                                                                     alpha, beta);
         SAGA_CHECK_LAUNCH();
         return 0;
