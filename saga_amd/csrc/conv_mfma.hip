@@ -419,17 +419,8 @@ __global__ void __launch_bounds__(64 * (WGM * WGN + PROD), PROD ? (WGM * WGN + P
     const int ktot = g.R * g.S * g.Cred;
     const int csteps = (g.Cred + BKT - 1) / BKT;
     const int KT = nr * ns * csteps;
+    const bool ragged = g.Cred % BKT != 0;
     int ri = 0, si = 0, c0 = 0; // tap counters and channel offset of the NEXT slice to be issued
-    auto advance = [&]() {
-        c0 += BKT;
-        if(c0 >= g.Cred) {
-            c0 = 0;
-            if(++si == ns) {
-                si = 0;
-                ++ri;
-            }
-        }
-    };
 
     // With PROD > 0 the block has PROD extra wavefronts that do nothing but issue the loads:
     // a load-to-LDS instruction holds its wavefront at issue until the memory pipeline takes
@@ -455,38 +446,75 @@ __global__ void __launch_bounds__(64 * (WGM * WGN + PROD), PROD ? (WGM * WGN + P
                 bok[i] = n < g.Ngemm;
                 bo[i] = ((bok[i] ? n : 0) * ktot + pkv) * 2;
             }
+            // Per tap: the byte offset of every piece this lane loads, or OOB where the tap falls outside
+            // the image or the row / column lies beyond the tensor; the slice's channel offset rides in
+            // the load's scalar offset.  Only a channel count that is no multiple of the slice depth makes
+            // the offsets depend on the slice (its last slice per tap is ragged): then they are rebuilt
+            // for every slice.
+            unsigned av[PA], bv[PB];
+            auto tap_setup = [&]() {
+                const bool cok = !ragged || c0 + pkv < g.Cred;
+                const int tapoff = ((ri * g.IW + si) * sy * g.lda) * 2; // same for all lanes
+                const int tap = ri * ns + si;
+#pragma unroll
+                for(int i = 0; i < PA; i++)
+                    av[i] = (cok && ((mk[i] >> tap) & 1)) ? (unsigned)(ro[i] + tapoff) : OOB;
+                const int r = r0 + ri * rstep, s = s0 + si * rstep;
+                const int kb = (r * g.S + s) * g.Cred * 2;
+#pragma unroll
+                for(int i = 0; i < PB; i++)
+                    bv[i] = (bok[i] && cok) ? (unsigned)(bo[i] + kb) : OOB;
+            };
+            auto step_cursor = [&]() {
+                bool newtap = false;
+                c0 += BKT;
+                if(c0 >= g.Cred) {
+                    c0 = 0;
+                    newtap = true;
+                    if(++si == ns) {
+                        si = 0;
+                        ++ri;
+                    }
+                }
+                if((newtap || ragged) && ri < nr)
+                    tap_setup();
+            };
             auto produce = [&](int stage) {
                 char *sa = smem + stage * STAGE_BYTES + pw * PA * 16 * ROWB;
                 char *sb = smem + stage * STAGE_BYTES + BM * ROWB + pw * PB * 16 * ROWB;
-                const bool cok = c0 + pkv < g.Cred;
-                const int tapoff = ((ri * g.IW + si) * sy * g.lda + c0) * 2; // same for all lanes
-                const int tap = ri * ns + si;
+                const int koff = c0 * 2;
 #pragma unroll
                 for(int i = 0; i < PA; i++) {
-                    const bool ok = cok && ((mk[i] >> tap) & 1);
-                    const unsigned off = ok ? (unsigned)(ro[i] + tapoff) : OOB;
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(sa + i * 16 * ROWB), 16, off, 0, 0, 0);
+                    const unsigned off = av[i]; // (a captured array element passed directly makes the host pass drop the kernel)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(sa + i * 16 * ROWB), 16, off, koff, 0, 0);
                 }
-                const int r = r0 + ri * rstep, s = s0 + si * rstep;
-                const int kb = ((r * g.S + s) * g.Cred + c0) * 2;
 #pragma unroll
                 for(int i = 0; i < PB; i++) {
-                    const unsigned off = (bok[i] && cok) ? (unsigned)(bo[i] + kb) : OOB;
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(sb + i * 16 * ROWB), 16, off, 0, 0, 0);
+                    const unsigned off = bv[i];
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(sb + i * 16 * ROWB), 16, off, koff, 0, 0);
                 }
-                advance();
+                step_cursor();
             };
+            if(KT > 0)
+                tap_setup();
 #pragma unroll
             for(int st = 0; st < STAGES - 1; st++)
                 if(st < KT)
                     produce(st);
-            for(int kt = 0; kt < KT; kt++) {
-                if(kt + STAGES - 2 < KT)
-                    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((PA + PB) * (STAGES - 2)) : "memory");
-                else
-                    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-                if(kt + STAGES - 1 < KT)
-                    produce((kt + STAGES - 1) % STAGES);
+            // unrolled by the stage count: every stage address is a constant
+            for(int kt0 = 0; kt0 < KT; kt0 += STAGES) {
+#pragma unroll
+                for(int u = 0; u < STAGES; u++) {
+                    const int kt = kt0 + u;
+                    if(kt >= KT)
+                        break;
+                    if(kt + STAGES - 2 < KT)
+                        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((PA + PB) * (STAGES - 2)) : "memory");
+                    else
+                        asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+                    if(kt + STAGES - 1 < KT)
+                        produce((u + STAGES - 1) % STAGES);
+                }
             }
             if constexpr(!BWD) {
                 if(g.bn_s) { // the two barriers around the folded batch norm's parameter table
@@ -523,30 +551,54 @@ __global__ void __launch_bounds__(64 * (WGM * WGN + PROD), PROD ? (WGM * WGN + P
     }
 
     // one slice = AV + BV load instructions ("pieces"); issue_piece(stage, p) emits piece p of
-    // the next slice, advance() steps the slice cursor once all its pieces are out
+    // the next slice, step_cursor() moves on once all its pieces are out.  As in the producer
+    // branch the per-lane offsets are fixed per tap and the slice's channel offset is scalar.
+    unsigned av[AV], bv[BV];
+    auto tap_setup = [&]() {
+        const bool cok = !ragged || c0 + kv < g.Cred;
+        const int tapoff = ((ri * g.IW + si) * sy * g.lda) * 2; // same for all lanes
+        const int tap = ri * ns + si;
+#pragma unroll
+        for(int j = 0; j < AV; j++)
+            av[j] = (cok && ((amask[j] >> tap) & 1)) ? (unsigned)(rowoff[j] + tapoff) : OOB;
+        const int r = r0 + ri * rstep, s = s0 + si * rstep;
+        const int kb = (r * g.S + s) * g.Cred * 2;
+#pragma unroll
+        for(int j = 0; j < BV; j++)
+            bv[j] = (b_ok[j] && cok) ? (unsigned)(b_off[j] + kb) : OOB;
+    };
+    auto step_cursor = [&]() {
+        bool newtap = false;
+        c0 += BKT;
+        if(c0 >= g.Cred) {
+            c0 = 0;
+            newtap = true;
+            if(++si == ns) {
+                si = 0;
+                ++ri;
+            }
+        }
+        if((newtap || ragged) && ri < nr)
+            tap_setup();
+    };
     auto issue_piece = [&](int stage, int p) {
         char *sa = smem + stage * STAGE_BYTES;
         char *sb = sa + BM * ROWB;
-        const bool cok = c0 + kv < g.Cred;
+        const int koff = c0 * 2;
+        // (the offset goes through a local: a captured array element passed directly makes the host pass drop the kernel)
         if(p < AV) {
-            const int j = p;
-            const int tapoff = ((ri * g.IW + si) * sy * g.lda + c0) * 2; // same for all lanes
-            const bool ok = cok && ((amask[j] >> (ri * ns + si)) & 1);
-            const unsigned off = ok ? (unsigned)(rowoff[j] + tapoff) : OOB;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(sa + (j * RPR + wave * RPI) * ROWB), 16, off, 0, 0, 0);
+            const unsigned off = av[p];
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(sa + (p * RPR + wave * RPI) * ROWB), 16, off, koff, 0, 0);
         } else {
-            const int j = p - AV;
-            const int r = r0 + ri * rstep, s = s0 + si * rstep;
-            const int kb = ((r * g.S + s) * g.Cred + c0) * 2;
-            const unsigned off = (b_ok[j] && cok) ? (unsigned)(b_off[j] + kb) : OOB;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(sb + (j * RPR + wave * RPI) * ROWB), 16, off, 0, 0, 0);
+            const unsigned off = bv[p - AV];
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(sb + ((p - AV) * RPR + wave * RPI) * ROWB), 16, off, koff, 0, 0);
         }
     };
     auto issue = [&](int stage) {
 #pragma unroll
         for(int p = 0; p < AV + BV; p++)
             issue_piece(stage, p);
-        advance();
+        step_cursor();
     };
 
     float16_t acc[TM][TN];
@@ -569,6 +621,8 @@ __global__ void __launch_bounds__(64 * (WGM * WGN + PROD), PROD ? (WGM * WGN + P
         fo[kk] = ((2 * kk + (lane >> 5)) ^ swz) * 16;
 
     if constexpr(PROD == 0) {
+        if(KT > 0)
+            tap_setup();
 #pragma unroll
         for(int st = 0; st < STAGES - 1; st++)
             if(st < KT)
@@ -576,46 +630,54 @@ __global__ void __launch_bounds__(64 * (WGM * WGN + PROD), PROD ? (WGM * WGN + P
     }
 
     constexpr int NP = PROD ? 0 : AV + BV, NQ = KS * TM * TN; // load pieces and MFMAs per iteration
-    for(int kt = 0; kt < KT; kt++) {
-        // oldest outstanding slice = kt; newer ones may stay in flight
-        // (a plain __syncthreads() would make the compiler drain every outstanding load)
-        if constexpr(PROD > 0)
-            asm volatile("s_barrier" ::: "memory");
-        else if(kt + STAGES - 2 < KT)
-            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(NP * (STAGES - 2)) : "memory");
-        else
-            asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-        const bool more = !PROD && kt + STAGES - 1 < KT;
-        const int nst = (kt + STAGES - 1) % STAGES;
-        const char *sa = smem + (kt % STAGES) * STAGE_BYTES;
-        const char *sb = sa + BM * ROWB;
-        half8_t fa[KS][TM], fb[KS][TN];
+    // unrolled by the stage count: the stage a slice is read from and the one the next loads go to are
+    // constants, so the LDS addresses are one register per operand and k-step plus immediate offsets
+    for(int kt0 = 0; kt0 < KT; kt0 += STAGES) {
 #pragma unroll
-        for(int kk = 0; kk < KS; kk++) {
+        for(int u = 0; u < STAGES; u++) {
+            const int kt = kt0 + u;
+            if(kt >= KT)
+                break;
+            // oldest outstanding slice = kt; newer ones may stay in flight
+            // (a plain __syncthreads() would make the compiler drain every outstanding load)
+            if constexpr(PROD > 0)
+                asm volatile("s_barrier" ::: "memory");
+            else if(kt + STAGES - 2 < KT)
+                asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(NP * (STAGES - 2)) : "memory");
+            else
+                asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+            const bool more = !PROD && kt + STAGES - 1 < KT;
+            const int nst = (u + STAGES - 1) % STAGES;
+            const char *sa = smem + u * STAGE_BYTES;
+            const char *sb = sa + BM * ROWB;
+            half8_t fa[KS][TM], fb[KS][TN];
 #pragma unroll
-            for(int i = 0; i < TM; i++)
-                fa[kk][i] = *(const half8_t *)(sa + (wm + i * 32 + frow) * ROWB + fo[kk]);
+            for(int kk = 0; kk < KS; kk++) {
 #pragma unroll
-            for(int j = 0; j < TN; j++)
-                fb[kk][j] = *(const half8_t *)(sb + (wn + j * 32 + frow) * ROWB + fo[kk]);
+                for(int i = 0; i < TM; i++)
+                    fa[kk][i] = *(const half8_t *)(sa + (wm + i * 32 + frow) * ROWB + fo[kk]);
+#pragma unroll
+                for(int j = 0; j < TN; j++)
+                    fb[kk][j] = *(const half8_t *)(sb + (wn + j * 32 + frow) * ROWB + fo[kk]);
+            }
+            // the next slice's loads go out between the MFMAs, so that a load waiting for the
+            // memory pipeline does not hold back this wavefront's matrix work
+#pragma unroll
+            for(int q = 0; q < NQ; q++) {
+                const int kk = q / (TM * TN), i = (q / TN) % TM, j = q % TN;
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk][j], fa[kk][i], acc[i][j], 0, 0, 0);
+#pragma unroll
+                for(int p = 0; p < NP; p++)
+                    if(q == (p * NQ) / (NP ? NP : 1)) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        if(more)
+                            issue_piece(nst, p);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+            }
+            if(more)
+                step_cursor();
         }
-        // the next slice's loads go out between the MFMAs, so that a load waiting for the
-        // memory pipeline does not hold back this wavefront's matrix work
-#pragma unroll
-        for(int q = 0; q < NQ; q++) {
-            const int kk = q / (TM * TN), i = (q / TN) % TM, j = q % TN;
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk][j], fa[kk][i], acc[i][j], 0, 0, 0);
-#pragma unroll
-            for(int p = 0; p < NP; p++)
-                if(q == (p * NQ) / (NP ? NP : 1)) {
-                    __builtin_amdgcn_sched_barrier(0);
-                    if(more)
-                        issue_piece(nst, p);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-        }
-        if(more)
-            advance();
     }
 
     // Inference with a folded batch norm: scale = s/sqrt(v+eps) and shift = b - m*scale of the
