@@ -38,9 +38,9 @@ CONV_KINDS = ("convfwd", "convbwddata", "convbwdfilter")
 MEASURED_HBM_BYTES_PER_LAUNCH = {
     # the counters cannot tell fused from plain batch-norm launches (same kernels): both kinds carry
     # the average over all 53 batch-norm launches of a step
-    "bnbwd.fused": 635805665, "bnbwd": 635805665,
-    "bntrain.fused": 285298731, "bntrain": 285298731,
-    "convfwd": 263642790, "convbwddata": 287438380, "convbwdfilter": 308631930,
+    "bnbwd.fused": 635766864, "bnbwd": 635766864,
+    "bntrain.fused": 285296176, "bntrain": 285296176,
+    "convfwd": 264453518, "convbwddata": 287846167, "convbwdfilter": 309137125,
 }
 
 
