@@ -103,6 +103,30 @@ int saga_hip_conv2d_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy
                                const SagaConvParams *p, float alpha, float beta, void *workspace,
                                size_t ws_bytes, saga_stream_t stream);
 
+/* ---- backward data with the filter transposed ahead of time.  No counterpart in the reference (cuDNN
+ *      keeps filter handling inside cudnnConvolutionBackwardData, src/cuda/cuda_dnn.cpp:447-493).
+ *      The fp16 channels-last path of saga_hip_conv2d_bwd_data first copies the K,R,S,C filter to
+ *      C,R,S,K in its workspace - one small launch per layer and step.  A caller that owns a buffer
+ *      per layer can instead transpose every filter of a network in ONE launch
+ *      (saga_hip_filter_transpose_batched, after the optimizer changed the weights) and hand the copy
+ *      in.  saga_hip_conv2d_bwd_data_wt_bytes: size of that copy, 0 when this convolution would not
+ *      take the path (use saga_hip_conv2d_bwd_data).  jobs_device: array in device memory; first_block
+ *      of job j = sum of saga_hip_filter_transpose_blocks over the jobs before it, total_blocks the sum
+ *      over all.  saga_hip_conv2d_bwd_data_wt with wt == NULL is saga_hip_conv2d_bwd_data. */
+typedef struct SagaFilterTransposeJob {
+    const void *w; /* K,R,S,C fp16, dense */
+    void *wt;      /* C,R,S,K fp16, dense, 16-byte aligned */
+    int32_t K, C, RS, first_block;
+} SagaFilterTransposeJob;
+size_t saga_hip_conv2d_bwd_data_wt_bytes(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx,
+                                         const SagaConvParams *p);
+int saga_hip_filter_transpose_blocks(const SagaTensorView *w);
+int saga_hip_filter_transpose_batched(const SagaFilterTransposeJob *jobs_device, int njobs, int total_blocks,
+                                      saga_stream_t stream);
+int saga_hip_conv2d_bwd_data_wt(const SagaTensorView *dy, const SagaTensorView *w, const void *wt, const SagaTensorView *dx,
+                                const SagaConvParams *p, float alpha, float beta, void *workspace, size_t ws_bytes,
+                                saga_stream_t stream);
+
 /* ---- convolution forward that also leaves, for a batch normalisation that consumes y, the
  *      per-channel sum and sum of squares of y as partial[rows][K][2] (one row per block of
  *      output pixels; *partial_rows receives the count).  The reference runs

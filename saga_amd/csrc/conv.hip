@@ -133,6 +133,45 @@ int saga_hip_conv2d_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, 
     return conv_direct_bwd_data(dy, w, dx, g, alpha, beta, as_stream(stream));
 }
 
+size_t saga_hip_conv2d_bwd_data_wt_bytes(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx,
+                                         const SagaConvParams *p)
+{
+    ConvGeom g;
+    if(geometry(dx, w, dy, p, &g) || force_direct() || !conv_mfma_bwd_data_ok(dy, w, dx, g))
+        return 0;
+    return (size_t)g.K * g.C * g.R * g.S * 2;
+}
+
+int saga_hip_filter_transpose_blocks(const SagaTensorView *w)
+{
+    if(!valid_view(w))
+        return 0;
+    return conv_mfma_transpose_blocks(w->dims[0], w->dims[1], w->dims[2] * w->dims[3]);
+}
+
+int saga_hip_filter_transpose_batched(const SagaFilterTransposeJob *jobs_device, int njobs, int total_blocks,
+                                      saga_stream_t stream)
+{
+    if(!jobs_device || njobs < 1 || total_blocks < 1)
+        return SAGA_HIP_EINVAL;
+    return conv_mfma_transpose_batched(jobs_device, njobs, total_blocks, as_stream(stream));
+}
+
+int saga_hip_conv2d_bwd_data_wt(const SagaTensorView *dy, const SagaTensorView *w, const void *wt, const SagaTensorView *dx,
+                                const SagaConvParams *p, float alpha, float beta, void *workspace, size_t ws_bytes,
+                                saga_stream_t stream)
+{
+    if(!wt)
+        return saga_hip_conv2d_bwd_data(dy, w, dx, p, alpha, beta, workspace, ws_bytes, stream);
+    ConvGeom g;
+    int r = geometry(dx, w, dy, p, &g);
+    if(r)
+        return r;
+    if(force_direct() || !conv_mfma_bwd_data_ok(dy, w, dx, g))
+        return SAGA_HIP_EUNSUPPORTED; // only the path saga_hip_conv2d_bwd_data_wt_bytes answered for takes wt
+    return conv_mfma_bwd_data(dy, w, dx, g, alpha, beta, workspace, ws_bytes, as_stream(stream), wt);
+}
+
 int saga_hip_conv2d_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, const SagaTensorView *dw,
                                const SagaConvParams *p, float alpha, float beta, void *workspace,
                                size_t ws_bytes, saga_stream_t stream)

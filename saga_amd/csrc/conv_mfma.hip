@@ -855,6 +855,62 @@ __global__ void __launch_bounds__(64 * (WGM * WGN + PROD), PROD ? (WGM * WGN + P
     }
 }
 
+// Many filters in one launch: job j owns the blocks first_block[j] .. first_block[j+1]-1, one block per
+// (tap, 64 output channels, 64 input channels) tile, transposed through LDS with 16-byte accesses on both
+// sides where K and C are multiples of 8 (element by element otherwise).
+__global__ void __launch_bounds__(256) transpose_filter_batched(const SagaFilterTransposeJob *__restrict__ jobs, int njobs)
+{
+    __shared__ half_t tile[64][72];
+    int lo = 0, hi = njobs - 1;
+    const int b = blockIdx.x;
+    while(lo < hi) { // last job whose first block is <= b
+        const int mid = (lo + hi + 1) >> 1;
+        if(jobs[mid].first_block <= b)
+            lo = mid;
+        else
+            hi = mid - 1;
+    }
+    const SagaFilterTransposeJob job = jobs[lo];
+    const half_t *__restrict__ w = (const half_t *)job.w;
+    half_t *__restrict__ wt = (half_t *)job.wt;
+    const int K = job.K, C = job.C, RS = job.RS;
+    const int tk = (K + 63) / 64, tc = (C + 63) / 64;
+    int r = b - job.first_block;
+    const int c0 = (r % tc) * 64;
+    r /= tc;
+    const int k0 = (r % tk) * 64, tap = r / tk;
+    const int t = threadIdx.x;
+    const bool vec = ((K | C) & 7) == 0 && (((uintptr_t)w | (uintptr_t)wt) & 15) == 0;
+    if(vec) {
+#pragma unroll
+        for(int pass = 0; pass < 2; pass++) {
+            const int row = pass * 32 + (t >> 3), col = (t & 7) * 8;
+            half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+            if(k0 + row < K && c0 + col < C)
+                v = *(const half8_t *)(w + ((int64_t)(k0 + row) * RS + tap) * C + c0 + col);
+            *(half8_t *)&tile[row][col] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for(int pass = 0; pass < 2; pass++) {
+            const int row = pass * 32 + (t >> 3), col = (t & 7) * 8; // row: input channel, col: first of 8 output channels
+            if(c0 + row < C && k0 + col < K) {
+                half8_t v;
+#pragma unroll
+                for(int e = 0; e < 8; e++)
+                    v[e] = tile[col + e][row];
+                *(half8_t *)(wt + ((int64_t)(c0 + row) * RS + tap) * K + k0 + col) = v;
+            }
+        }
+    } else {
+        for(int i = t; i < 64 * 64; i += 256) {
+            const int c = c0 + (i >> 6), k = k0 + (i & 63);
+            if(c < C && k < K)
+                wt[((int64_t)c * RS + tap) * K + k] = w[((int64_t)k * RS + tap) * C + c];
+        }
+    }
+}
+
 // w (K, C, R, S logical; stored K,R,S,C) -> wT stored C,R,S,K
 __global__ void __launch_bounds__(256) transpose_filter(const half_t *__restrict__ w, half_t *__restrict__ wt, int K, int C, int RS)
 {
@@ -1806,8 +1862,26 @@ int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTe
     return rc;
 }
 
+int conv_mfma_transpose_blocks(int K, int C, int RS) { return RS * ((K + 63) / 64) * ((C + 63) / 64); }
+
+int conv_mfma_transpose_batched(const SagaFilterTransposeJob *jobs, int njobs, int total_blocks, hipStream_t st)
+{
+    transpose_filter_batched<<<total_blocks, 256, 0, st>>>(jobs, njobs);
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
+bool conv_mfma_bwd_data_ok(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx, const ConvGeom &g)
+{
+    CLInfo ldy, ldx;
+    return common_ok(dy, w, dx, g, &ldy, &ldx) && ilog2_exact(g.stride) >= 0;
+}
+
+// wt_ready: the filter already transposed to C,R,S,K (by transpose_filter or the batched kernel below);
+// otherwise it is transposed into the workspace first
 int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx,
-                       const ConvGeom &g, float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st)
+                       const ConvGeom &g, float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st,
+                       const void *wt_ready)
 {
     CLInfo ldy, ldx;
     if(!common_ok(dy, w, dx, g, &ldy, &ldx))
@@ -1815,12 +1889,18 @@ int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const 
     const int sshift = ilog2_exact(g.stride);
     if(sshift < 0)
         return SAGA_HIP_EUNSUPPORTED;
-    const size_t need = (size_t)g.K * g.C * g.R * g.S * sizeof(half_t);
-    if(!ws || ws_bytes < need || !aligned16(ws))
-        return SAGA_HIP_EWORKSPACE;
-    half_t *wt = (half_t *)ws;
-    const int64_t total = (int64_t)g.K * g.C * g.R * g.S;
-    transpose_filter<<<grid_for(total, 256, 256 * 16), 256, 0, st>>>((const half_t *)w->ptr, wt, g.K, g.C, g.R * g.S);
+    const half_t *wt = (const half_t *)wt_ready;
+    if(!wt) {
+        const size_t need = (size_t)g.K * g.C * g.R * g.S * sizeof(half_t);
+        if(!ws || ws_bytes < need || !aligned16(ws))
+            return SAGA_HIP_EWORKSPACE;
+        const int64_t total = (int64_t)g.K * g.C * g.R * g.S;
+        transpose_filter<<<grid_for(total, 256, 256 * 16), 256, 0, st>>>((const half_t *)w->ptr, (half_t *)ws, g.K, g.C,
+                                                                        g.R * g.S);
+        wt = (const half_t *)ws;
+    } else if(!aligned16(wt)) {
+        return SAGA_HIP_EINVAL;
+    }
     GatherArgs a;
     a.a = (const half_t *)dy->ptr;
     a.b = wt;

@@ -24,6 +24,11 @@ class ConvParams(C.Structure):
     _fields_ = [("pad", C.c_int32), ("stride", C.c_int32), ("dilation", C.c_int32), ("group", C.c_int32)]
 
 
+class FilterTransposeJob(C.Structure):
+    _fields_ = [("w", C.c_void_p), ("wt", C.c_void_p), ("K", C.c_int32), ("C", C.c_int32), ("RS", C.c_int32),
+                ("first_block", C.c_int32)]
+
+
 class SagaHipError(RuntimeError):
     pass
 
@@ -45,6 +50,10 @@ SIGNATURES = {
                                           _VP]),
     "saga_hip_conv2d_bwd_data": (_I, [_TV, _TV, _TV, C.POINTER(ConvParams), _F, _F, _VP, _SZ, _VP]),
     "saga_hip_conv2d_bwd_filter": (_I, [_TV, _TV, _TV, C.POINTER(ConvParams), _F, _F, _VP, _SZ, _VP]),
+    "saga_hip_conv2d_bwd_data_wt_bytes": (_SZ, [_TV, _TV, _TV, C.POINTER(ConvParams)]),
+    "saga_hip_filter_transpose_blocks": (_I, [_TV]),
+    "saga_hip_filter_transpose_batched": (_I, [_VP, _I, _I, _VP]),
+    "saga_hip_conv2d_bwd_data_wt": (_I, [_TV, _TV, _VP, _TV, C.POINTER(ConvParams), _F, _F, _VP, _SZ, _VP]),
     "saga_hip_bias_add": (_I, [_TV, _TV, _VP]),
     "saga_hip_bias_bwd_workspace_size": (_SZ, [_TV]),
     "saga_hip_bias_bwd": (_I, [_TV, _TV, _F, _VP, _SZ, _VP]),

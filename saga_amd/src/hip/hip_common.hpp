@@ -336,6 +336,9 @@ public:
     void dropGraphs();
     void runOpsGraphed();
 
+    // the operation that transposes the filters of all backward-data convolutions in one launch (hip_ops.cpp)
+    std::shared_ptr<HipOperation> m_transpose_batch;
+
     SagaAux *m_aux = nullptr; // pinned host memory the optimizer kernels write their flags to
     float m_mp_scaling = 1.0f;
     bool m_mp_enabled = false;

@@ -141,23 +141,126 @@ struct ConvFwd : public HipOperation {
     }
 };
 
+// The fp16 channels-last backward-data kernel reads the filter as C,R,S,K.  Instead of one small transpose
+// launch per layer and step, every backward-data operation of a program registers its filter here, and this
+// one operation - placed in the forward list, i.e. after the previous step's optimizer and before any
+// backward operation - transposes them all in a single launch into per-layer tensors.
+struct FilterTransposeBatch : public HipOperation {
+    struct Item {
+        T w, wt;
+    };
+    std::vector<Item> items_;
+    std::unique_ptr<HipMemory> jobs_dev_;
+    std::vector<SagaFilterTransposeJob> jobs_;
+    uint64_t epoch_ = ~(uint64_t)0;
+    int total_blocks_ = 0;
+    bool dirty_ = true;
+    FilterTransposeBatch() : HipOperation("filtertranspose") {}
+    void add(T w, T wt)
+    {
+        items_.push_back({w, wt});
+        dirty_ = true;
+    }
+    void exec(HipProgram &p) override
+    {
+        if(items_.empty())
+            return;
+        if(dirty_ || epoch_ != p.m_ctx->m_mem_epoch) { // a storage moved: the job table holds addresses
+            jobs_.clear();
+            total_blocks_ = 0;
+            for(auto &it : items_) {
+                const SagaTensorView vw = it.w->view();
+                SagaFilterTransposeJob j;
+                j.w = it.w->deviceMem();
+                j.wt = it.wt->deviceMem();
+                j.K = vw.dims[0];
+                j.C = vw.dims[1];
+                j.RS = vw.dims[2] * vw.dims[3];
+                j.first_block = total_blocks_;
+                total_blocks_ += saga_hip_filter_transpose_blocks(&vw);
+                jobs_.push_back(j);
+            }
+            const size_t bytes = jobs_.size() * sizeof(SagaFilterTransposeJob);
+            if(!jobs_dev_ || jobs_dev_->m_bytes < bytes)
+                jobs_dev_ = std::make_unique<HipMemory>(bytes);
+            // synchronous copy of a few kilobytes, only when the table changed; jobs_ stays valid meanwhile
+            chkHip(hipStreamSynchronize(p.m_ctx->m_stream));
+            chkHip(hipMemcpy(jobs_dev_->m_ptr, jobs_.data(), bytes, hipMemcpyHostToDevice));
+            epoch_ = p.m_ctx->m_mem_epoch;
+            dirty_ = false;
+        }
+        chkSaga(saga_hip_filter_transpose_batched((const SagaFilterTransposeJob *)jobs_dev_->m_ptr, (int)jobs_.size(),
+                                                  total_blocks_, S(p)));
+    }
+    HipOpArgs listInputs() const override
+    {
+        HipOpArgs r;
+        for(auto &it : items_)
+            r.push_back({"w", it.w});
+        return r;
+    }
+    HipOpArgs listOutputs() const override
+    {
+        HipOpArgs r;
+        for(auto &it : items_)
+            r.push_back({"wt", it.wt});
+        return r;
+    }
+    bool killOutput(const std::shared_ptr<HipStorage> &s) override
+    {
+        for(size_t i = 0; i < items_.size(); i++)
+            if(items_[i].wt->m_storage == s) {
+                items_.erase(items_.begin() + i);
+                dirty_ = true;
+                return true;
+            }
+        return false;
+    }
+    // the table upload synchronises; keep the operation out of recorded graphs
+    bool graphSafe() const override { return false; }
+    double bytes() const override
+    {
+        double b = 0;
+        for(auto &it : items_)
+            b += 2.0 * nbytes(it.w);
+        return b;
+    }
+};
+
 struct ConvBwdData : public HipOperation {
     const T w_, dy_, dx_;
+    T wt_; // the filter as C,R,S,K, written by the program's FilterTransposeBatch (null: transposed per call)
     const SagaConvParams cp_;
     float beta_ = 0;
-    ConvBwdData(HipProgram &p, T w, T dy, T dx, SagaConvParams cp)
+    ConvBwdData(HipProgram &p, HipProgramUnit &pu, T w, T dy, T dx, SagaConvParams cp)
       : HipOperation("convbwddata"), w_(w), dy_(dy), dx_(dx), cp_(cp)
     {
         const SagaTensorView vx = dx->shapeView(), vw = w->shapeView(), vy = dy->shapeView();
         p.m_ctx->m_workspace.request(saga_hip_conv2d_workspace_size(SAGA_CONV_BWD_DATA, &vx, &vw, &vy, &cp_));
+        const size_t wt_bytes = saga_hip_conv2d_bwd_data_wt_bytes(&vy, &vw, &vx, &cp_);
+        if(wt_bytes && !getenv("SAGA_HIP_NO_BATCHED_TRANSPOSE")) {
+            wt_ = std::make_shared<HipTensor>(Tensor::DataType::HALF, Dims{(int64_t)(wt_bytes / 2)}, HipLayout::NCHW,
+                                              p.m_ctx.get(), w->namePostfix("transposed"));
+            if(!p.m_transpose_batch) {
+                p.m_transpose_batch = std::make_shared<FilterTransposeBatch>();
+                pu.fwd(p.m_transpose_batch);
+            }
+            static_cast<FilterTransposeBatch *>(p.m_transpose_batch.get())->add(w, wt_);
+        }
     }
     void exec(HipProgram &p) override
     {
         const SagaTensorView vdy = dy_->view(), vw = w_->view(), vdx = dx_->view();
-        chkSaga(saga_hip_conv2d_bwd_data(&vdy, &vw, &vdx, &cp_, 1.0f, beta_, p.m_ctx->m_workspace.ptr(),
-                                         p.m_ctx->m_workspace.size(), S(p)));
+        chkSaga(saga_hip_conv2d_bwd_data_wt(&vdy, &vw, wt_ ? wt_->deviceMem() : nullptr, &vdx, &cp_, 1.0f, beta_,
+                                            p.m_ctx->m_workspace.ptr(), p.m_ctx->m_workspace.size(), S(p)));
     }
-    HipOpArgs listInputs() const override { return {{"w", w_}, {"dy", dy_}}; }
+    HipOpArgs listInputs() const override
+    {
+        HipOpArgs r{{"w", w_}, {"dy", dy_}};
+        if(wt_)
+            r.push_back({"wt", wt_});
+        return r;
+    }
     HipOpArgs listOutputs() const override { return {{"dx", dx_}}; }
     float *getBeta(const T &t) override { return t == dx_ ? &beta_ : nullptr; }
     double flops() const override { return conv_flops(dx_, w_, dy_, cp_.group); }
@@ -252,10 +355,10 @@ void conv_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
         pu.bwd(std::make_shared<ConvBwdFilter>(p, x, dy, dw, cp));
         p.upd(n.m_inputs["w"], w, dw);
         if(auto dx = p.lowerGrad(pu, n.m_inputs["x"]))
-            pu.bwd(std::make_shared<ConvBwdData>(p, w, dy, dx, cp));
+            pu.bwd(std::make_shared<ConvBwdData>(p, pu, w, dy, dx, cp));
     } else {
         // transposed convolution: the three kernels with x and y exchanged (:542-574)
-        pu.fwd(std::make_shared<ConvBwdData>(p, w, x, y, cp));
+        pu.fwd(std::make_shared<ConvBwdData>(p, pu, w, x, y, cp));
         if(b)
             pu.fwd(std::make_shared<BiasAdd>(b, y));
         if(!training)
