@@ -38,9 +38,9 @@ CONV_KINDS = ("convfwd", "convbwddata", "convbwdfilter")
 MEASURED_HBM_BYTES_PER_LAUNCH = {
     # the counters cannot tell fused from plain batch-norm launches (same kernels): both kinds carry
     # the average over all 53 batch-norm launches of a step
-    "bnbwd.fused": 635766864, "bnbwd": 635766864,
-    "bntrain.fused": 285296176, "bntrain": 285296176,
-    "convfwd": 264453518, "convbwddata": 287846167, "convbwdfilter": 309137125,
+    "bnbwd.fused": 635799930, "bnbwd": 635799930,
+    "bntrain.fused": 285296483, "bntrain": 285296483,
+    "convfwd": 264287030, "convbwddata": 283369189, "convbwdfilter": 309133801,
 }
 
 
