@@ -109,6 +109,14 @@ int saga_program_run(saga_program_t p, long batches);
 double saga_program_loss_scale(saga_program_t p);
 int saga_program_dump(saga_program_t p, const char *path, int detailed);
 
+/* Optimizer state of a training program: Adam's moments and step counts, the fp32 master weights of
+ * mixed precision and the loss scale, keyed by tensor name ("sagaO001" file).  No counterpart in the
+ * reference, which saves tensors only (Graph::saveTensors, src/graph.cpp:60-104) and so restarts the
+ * optimizer after a reload.  Load into a program built from the same graph after its weights are in
+ * place; every trained tensor needs a name. */
+int saga_program_save_optimizer(saga_program_t p, const char *path);
+int saga_program_load_optimizer(saga_program_t p, const char *path);
+
 /* Per-operation-kind timing (HIP events on the program's stream around every operation) with the
  * algorithmic flops / bytes of the timed launches.  No counterpart in the reference, whose only
  * timing is samples per second (src/cuda/cuda_program.cpp:309-312). */

@@ -87,6 +87,8 @@ SIGNATURES = {
     "saga_program_run": (C.c_int, [_VP, C.c_long]),
     "saga_program_loss_scale": (C.c_double, [_VP]),
     "saga_program_dump": (C.c_int, [_VP, C.c_char_p, C.c_int]),
+    "saga_program_save_optimizer": (C.c_int, [_VP, C.c_char_p]),
+    "saga_program_load_optimizer": (C.c_int, [_VP, C.c_char_p]),
     "saga_program_set_profiling": (C.c_int, [_VP, C.c_int]),
     "saga_program_profile": (C.c_int, [_VP, C.POINTER(_ProfileRow), C.c_int]),
 }
@@ -383,6 +385,15 @@ class Program:
 
     def loss_scale(self):
         return lib().saga_program_loss_scale(self._h)
+
+    def save_optimizer(self, path):
+        """Adam moments, step counts, fp32 master weights and loss scale -> a sagaO001 file."""
+        if lib().saga_program_save_optimizer(self._h, str(path).encode()):
+            raise _err("save_optimizer")
+
+    def load_optimizer(self, path):
+        if lib().saga_program_load_optimizer(self._h, str(path).encode()):
+            raise _err("load_optimizer")
 
     def set_profiling(self, on=True):
         """Time every operation with HIP events on the program's stream (cleared when switched on)."""

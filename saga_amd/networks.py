@@ -243,7 +243,7 @@ def build_graph(net, x, labels=None, with_classifier=True, param_dtype=None):
     for name, a in net.params.items():
         is_bn = name.endswith(("-s", "-m", "-v")) or (name.endswith("-b") and name[:-2] + "-s" in net.params)
         pd = S.FLOAT if is_bn else (param_dtype if param_dtype is not None else dt)
-        t[name] = S.Tensor.from_numpy(a.astype(np_dtype(pd)))
+        t[name] = S.Tensor.from_numpy(a.astype(np_dtype(pd)), name=name)
     for n in net.nodes:
         node = g.add_node(n["type"], {k: t[v] for k, v in n["in"].items()}, n["attrs"], n["name"])
         t[n["out"]] = node.y()

@@ -422,6 +422,24 @@ int saga_context_memory(saga_context_t c, size_t *arena_bytes, size_t *planned_b
 
 double saga_program_loss_scale(saga_program_t p) { return ((ProgramBox *)p)->p->getMPS(); }
 
+static int optimizer_state(saga_program_t p, const char *path, bool save)
+{
+    return guard([&] {
+        auto hp = std::dynamic_pointer_cast<HipProgram>(((ProgramBox *)p)->p);
+        if(!hp)
+            throw std::runtime_error("not a hip program");
+        if(!path)
+            throw std::runtime_error("no path");
+        if(save)
+            hp->saveOptimizerState(path);
+        else
+            hp->loadOptimizerState(path);
+    });
+}
+
+int saga_program_save_optimizer(saga_program_t p, const char *path) { return optimizer_state(p, path, true); }
+int saga_program_load_optimizer(saga_program_t p, const char *path) { return optimizer_state(p, path, false); }
+
 int saga_program_set_profiling(saga_program_t p, int on)
 {
     return guard([&] {

@@ -285,6 +285,9 @@ public:
     void eliminateDeadOps();
     void checkAnomaly(HipOperation &op, const HipOpArgs &tensors, const char *what);
     HipOps createOptimizers();
+    // Adam's moments, step counts, fp32 master weights and the loss scale (hip_optimizer.cpp)
+    void saveOptimizerState(const char *path);
+    void loadOptimizerState(const char *path);
     HipOp createOptimizer(Tensor::DataType dt);
 
     const std::shared_ptr<HipContext> m_ctx;

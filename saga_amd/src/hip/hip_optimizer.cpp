@@ -4,6 +4,7 @@
 // (reference: src/cuda/cuda_optimizer.cpp:196-292; the multi-GPU reduce-scatter / all-gather
 // around the update is not part of this single-GPU engine).
 #include <math.h>
+#include <string.h>
 
 #include "hip_common.hpp"
 
@@ -14,11 +15,20 @@ namespace {
 constexpr double ADAM_B1 = 0.9;   // reference: src/cuda/cuda_kernels.hpp:54
 constexpr double ADAM_B2 = 0.999; // reference: src/cuda/cuda_kernels.hpp:55
 
+// where one parameter sits in the optimizer's flat arrays (elements from the start), by front-end tensor name
+struct OptimizerSlot {
+    std::string name;
+    size_t offset, elements;
+};
+
 struct Optimizer : public HipOperation {
     HipOpArgs m_inputs, m_outputs;
     const std::shared_ptr<HipMemory> m_arena;
     const size_t m_elements; // per half of the arena
     int m_iter = 0;
+    std::vector<OptimizerSlot> m_slots;
+    // the fp32 state arrays, each m_elements long: m, v and - mixed precision - the master weights
+    virtual std::vector<std::pair<const char *, float *>> stateArrays() = 0;
     Optimizer(const char *name, const HipOpArgs &in, const HipOpArgs &out, std::shared_ptr<HipMemory> arena,
               size_t elements)
       : HipOperation(name), m_inputs(in), m_outputs(out), m_arena(arena), m_elements(elements)
@@ -39,6 +49,10 @@ struct AdamF32 : public Optimizer {
     AdamF32(const HipOpArgs &in, const HipOpArgs &out, std::shared_ptr<HipMemory> arena, size_t elements)
       : Optimizer("adam-f32", in, out, arena, elements), m_m(elements * sizeof(float)), m_v(elements * sizeof(float))
     {
+    }
+    std::vector<std::pair<const char *, float *>> stateArrays() override
+    {
+        return {{"m", (float *)m_m.m_ptr}, {"v", (float *)m_v.m_ptr}};
     }
     void exec(HipProgram &p) override
     {
@@ -79,6 +93,10 @@ struct AdamMixed : public Optimizer {
             chkSaga(saga_hip_convert(&src, &dst, 1.0f, (saga_stream_t)p.m_ctx->m_stream));
         }
     }
+    std::vector<std::pair<const char *, float *>> stateArrays() override
+    {
+        return {{"m", (float *)m_m.m_ptr}, {"v", (float *)m_v.m_ptr}, {"master", (float *)m_c.m_ptr}};
+    }
     void exec(HipProgram &p) override
     {
         const int t = ++m_iter;
@@ -117,6 +135,7 @@ HipOp HipProgram::createOptimizer(Tensor::DataType dt)
     char *gbase = wbase + total * esize;
     size_t at = 0;
     HipOpArgs inputs, outputs;
+    std::vector<OptimizerSlot> slots;
     m_ctx->sync();
     for(const auto &u : m_updates) {
         const auto &w = u.second.first;
@@ -142,14 +161,151 @@ HipOp HipProgram::createOptimizer(Tensor::DataType dt)
         inputs.push_back({"g", g});
         inputs.push_back({"w", w});
         outputs.push_back({"w", w});
+        slots.push_back({u.first->m_name ? *u.first->m_name : std::string(), at, n});
         at += (n + align - 1) & ~(align - 1);
     }
+    std::shared_ptr<Optimizer> opt;
     switch(dt) {
-    case Tensor::DataType::FLOAT: return std::make_shared<AdamF32>(inputs, outputs, arena, total);
-    case Tensor::DataType::HALF: return std::make_shared<AdamMixed>(*this, inputs, outputs, arena, total);
+    case Tensor::DataType::FLOAT: opt = std::make_shared<AdamF32>(inputs, outputs, arena, total); break;
+    case Tensor::DataType::HALF: opt = std::make_shared<AdamMixed>(*this, inputs, outputs, arena, total); break;
     default:
         throw std::runtime_error(fmt("Unsupported datatype %s in optimizer", Tensor::DataTypeStr(dt)));
     }
+    opt->m_slots = std::move(slots);
+    return opt;
+}
+
+// ---------------------------------------------------------------- optimizer state files
+//
+// The reference saves tensors only (Graph::saveTensors, src/graph.cpp:60-104), so a reloaded run restarts
+// Adam's moments, bias corrections and loss scale.  This file carries them: per optimizer the step count,
+// and per parameter - keyed by the front-end tensor's name, because the order of the arena follows
+// pointer values and differs from process to process - the slices of m, v and the fp32 master weights.
+//   "sagaO001" | f32 loss scale | u32 optimizers | { char kind[16] | i32 step | u32 arrays | u32 slots |
+//   { u16 name length | name | u64 elements | arrays x f32[elements] } }
+
+namespace {
+const char OPT_MAGIC[8] = {'s', 'a', 'g', 'a', 'O', '0', '0', '1'};
+
+template <typename V> void put(FILE *f, const V &v)
+{
+    if(fwrite(&v, sizeof(V), 1, f) != 1)
+        throw std::runtime_error("optimizer state: write failed");
+}
+template <typename V> V get(FILE *f)
+{
+    V v;
+    if(fread(&v, sizeof(V), 1, f) != 1)
+        throw std::runtime_error("optimizer state: file truncated");
+    return v;
+}
+struct FileCloser {
+    FILE *f;
+    ~FileCloser()
+    {
+        if(f)
+            fclose(f);
+    }
+};
+}  // namespace
+
+void HipProgram::saveOptimizerState(const char *path)
+{
+    finalize();
+    m_ctx->sync();
+    FileCloser fc{fopen(path, "wb")};
+    if(!fc.f)
+        throw std::runtime_error(fmt("optimizer state: cannot create %s", path));
+    std::vector<Optimizer *> opts;
+    for(auto &op : m_ops)
+        if(auto *o = dynamic_cast<Optimizer *>(op.get()))
+            opts.push_back(o);
+    fwrite(OPT_MAGIC, 8, 1, fc.f);
+    put<float>(fc.f, m_mp_scaling);
+    put<uint32_t>(fc.f, (uint32_t)opts.size());
+    std::vector<float> host;
+    for(Optimizer *o : opts) {
+        char kind[16] = {};
+        snprintf(kind, sizeof(kind), "%s", o->name().c_str());
+        fwrite(kind, 16, 1, fc.f);
+        auto arrays = o->stateArrays();
+        put<int32_t>(fc.f, o->m_iter);
+        put<uint32_t>(fc.f, (uint32_t)arrays.size());
+        put<uint32_t>(fc.f, (uint32_t)o->m_slots.size());
+        for(const auto &sl : o->m_slots) {
+            if(sl.name.empty() || sl.name.size() > 65535)
+                throw std::runtime_error("optimizer state: every trained tensor needs a name");
+            put<uint16_t>(fc.f, (uint16_t)sl.name.size());
+            fwrite(sl.name.data(), 1, sl.name.size(), fc.f);
+            put<uint64_t>(fc.f, sl.elements);
+            host.resize(sl.elements);
+            for(auto &a : arrays) {
+                chkHip(hipMemcpy(host.data(), a.second + sl.offset, sl.elements * sizeof(float), hipMemcpyDeviceToHost));
+                if(fwrite(host.data(), sizeof(float), sl.elements, fc.f) != sl.elements)
+                    throw std::runtime_error("optimizer state: write failed");
+            }
+        }
+    }
+}
+
+void HipProgram::loadOptimizerState(const char *path)
+{
+    finalize();
+    m_ctx->sync();
+    FileCloser fc{fopen(path, "rb")};
+    if(!fc.f)
+        throw std::runtime_error(fmt("optimizer state: cannot open %s", path));
+    char magic[8];
+    if(fread(magic, 8, 1, fc.f) != 1 || memcmp(magic, OPT_MAGIC, 8))
+        throw std::runtime_error(fmt("optimizer state: %s is not a sagaO001 file", path));
+    const float scale = get<float>(fc.f);
+    const uint32_t nopt = get<uint32_t>(fc.f);
+    std::vector<Optimizer *> opts;
+    for(auto &op : m_ops)
+        if(auto *o = dynamic_cast<Optimizer *>(op.get()))
+            opts.push_back(o);
+    if(nopt != opts.size())
+        throw std::runtime_error(fmt("optimizer state: file has %u optimizers, the program %zu", nopt, opts.size()));
+    std::vector<float> host;
+    for(uint32_t i = 0; i < nopt; i++) {
+        char kind[17] = {};
+        if(fread(kind, 16, 1, fc.f) != 1)
+            throw std::runtime_error("optimizer state: file truncated");
+        Optimizer *o = nullptr;
+        for(Optimizer *c : opts)
+            if(c->name() == kind)
+                o = c;
+        if(!o)
+            throw std::runtime_error(fmt("optimizer state: the program has no %s optimizer", kind));
+        auto arrays = o->stateArrays();
+        const int32_t iter = get<int32_t>(fc.f);
+        const uint32_t narr = get<uint32_t>(fc.f), nslots = get<uint32_t>(fc.f);
+        if(narr != arrays.size() || nslots != o->m_slots.size())
+            throw std::runtime_error(fmt("optimizer state: %s holds %u arrays of %u tensors, the program %zu of %zu", kind,
+                                         narr, nslots, arrays.size(), o->m_slots.size()));
+        for(uint32_t s = 0; s < nslots; s++) {
+            const uint16_t len = get<uint16_t>(fc.f);
+            std::string name(len, '\0');
+            if(len && fread(&name[0], 1, len, fc.f) != len)
+                throw std::runtime_error("optimizer state: file truncated");
+            const uint64_t n = get<uint64_t>(fc.f);
+            const OptimizerSlot *sl = nullptr;
+            for(const auto &c : o->m_slots)
+                if(c.name == name)
+                    sl = &c;
+            if(!sl || sl->elements != n)
+                throw std::runtime_error(fmt("optimizer state: tensor %s (%llu elements) does not match the program",
+                                             name.c_str(), (unsigned long long)n));
+            host.resize(n);
+            for(auto &a : arrays) {
+                if(fread(host.data(), sizeof(float), n, fc.f) != n)
+                    throw std::runtime_error("optimizer state: file truncated");
+                chkHip(hipMemcpy(a.second + sl->offset, host.data(), n * sizeof(float), hipMemcpyHostToDevice));
+            }
+        }
+        o->m_iter = iter;
+    }
+    m_mp_scaling = scale;
 }
 
 HipOps HipProgram::createOptimizers()
