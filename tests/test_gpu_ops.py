@@ -47,6 +47,11 @@ CONV_CASES = [
     (1, 3, 21, 21, 72, 8, 3, 4, 1),
     (2, 32, 12, 11, 72, 5, 2, 2, 1),
     (5, 96, 10, 10, 40, 3, 1, 1, 1),
+    # dilated (a tenth entry: dilation)
+    (2, 16, 13, 12, 24, 3, 2, 1, 1, 2),
+    (2, 32, 15, 15, 16, 3, 3, 2, 1, 3),
+    (1, 8, 17, 17, 8, 5, 4, 1, 1, 2),
+    (2, 64, 14, 14, 64, 3, 2, 1, 1, 2),
 ]
 
 
@@ -54,31 +59,32 @@ CONV_CASES = [
 @pytest.mark.parametrize("layout,padc", LAYOUTS)
 @pytest.mark.parametrize("case", CONV_CASES)
 def test_conv_fwd_bwd(case, layout, padc, dtype):
-    N, Cc, H, W, Kk, R, pad, stride, group = case
+    N, Cc, H, W, Kk, R, pad, stride, group = case[:9]
+    dil = case[9] if len(case) > 9 else 1
     rng = np.random.default_rng(hash(case) % 1000)
     x = rnd(rng, N, Cc, H, W, dtype=dtype)
     w = rnd(rng, Kk, Cc // group, R, R, dtype=dtype, scale=(2.0 / (Cc // group * R * R)) ** 0.5)
-    y_ref = ref.conv2d_fwd(x, w, pad, stride, 1, group)
+    y_ref = ref.conv2d_fwd(x, w, pad, stride, dil, group)
     dy = rnd(rng, *y_ref.shape, dtype=dtype)
-    dx_ref = ref.conv2d_bwd_data(dy, w, x.shape, pad, stride, 1, group)
-    dw_ref = ref.conv2d_bwd_filter(x, dy, w.shape, pad, stride, 1, group)
+    dx_ref = ref.conv2d_bwd_data(dy, w, x.shape, pad, stride, dil, group)
+    dw_ref = ref.conv2d_bwd_filter(x, dy, w.shape, pad, stride, dil, group)
 
     xd, wd = dev(x, dtype, layout, padc), w_dev(w, dtype, layout)
     yd = dev(np.zeros_like(y_ref), dtype, layout, padc)
-    K.conv2d(K.CONV_FWD, xd, wd, yd, pad, stride, 1, group)
+    K.conv2d(K.CONV_FWD, xd, wd, yd, pad, stride, dil, group)
     assert_close(host(yd), y_ref, dtype, "y")
     # beta = 1 accumulates into the existing output (residual sum folded into the conv)
-    K.conv2d(K.CONV_FWD, xd, wd, yd, pad, stride, 1, group, 1.0, 1.0)
+    K.conv2d(K.CONV_FWD, xd, wd, yd, pad, stride, dil, group, 1.0, 1.0)
     assert_close(host(yd), 2 * y_ref, dtype, "y beta=1")
 
     dyd = dev(dy, dtype, layout, padc)
     dxd = dev(np.zeros_like(x), dtype, layout, padc)
-    K.conv2d(K.CONV_BWD_DATA, dyd, wd, dxd, pad, stride, 1, group)
+    K.conv2d(K.CONV_BWD_DATA, dyd, wd, dxd, pad, stride, dil, group)
     assert_close(host(dxd), dx_ref, dtype, "dx")
     dwd = w_dev(np.zeros_like(w), dtype, layout)
-    K.conv2d(K.CONV_BWD_FILTER, xd, dyd, dwd, pad, stride, 1, group)
+    K.conv2d(K.CONV_BWD_FILTER, xd, dyd, dwd, pad, stride, dil, group)
     assert_close(host(dwd), dw_ref, dtype, "dw")
-    K.conv2d(K.CONV_BWD_FILTER, xd, dyd, dwd, pad, stride, 1, group, 1.0, 1.0)
+    K.conv2d(K.CONV_BWD_FILTER, xd, dyd, dwd, pad, stride, dil, group, 1.0, 1.0)
     assert_close(host(dwd), 2 * dw_ref, dtype, "dw beta=1")
 
 
