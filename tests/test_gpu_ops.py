@@ -88,6 +88,29 @@ def test_conv_fwd_bwd(case, layout, padc, dtype):
     assert_close(host(dwd), 2 * dw_ref, dtype, "dw beta=1")
 
 
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("layout", ["nchw", "nhwc"])
+@pytest.mark.parametrize("R,S", [(1, 3), (3, 1), (2, 5)])
+def test_conv_nonsquare_filter(R, S, layout, dtype):
+    """Filters with R != S (the oracle's pad applies to both axes, as the reference's single `pad` does)."""
+    rng = np.random.default_rng(R * 10 + S)
+    N, Cc, H, W, Kk, pad, stride = 2, 16, 11, 12, 24, 1, 1
+    x = rnd(rng, N, Cc, H, W, dtype=dtype)
+    w = rnd(rng, Kk, Cc, R, S, dtype=dtype, scale=(2.0 / (Cc * R * S)) ** 0.5)
+    y_ref = ref.conv2d_fwd(x, w, pad, stride)
+    dy = rnd(rng, *y_ref.shape, dtype=dtype)
+    xd, wd = dev(x, dtype, layout), w_dev(w, dtype, layout)
+    yd = dev(np.zeros_like(y_ref), dtype, layout)
+    K.conv2d(K.CONV_FWD, xd, wd, yd, pad, stride)
+    assert_close(host(yd), y_ref, dtype, "y")
+    dyd, dxd = dev(dy, dtype, layout), dev(np.zeros_like(x), dtype, layout)
+    K.conv2d(K.CONV_BWD_DATA, dyd, wd, dxd, pad, stride)
+    assert_close(host(dxd), ref.conv2d_bwd_data(dy, w, x.shape, pad, stride), dtype, "dx")
+    dwd = w_dev(np.zeros_like(w), dtype, layout)
+    K.conv2d(K.CONV_BWD_FILTER, xd, dyd, dwd, pad, stride)
+    assert_close(host(dwd), ref.conv2d_bwd_filter(x, dy, w.shape, pad, stride), dtype, "dw")
+
+
 @pytest.mark.parametrize("case", [(2, 64, 14, 64, 3, 1, 1, 3), (3, 32, 9, 160, 1, 0, 1, 1), (2, 128, 13, 24, 3, 1, 2, 0),
                                   (2, 3, 30, 64, 7, 3, 2, 3), (2, 16, 8, 20, 3, 1, 1, 3)])
 def test_conv_with_folded_bn_inference(case):
