@@ -252,6 +252,16 @@ int saga_hip_softmax(const SagaTensorView *x, const SagaTensorView *y, saga_stre
 int saga_hip_spatial_transform(const SagaTensorView *x, const float *theta, const SagaTensorView *y,
                                saga_stream_t stream);
 
+/* ---- dropout: cudnnDropoutForward / cudnnDropoutBackward (src/cuda/cuda_dnn.cpp:1486-1574).
+ *      y = x * keep / (1 - prob), dx = beta*dx + dy * keep / (1 - prob), keep ~ Bernoulli(1 - prob).
+ *      keep is a pure function of (seed, offset, logical N,C,H,W index of the element): the backward pass
+ *      recomputes the mask from the key the forward pass used, nothing is stored (cuDNN keeps it in a
+ *      reserve space).  cuDNN's generator is closed, so masks differ from the reference's; the rule does not. */
+int saga_hip_dropout_fwd(const SagaTensorView *x, const SagaTensorView *y, float prob, uint64_t seed, uint64_t offset,
+                         saga_stream_t stream);
+int saga_hip_dropout_bwd(const SagaTensorView *dy, const SagaTensorView *dx, float prob, uint64_t seed, uint64_t offset,
+                         float beta, saga_stream_t stream);
+
 /* ---- classifier head: catclassifier_fwd / catclassifier_bwd (src/cuda/cuda_kernels.cu:11-96).
  *      x is [N,C] with contiguous rows; pred/labels are int32 [N]; loss fp32 [N] (may be NULL). */
 int saga_hip_catclassifier_fwd(const SagaTensorView *x, int32_t *pred, saga_stream_t stream);

@@ -461,6 +461,86 @@ __global__ void __launch_bounds__(256) fill_bytes(uint8_t *p, uint8_t v, size_t 
 
 } // namespace
 
+// ---------------------------------------------------------------- dropout
+// keep(i) for the logical element index i (N,C,H,W order) comes from a counter-based generator: a 64-bit
+// mix of (seed, offset, i) whose top 32 bits are compared with prob * 2^32.  The backward pass calls the
+// same function with the same key, so no mask is stored.
+__device__ __forceinline__ bool dropout_keep(uint64_t key, uint64_t i, unsigned threshold)
+{
+    uint64_t z = key + i * 0x9e3779b97f4a7c15ull; // splitmix64 finaliser over a Weyl sequence
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    z ^= z >> 31;
+    return (unsigned)(z >> 32) >= threshold;
+}
+
+template <typename T, bool READ_OLD>
+__global__ void __launch_bounds__(256)
+    dropout_k(DView out, DView a, int64_t total, int cl, uint64_t key, unsigned threshold, float scale, float beta)
+{
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    const int C = out.d[1], H = out.d[2], W = out.d[3];
+    for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        int n, c, h, w;
+        int64_t t = i;
+        if(cl) { // walk in the order of a channels-last tensor's memory
+            c = (int)(t % C);
+            t /= C;
+            w = (int)(t % W);
+            t /= W;
+            h = (int)(t % H);
+            n = (int)(t / H);
+        } else {
+            w = (int)(t % W);
+            t /= W;
+            h = (int)(t % H);
+            t /= H;
+            c = (int)(t % C);
+            n = (int)(t / C);
+        }
+        const int64_t logical = (((int64_t)n * C + c) * H + h) * W + w;
+        const int64_t oa = n * a.s[0] + c * a.s[1] + h * a.s[2] + w * a.s[3];
+        const int64_t oo = n * out.s[0] + c * out.s[1] + h * out.s[2] + w * out.s[3];
+        float v = dropout_keep(key, (uint64_t)logical, threshold) ? (float)((const T *)a.ptr)[oa] * scale : 0.0f;
+        if(READ_OLD)
+            v += beta * (float)((T *)out.ptr)[oo];
+        ((T *)out.ptr)[oo] = (T)v;
+    }
+}
+
+static int dropout_launch(const SagaTensorView *a, const SagaTensorView *out, float prob, uint64_t seed, uint64_t offset,
+                          float beta, saga_stream_t stream)
+{
+    if(!valid_view(a) || !valid_view(out) || !(prob >= 0.0f) || !(prob < 1.0f))
+        return SAGA_HIP_EINVAL;
+    if(!same_dims(a, out))
+        return SAGA_HIP_ESHAPE;
+    if(a->dtype != out->dtype || (a->dtype != SAGA_HALF && a->dtype != SAGA_FLOAT))
+        return SAGA_HIP_EUNSUPPORTED;
+    const int64_t total = view_elements(out);
+    const int cl = out->dims[1] > 1 && out->strides[1] == 1;
+    const unsigned threshold = (unsigned)((double)prob * 4294967296.0);
+    const float scale = 1.0f / (1.0f - prob);
+    // one key per (seed, call): the Weyl step inside dropout_keep spreads the element index
+    uint64_t key = seed * 0xd1342543de82ef95ull + offset * 0x2545f4914f6cdd1dull + 0x632be59bd9b4e019ull;
+    hipStream_t st = as_stream(stream);
+    const int g = grid_for(total, 256, 256 * 32);
+#define GO(T)                                                                                                   \
+    do {                                                                                                        \
+        if(beta != 0.0f)                                                                                        \
+            dropout_k<T, true><<<g, 256, 0, st>>>(dview(out), dview(a), total, cl, key, threshold, scale, beta);  \
+        else                                                                                                    \
+            dropout_k<T, false><<<g, 256, 0, st>>>(dview(out), dview(a), total, cl, key, threshold, scale, 0.0f); \
+    } while(0)
+    if(a->dtype == SAGA_HALF)
+        GO(half_t);
+    else
+        GO(float);
+#undef GO
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
 extern "C" {
 
 int saga_hip_act_fwd(int mode, float alpha, const SagaTensorView *x, const SagaTensorView *y, float beta,
@@ -639,6 +719,18 @@ int saga_hip_init(int device, int *cus)
     if(cus)
         *cus = prop.multiProcessorCount;
     return 0;
+}
+
+int saga_hip_dropout_fwd(const SagaTensorView *x, const SagaTensorView *y, float prob, uint64_t seed, uint64_t offset,
+                         saga_stream_t stream)
+{
+    return dropout_launch(x, y, prob, seed, offset, 0.0f, stream);
+}
+
+int saga_hip_dropout_bwd(const SagaTensorView *dy, const SagaTensorView *dx, float prob, uint64_t seed, uint64_t offset,
+                         float beta, saga_stream_t stream)
+{
+    return dropout_launch(dy, dx, prob, seed, offset, beta, stream);
 }
 
 } // extern "C"

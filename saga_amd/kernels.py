@@ -77,6 +77,8 @@ SIGNATURES = {
     "saga_hip_maxpool_bwd_codes": (_I, [_VP, _TV, _TV, _I, _I, _I, _F, _VP]),
     "saga_hip_softmax": (_I, [_TV, _TV, _VP]),
     "saga_hip_spatial_transform": (_I, [_TV, _VP, _TV, _VP]),
+    "saga_hip_dropout_fwd": (_I, [_TV, _TV, _F, C.c_uint64, C.c_uint64, _VP]),
+    "saga_hip_dropout_bwd": (_I, [_TV, _TV, _F, C.c_uint64, C.c_uint64, _F, _VP]),
     "saga_hip_catclassifier_fwd": (_I, [_TV, _VP, _VP]),
     "saga_hip_catclassifier_bwd": (_I, [_TV, _TV, _VP, _VP, _VP, _F, _VP]),
     "saga_hip_adam_f32": (_I, [_SZ, _VP, _VP, _VP, _VP, _F, _F, _F, _F, _VP, _VP]),

@@ -1283,16 +1283,62 @@ void spatialtransform_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
 REGISTER_HIP_OP("spatialtransform", spatialtransform_setup);
 
 // ---------------------------------------------------------------- dropout
-// Inference: identity (the reference aliases it away, :1576-1616).  Training needs a random
-// stream bit-compatible with nothing in particular; it is not offered by this engine.
+// Inference: identity (the reference aliases it away, :1576-1616).  Training (:1486-1574): the mask is a
+// function of (seed, call number, element index); the forward operation counts its calls and the backward
+// operation asks it for the number of the call it answers, so the pair agrees without a stored mask.
+
+struct DropoutFwd : public HipOperation {
+    const T x_, y_;
+    const float prob_;
+    const uint64_t seed_;
+    uint64_t calls_ = 0;
+    DropoutFwd(T x, T y, float prob, uint64_t seed) : HipOperation("dropoutfwd"), x_(x), y_(y), prob_(prob), seed_(seed) {}
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vx = x_->view(), vy = y_->view();
+        chkSaga(saga_hip_dropout_fwd(&vx, &vy, prob_, seed_, ++calls_, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"x", x_}}; }
+    HipOpArgs listOutputs() const override { return {{"y", y_}}; }
+    bool graphSafe() const override { return false; } // the call number is a launch argument
+    double bytes() const override { return nbytes(x_) + nbytes(y_); }
+};
+
+struct DropoutBwd : public HipOperation {
+    const std::shared_ptr<DropoutFwd> fwd_;
+    const T dy_, dx_;
+    float beta_ = 0;
+    DropoutBwd(std::shared_ptr<DropoutFwd> fwd, T dy, T dx) : HipOperation("dropoutbwd"), fwd_(fwd), dy_(dy), dx_(dx) {}
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vdy = dy_->view(), vdx = dx_->view();
+        chkSaga(saga_hip_dropout_bwd(&vdy, &vdx, fwd_->prob_, fwd_->seed_, fwd_->calls_, beta_, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"dy", dy_}}; }
+    HipOpArgs listOutputs() const override { return {{"dx", dx_}}; }
+    float *getBeta(const T &t) override { return t == dx_ ? &beta_ : nullptr; }
+    bool graphSafe() const override { return false; }
+    double bytes() const override { return nbytes(dy_) + nbytes(dx_) * (beta_ != 0 ? 2 : 1); }
+};
 
 void dropout_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
 {
-    if(p.m_pt != ProgramType::INFERENCE)
-        throw std::runtime_error{"dropout is not supported for training by the hip engine"};
     auto x = p.lower(pu, n.m_inputs["x"]);
-    p.m_ctx->m_tensors[n.m_outputs["y"]] =
-        alias_of(x, x->m_dims, x->m_strides, x->m_offset, n.m_outputs["y"]->namePostfix("nop-dropout"));
+    if(p.m_pt == ProgramType::INFERENCE) {
+        p.m_ctx->m_tensors[n.m_outputs["y"]] =
+            alias_of(x, x->m_dims, x->m_strides, x->m_offset, n.m_outputs["y"]->namePostfix("nop-dropout"));
+        return;
+    }
+    auto y = p.lowerLike(pu, n.m_outputs["y"], *x);
+    const float prob = n.m_attributes.get("prob", 0.5f);
+    if(!(prob >= 0.0f && prob < 1.0f))
+        throw std::runtime_error{fmt("dropout: prob %f is outside [0, 1)", prob)};
+    // a different stream of masks per dropout node of the program
+    static const uint64_t base = 0x5a6a5eedull;
+    auto fwd = std::make_shared<DropoutFwd>(x, y, prob, base + 0x100000001b3ull * (uint64_t)(pu.m_fwd.size() + 1));
+    pu.fwd(fwd);
+    if(auto dx = p.lowerGrad(pu, n.m_inputs["x"]))
+        pu.bwd(std::make_shared<DropoutBwd>(fwd, p.lowerGrad(pu, n.m_outputs["y"]), dx));
 }
 REGISTER_HIP_OP("dropout", dropout_setup);
 
