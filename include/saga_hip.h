@@ -268,6 +268,18 @@ int saga_hip_catclassifier_fwd(const SagaTensorView *x, int32_t *pred, saga_stre
 int saga_hip_catclassifier_bwd(const SagaTensorView *x, const SagaTensorView *dx, const int32_t *pred,
                                const int32_t *labels, float *loss, float scale, saga_stream_t stream);
 
+/* ---- L2 loss: loss_bwd_* (src/cuda/cuda_kernels.cu:396-473, called from CudaLossBwd,
+ *      src/cuda/cuda_dnn.cpp:1394-1458).  Per sample n over its c elements: v = x - target,
+ *      dx = v * scale, mmss[n] = {min(0, min v), max(0, max v), mean v, mean v^2} (fp32 [N][4]); the zeros
+ *      in min / max are the reference's (its block reduction pads with zeros).  x, dx: fp16 or fp32,
+ *      target: fp32, or fp16 with fp16 x.  The forward pass of the node is a copy (saga_hip_convert).
+ * ---- tensor statistics: tensor_stats_* (src/cuda/cuda_kernels.cu:313-383, the "stats" node):
+ *      out4 = {min(0, min), max(0, max), mean, variance} over all elements of x. */
+int saga_hip_loss_bwd(const SagaTensorView *x, const SagaTensorView *target, const SagaTensorView *dx, float *mmss,
+                      float scale, saga_stream_t stream);
+size_t saga_hip_tensor_stats_workspace_size(void);
+int saga_hip_tensor_stats(const SagaTensorView *x, float *out4, void *workspace, size_t ws_bytes, saga_stream_t stream);
+
 /* ---- optimizer: adam_float / adam_mixed (src/cuda/cuda_kernels.cu:159-250).
  *      b1t = 1/(1-0.9^t), b2t = 1/(1-0.999^t) are computed by the caller (src/cuda/cuda_optimizer.cpp:79-80).
  *      aux points to a SagaAux in device-visible memory. */

@@ -235,6 +235,25 @@ def avgpool_bwd(dy, xshape, k, pad=0, stride=1, dx=None, beta=0.0):
     return dx
 
 
+def loss_bwd(x, target, scale):
+    """L2 loss node backward: returns dx (like x) and mmss [N,4]"""
+    x, target = _f(x), _f(target)
+    N = x.shape[0]
+    c = int(np.prod(x.shape[1:]))
+    dx = np.empty_like(x)
+    mmss = np.zeros((N, 4), np.float32)
+    lib().so_loss_bwd(_p(x), _p(target), _p(dx), _p(mmss), _i(N), _i(c), _fl(scale))
+    return dx, mmss
+
+
+def tensor_stats(x):
+    """the stats node: {min(0,min), max(0,max), mean, variance}"""
+    x = _f(x)
+    out = np.zeros(4, np.float32)
+    lib().so_tensor_stats(_p(x), _p(out), C.c_size_t(x.size))
+    return out
+
+
 def softmax(x):
     x = _f(x)
     N, Cc, HW = _nchw(x)

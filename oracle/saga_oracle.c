@@ -26,6 +26,8 @@
  *   so_catclassifier_*             in-tree kernel src/cuda/cuda_kernels.cu:11-64 is the spec; closed forms
  *   so_adam_*                      in-tree kernel src/cuda/cuda_kernels.cu:159-230 is the spec; t=1 closed form
  *   so_softmax                     closed form, rows sum to one
+ *   so_loss_bwd, so_tensor_stats   in-tree kernels src/cuda/cuda_kernels.cu:252-473 are the spec (incl. the zeros their
+ *                                  block reduction feeds into min / max); hand-computed case + numpy closed forms
  *   so_spatial_transform           cuDNN's spatial transformer is third-party code outside the reference tree and
  *                                  the reference holds no vectors for it; restated from cuDNN's published rule
  *                                  (normalised coordinates, -1 / 1 = centres of the border pixels, zeros outside)
@@ -641,6 +643,54 @@ void so_spatial_transform(const float *x, const float *theta, float *y, int N, i
 
 /* softmax over C for every (n, spatial) position, max-subtracted
  * (CUDNN_SOFTMAX_ACCURATE, MODE_CHANNEL, src/cuda/cuda_dnn.cpp:1941-1944) */
+/* L2 loss backward (reference: deviceLossReduction + loss_bwd_*, src/cuda/cuda_kernels.cu:396-473): per
+ * sample v = x - target, dx = v * scale; mmss = {min, max, sum / c, sum of squares / c}.  The reference feeds
+ * its per-thread SUMS into the min / max lanes and pads the last reduction stage with zeros
+ * (blockReduceStats, :273-290); with its launch shape (one element per thread) that is min(0, min v) and
+ * max(0, max v). */
+void so_loss_bwd(const float *x, const float *target, float *dx, float *mmss, int N, int c, float scale)
+{
+    for(int n = 0; n < N; n++) {
+        double s = 0, ss = 0;
+        float mn = 0.0f, mx = 0.0f;
+        for(int e = 0; e < c; e++) {
+            const float v = x[(size_t)n * c + e] - target[(size_t)n * c + e];
+            dx[(size_t)n * c + e] = v * scale;
+            if(v < mn)
+                mn = v;
+            if(v > mx)
+                mx = v;
+            s += v;
+            ss += (double)v * v;
+        }
+        mmss[n * 4 + 0] = mn;
+        mmss[n * 4 + 1] = mx;
+        mmss[n * 4 + 2] = (float)(s / c);
+        mmss[n * 4 + 3] = (float)(ss / c);
+    }
+}
+
+/* the "stats" node (reference: deviceReduceStats + compute_mean_stddev, src/cuda/cuda_kernels.cu:313-383):
+ * {min(0, min), max(0, max), mean, (sum of squares - sum^2 / n) / n} */
+void so_tensor_stats(const float *x, float *out4, size_t n)
+{
+    double s = 0, ss = 0;
+    float mn = 0.0f, mx = 0.0f;
+    for(size_t i = 0; i < n; i++) {
+        const float v = x[i];
+        if(v < mn)
+            mn = v;
+        if(v > mx)
+            mx = v;
+        s += v;
+        ss += (double)v * v;
+    }
+    out4[0] = mn;
+    out4[1] = mx;
+    out4[2] = (float)(s / (double)n);
+    out4[3] = (float)((ss - s * s / (double)n) / (double)n);
+}
+
 void so_softmax(const float *x, float *y, int N, int C, int HW)
 {
     for(int n = 0; n < N; n++)

@@ -106,6 +106,108 @@ __global__ void __launch_bounds__(256) softmax_k(DView x, DView y, int64_t total
 
 } // namespace
 
+// ---------------------------------------------------------------- L2 loss and tensor statistics
+//
+// Both report {min, max, mean, second moment or variance} the way the reference's kernels do
+// (src/cuda/cuda_kernels.cu:252-430): its block reduction pads the last stage with zeros, so the reported
+// minimum is min(0, smallest value) and the maximum max(0, largest value).
+
+struct Stat4 {
+    float mn, mx;
+    double s, ss;
+};
+
+__device__ __forceinline__ Stat4 block_stat4(Stat4 v)
+{
+    __shared__ Stat4 red[4];
+#pragma unroll
+    for(int o = 32; o > 0; o >>= 1) {
+        v.mn = fminf(v.mn, __shfl_xor(v.mn, o, 64));
+        v.mx = fmaxf(v.mx, __shfl_xor(v.mx, o, 64));
+        v.s += __shfl_xor(v.s, o, 64);
+        v.ss += __shfl_xor(v.ss, o, 64);
+    }
+    if((threadIdx.x & 63) == 0)
+        red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    Stat4 r = red[0];
+    for(int w = 1; w < 4; w++) {
+        r.mn = fminf(r.mn, red[w].mn);
+        r.mx = fmaxf(r.mx, red[w].mx);
+        r.s += red[w].s;
+        r.ss += red[w].ss;
+    }
+    return r;
+}
+
+// element e (row-major over C,H,W) of sample n
+__device__ __forceinline__ int64_t sample_off(const DView &v, int n, int64_t e)
+{
+    const int w = (int)(e % v.d[3]);
+    e /= v.d[3];
+    const int h = (int)(e % v.d[2]);
+    const int c = (int)(e / v.d[2]);
+    return n * v.s[0] + c * v.s[1] + h * v.s[2] + w * v.s[3];
+}
+
+// one block per sample: v = x - target, dx = v * scale, mmss[n] = {min(0,v), max(0,v), mean v, mean v^2}
+template <typename T, typename TT>
+__global__ void __launch_bounds__(256) loss_bwd_k(DView x, DView target, DView dx, float *__restrict__ mmss, float scale)
+{
+    const int n = blockIdx.x;
+    const int64_t c = (int64_t)x.d[1] * x.d[2] * x.d[3];
+    Stat4 a = {0.0f, 0.0f, 0.0, 0.0};
+    for(int64_t e = threadIdx.x; e < c; e += 256) {
+        const float v = (float)((const T *)x.ptr)[sample_off(x, n, e)] - (float)((const TT *)target.ptr)[sample_off(target, n, e)];
+        ((T *)dx.ptr)[sample_off(dx, n, e)] = (T)(v * scale);
+        a.mn = fminf(a.mn, v);
+        a.mx = fmaxf(a.mx, v);
+        a.s += v;
+        a.ss += (double)v * v;
+    }
+    a = block_stat4(a);
+    if(threadIdx.x == 0) {
+        mmss[n * 4 + 0] = a.mn;
+        mmss[n * 4 + 1] = a.mx;
+        mmss[n * 4 + 2] = (float)(a.s / (double)c);
+        mmss[n * 4 + 3] = (float)(a.ss / (double)c);
+    }
+}
+
+// partial[b] = statistics of the elements block b strides over (logical order, any strides)
+template <typename T> __global__ void __launch_bounds__(256) stats_partial_k(DView x, int64_t total, Stat4 *__restrict__ partial)
+{
+    const int64_t per = (int64_t)x.d[1] * x.d[2] * x.d[3];
+    Stat4 a = {0.0f, 0.0f, 0.0, 0.0};
+    for(int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const float v = (float)((const T *)x.ptr)[sample_off(x, (int)(i / per), i % per)];
+        a.mn = fminf(a.mn, v);
+        a.mx = fmaxf(a.mx, v);
+        a.s += v;
+        a.ss += (double)v * v;
+    }
+    a = block_stat4(a);
+    if(threadIdx.x == 0)
+        partial[blockIdx.x] = a;
+}
+
+__global__ void __launch_bounds__(64) stats_final_k(const Stat4 *__restrict__ partial, int blocks, double n, float *__restrict__ out)
+{
+    if(threadIdx.x != 0)
+        return;
+    Stat4 r = partial[0];
+    for(int b = 1; b < blocks; b++) { // fixed order: the same result every run
+        r.mn = fminf(r.mn, partial[b].mn);
+        r.mx = fmaxf(r.mx, partial[b].mx);
+        r.s += partial[b].s;
+        r.ss += partial[b].ss;
+    }
+    out[0] = r.mn;
+    out[1] = r.mx;
+    out[2] = (float)(r.s / n);
+    out[3] = (float)((r.ss - r.s * r.s / n) / n);
+}
+
 extern "C" {
 
 int saga_hip_catclassifier_fwd(const SagaTensorView *x, int32_t *pred, saga_stream_t stream)
@@ -170,6 +272,51 @@ int saga_hip_softmax(const SagaTensorView *x, const SagaTensorView *y, saga_stre
         softmax_k<float><<<g, 256, 0, st>>>(dview(x), dview(y), total);
     else
         return SAGA_HIP_EUNSUPPORTED;
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
+int saga_hip_loss_bwd(const SagaTensorView *x, const SagaTensorView *target, const SagaTensorView *dx, float *mmss,
+                      float scale, saga_stream_t stream)
+{
+    if(!valid_view(x) || !valid_view(target) || !valid_view(dx) || !mmss)
+        return SAGA_HIP_EINVAL;
+    if(!same_dims(x, target) || !same_dims(x, dx))
+        return SAGA_HIP_ESHAPE;
+    if(x->dtype != dx->dtype)
+        return SAGA_HIP_EUNSUPPORTED;
+    hipStream_t st = as_stream(stream);
+    const int N = x->dims[0];
+    if(x->dtype == SAGA_HALF && target->dtype == SAGA_FLOAT)
+        loss_bwd_k<half_t, float><<<N, 256, 0, st>>>(dview(x), dview(target), dview(dx), mmss, scale);
+    else if(x->dtype == SAGA_HALF && target->dtype == SAGA_HALF)
+        loss_bwd_k<half_t, half_t><<<N, 256, 0, st>>>(dview(x), dview(target), dview(dx), mmss, scale);
+    else if(x->dtype == SAGA_FLOAT && target->dtype == SAGA_FLOAT)
+        loss_bwd_k<float, float><<<N, 256, 0, st>>>(dview(x), dview(target), dview(dx), mmss, scale);
+    else
+        return SAGA_HIP_EUNSUPPORTED; // the combinations of the reference (src/cuda/cuda_dnn.cpp:1415-1440)
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
+size_t saga_hip_tensor_stats_workspace_size(void) { return 256 * sizeof(Stat4); }
+
+int saga_hip_tensor_stats(const SagaTensorView *x, float *out4, void *workspace, size_t ws_bytes, saga_stream_t stream)
+{
+    if(!valid_view(x) || !out4)
+        return SAGA_HIP_EINVAL;
+    if(!workspace || ws_bytes < saga_hip_tensor_stats_workspace_size() || ((uintptr_t)workspace & 7))
+        return SAGA_HIP_EWORKSPACE;
+    const int64_t total = view_elements(x);
+    const int blocks = grid_for(total, 256 * 16, 256);
+    hipStream_t st = as_stream(stream);
+    if(x->dtype == SAGA_HALF)
+        stats_partial_k<half_t><<<blocks, 256, 0, st>>>(dview(x), total, (Stat4 *)workspace);
+    else if(x->dtype == SAGA_FLOAT)
+        stats_partial_k<float><<<blocks, 256, 0, st>>>(dview(x), total, (Stat4 *)workspace);
+    else
+        return SAGA_HIP_EUNSUPPORTED;
+    stats_final_k<<<1, 64, 0, st>>>((const Stat4 *)workspace, blocks, (double)total, out4);
     SAGA_CHECK_LAUNCH();
     return 0;
 }

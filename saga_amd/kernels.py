@@ -81,6 +81,9 @@ SIGNATURES = {
     "saga_hip_dropout_bwd": (_I, [_TV, _TV, _F, C.c_uint64, C.c_uint64, _F, _VP]),
     "saga_hip_catclassifier_fwd": (_I, [_TV, _VP, _VP]),
     "saga_hip_catclassifier_bwd": (_I, [_TV, _TV, _VP, _VP, _VP, _F, _VP]),
+    "saga_hip_loss_bwd": (_I, [_TV, _TV, _TV, _VP, _F, _VP]),
+    "saga_hip_tensor_stats_workspace_size": (_SZ, []),
+    "saga_hip_tensor_stats": (_I, [_TV, _VP, _VP, _SZ, _VP]),
     "saga_hip_adam_f32": (_I, [_SZ, _VP, _VP, _VP, _VP, _F, _F, _F, _F, _VP, _VP]),
     "saga_hip_adam_mixed": (_I, [_SZ, _F, _VP, _VP, _VP, _VP, _VP, _F, _F, _F, _F, _VP, _VP]),
     "saga_hip_fill": (_I, [_VP, _I, _SZ, _VP]),

@@ -1282,6 +1282,73 @@ void spatialtransform_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
 }
 REGISTER_HIP_OP("spatialtransform", spatialtransform_setup);
 
+// ---------------------------------------------------------------- L2 loss, tensor statistics
+// loss (reference: CudaLossFwd / CudaLossBwd, src/cuda/cuda_dnn.cpp:1358-1482): forward copies x to y (in
+// y's type), backward leaves dx = (x - target) * strength / N (times the loss scale) and the per-sample
+// {min, max, mean, mean square} of the residual in mmss.
+// stats (reference: CudaStats, :2638-2680): statistics of an already lowered tensor, run in the tail.
+
+struct LossBwd : public HipOperation {
+    const T x_, target_, dx_, mmss_;
+    const float strength_;
+    LossBwd(T x, T target, T dx, T mmss, float strength)
+      : HipOperation("lossbwd"), x_(x), target_(target), dx_(dx), mmss_(mmss), strength_(strength)
+    {
+    }
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vx = x_->view(), vt = target_->view(), vdx = dx_->view();
+        const float scale = strength_ / (float)x_->m_dims[0] * p.m_mp_scaling; // :1412, :1419
+        chkSaga(saga_hip_loss_bwd(&vx, &vt, &vdx, (float *)mmss_->deviceMem(), scale, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"x", x_}, {"target", target_}}; }
+    HipOpArgs listOutputs() const override { return {{"dx", dx_}, {"mmss", mmss_}}; }
+    bool graphSafe() const override { return false; } // the loss scale is a launch argument
+};
+
+void loss_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
+{
+    auto x = p.lower(pu, n.m_inputs["x"]);
+    auto y = p.lowerLike(pu, n.m_outputs["y"], *x);
+    pu.fwd(std::make_shared<Convert>(x, y, 1.0f));
+    if(p.m_pt == ProgramType::INFERENCE)
+        return;
+    auto dx = p.lowerGrad(pu, n.m_inputs["x"]);
+    auto target = p.lowerLike(pu, n.m_inputs["target"], *x);
+    auto mmss = p.lower(pu, n.m_outputs["mmss"]);
+    if(!dx || !mmss)
+        throw std::runtime_error{"loss: needs a gradient for x and the mmss output"};
+    pu.bwd(std::make_shared<LossBwd>(x, target, dx, mmss, n.m_attributes.get("strength", 1.0f)));
+}
+REGISTER_HIP_OP("loss", loss_setup);
+
+struct Stats : public HipOperation {
+    const T x_, y_;
+    Stats(HipProgram &p, T x, T y) : HipOperation("stats"), x_(x), y_(y)
+    {
+        p.m_ctx->m_workspace.request(saga_hip_tensor_stats_workspace_size());
+    }
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vx = x_->view();
+        chkSaga(saga_hip_tensor_stats(&vx, (float *)y_->deviceMem(), p.m_ctx->m_workspace.ptr(), p.m_ctx->m_workspace.size(),
+                                      S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"x", x_}}; }
+    HipOpArgs listOutputs() const override { return {{"y", y_}}; }
+};
+
+void stats_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
+{
+    // like the reference, the node inspects a tensor some other node of the program lowered (:2668-2678)
+    auto it = p.m_ctx->m_tensors.find(n.m_inputs["x"]);
+    if(it == p.m_ctx->m_tensors.end())
+        throw std::runtime_error{"x-tensor not found"};
+    auto y = p.lower(pu, n.m_outputs["y"]);
+    pu.tail(std::make_shared<Stats>(p, it->second, y));
+}
+REGISTER_HIP_OP("stats", stats_setup);
+
 // ---------------------------------------------------------------- dropout
 // Inference: identity (the reference aliases it away, :1576-1616).  Training (:1486-1574): the mask is a
 // function of (seed, call number, element index); the forward operation counts its calls and the backward

@@ -160,6 +160,27 @@ def test_catclassifier():
     np.testing.assert_allclose(dx.sum(1), 0, atol=1e-6)  # softmax gradient rows sum to zero
 
 
+def test_loss_and_stats():
+    # hand-computed: v = [1, -2, 3] and [0.5, 0.5, 4]
+    x = np.array([[2.0, 0.0, 4.0], [1.0, 2.5, 4.0]], np.float32)
+    t = np.array([[1.0, 2.0, 1.0], [0.5, 2.0, 0.0]], np.float32)
+    dx, mmss = ref.loss_bwd(x, t, 0.5)
+    np.testing.assert_allclose(dx, [[0.5, -1.0, 1.5], [0.25, 0.25, 2.0]])
+    np.testing.assert_allclose(mmss[0], [-2.0, 3.0, 2.0 / 3, 14.0 / 3], rtol=1e-6)
+    # all residuals positive: the minimum is the reference's padded zero, not 0.5
+    np.testing.assert_allclose(mmss[1], [0.0, 4.0, 5.0 / 3, 16.5 / 3], rtol=1e-6)
+    a = rnd(3, 4, 5, 6)
+    b = rnd(3, 4, 5, 6)
+    dx, mmss = ref.loss_bwd(a, b, 0.25)
+    v = (a - b).reshape(3, -1)
+    np.testing.assert_allclose(dx.reshape(3, -1), v * 0.25, rtol=1e-6)
+    np.testing.assert_allclose(mmss, np.stack([np.minimum(v.min(1), 0), np.maximum(v.max(1), 0), v.mean(1), (v * v).mean(1)], 1),
+                               rtol=1e-5, atol=1e-6)
+    st = ref.tensor_stats(a)
+    np.testing.assert_allclose(st, [min(a.min(), 0), max(a.max(), 0), a.mean(), a.var()], rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(ref.tensor_stats(np.abs(a) + 1)[0], 0.0)  # strictly positive data still report min 0
+
+
 def test_softmax():
     x = rnd(2, 5, 3, 3)
     y = ref.softmax(x)
