@@ -147,6 +147,38 @@ def copy_calibration():
     print(json.dumps({"copy_bytes": n * 4, "launches": 5}))
 
 
+def host_input_rate(args):
+    """The same two programs with the image batch and the labels declared as batched tensors: every step the
+    engine uploads the host's back buffers (pinned memory, hipMemcpyAsync on the program's stream) before it
+    runs, as it does for the reference's harness.  Reported beside the headline, never as `value`."""
+    import torch
+    from saga_amd import api as S
+    from saga_amd import networks as N
+
+    net = N.resnet50(args.batch, image=args.image)
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((args.batch, 3, args.image, args.image)).astype(np.float16)
+    ctx = S.Context()
+    graph, t = N.build_graph(net, x)
+    pre = 1  # Phase::PRE
+    train = ctx.create_program(graph, args.batch, training=True, learning_rate=1e-4, initial_loss_scale=1024.0,
+                               batched={t[net.input]: pre, t["labels"]: pre})
+    infer = ctx.create_program(graph, args.batch, training=False, batched={t[net.input]: pre})
+    ctx.resolve(t["loss"])
+    ctx.resolve(t["pred"])
+    out = {"host_bytes_per_step": int(x.nbytes + args.batch * 4)}
+    for name, prog in (("train", train), ("infer", infer)):
+        prog.run(args.warmup)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        prog.run(args.steps)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        out[name + "_images_per_sec"] = round(args.batch * args.steps / dt, 1)
+        out[name + "_ms_per_step"] = round(dt / args.steps * 1e3, 3)
+    print(json.dumps({"pcie_inclusive": out}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -159,6 +191,8 @@ def main():
     ap.add_argument("--no-profile", action="store_true")
     ap.add_argument("--per-op", metavar="FILE",
                     help="also write one line per operation of the training step (time, rate, own roofline bound)")
+    ap.add_argument("--host-input", action="store_true",
+                    help="time the programs with the batch handed over from host memory every step (PCIe included) and exit")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run a plain 1 GiB device copy five times and exit (reference for the HBM counters)")
     args = ap.parse_args()
@@ -166,6 +200,8 @@ def main():
         sys.exit("bench.py: this build drives exactly one GPU (no collectives, no sharding); run with --gpus 1")
     if args.copy_calibration:
         return copy_calibration()
+    if args.host_input:
+        return host_input_rate(args)
 
     os.environ.setdefault("SAGA_HIP_PROFILE_PER_OP", "1")  # profile rows per operation, see by_kind()
     from saga_amd import api as S

@@ -217,11 +217,17 @@ public:
     void reset() override;
     void bindToHostThread() override { chkHip(hipSetDevice(m_device)); }
 
-    void sync() { chkHip(hipStreamSynchronize(m_stream)); }
+    void sync()
+    {
+        chkHip(hipStreamSynchronize(m_stream));
+        chkHip(hipStreamSynchronize(m_copy_stream));
+    }
 
     const std::shared_ptr<UI> m_ui;
     const int m_device;
     hipStream_t m_stream = nullptr;
+    // uploads of the batched tensors' BACK buffers: they run beside the step that computes on the front buffers
+    hipStream_t m_copy_stream = nullptr;
     int m_num_cu = 0;
     int m_storage_id_gen = 0;
     int m_program_index_gen = 0;

@@ -142,6 +142,7 @@ HipContext::HipContext(const std::shared_ptr<UI> &ui, int device) : m_ui(ui), m_
     chkHip(hipSetDevice(device));
     chkSaga(saga_hip_init(device, &m_num_cu));
     chkHip(hipStreamCreateWithFlags(&m_stream, hipStreamDefault));
+    chkHip(hipStreamCreateWithFlags(&m_copy_stream, hipStreamDefault));
     hipDeviceProp_t prop;
     chkHip(hipGetDeviceProperties(&prop, device));
     m_ui->updateCell(getUiPage(), 0, 0, UI::Align::LEFT, "%s", prop.name);
@@ -154,6 +155,10 @@ HipContext::~HipContext()
     if(m_stream) {
         (void)hipStreamSynchronize(m_stream);
         (void)hipStreamDestroy(m_stream);
+    }
+    if(m_copy_stream) {
+        (void)hipStreamSynchronize(m_copy_stream);
+        (void)hipStreamDestroy(m_copy_stream);
     }
 }
 
@@ -611,12 +616,15 @@ void HipProgram::runCallbacks(const TensorBatchCallback &cb, long batch, Phase p
     cb(batch, *this, amap);
 }
 
-// Upload what the host wrote into the back buffers, then swap front and back.
+// Upload what the host wrote into the back buffers, then swap front and back.  The uploads go to the
+// copy stream: the operations of the step in flight only touch the front buffers, so the transfer
+// overlaps them; every caller synchronises both streams (HipContext::sync) before the next step is
+// enqueued, which is when the swapped buffers are first read.
 void HipProgram::flip(Phase upload_phase)
 {
     for(auto &bt : m_batched) {
         if(!!(bt.second.second & upload_phase))
-            bt.second.first->uploadBack(m_ctx->m_stream);
+            bt.second.first->uploadBack(m_ctx->m_copy_stream);
         bt.second.first->flip();
     }
 }
