@@ -72,7 +72,9 @@ __device__ __forceinline__ void decode(int64_t i, int C, int H, int W, int &n, i
     }
 }
 
-__device__ __forceinline__ bool better(float v, float best) { return v > best || (v != v && best == best); }
+// v replaces best when it is larger, or when it is the first NaN: "not (v <= best)" holds for both, and a NaN
+// already held is never replaced (two compares; the spelled-out form costs three and more mask logic)
+__device__ __forceinline__ bool better(float v, float best) { return !(v <= best) && best == best; }
 __device__ __forceinline__ bool same(float a, float b) { return a == b || (a != a && b != b); }
 
 template <typename T, int VN, int MODE>
