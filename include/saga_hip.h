@@ -38,7 +38,8 @@ enum SagaError {
     SAGA_HIP_EINVAL = -1,       /* malformed argument (null pointer, negative size ...) */
     SAGA_HIP_ESHAPE = -2,       /* operand shapes do not agree */
     SAGA_HIP_EUNSUPPORTED = -3, /* valid but not implemented (dtype / layout combination) */
-    SAGA_HIP_EWORKSPACE = -4    /* workspace missing or too small */
+    SAGA_HIP_EWORKSPACE = -4,   /* workspace missing or too small */
+    SAGA_HIP_ETOOLARGE = -5     /* operand beyond the fixed scratch of an entry point that allocates nothing */
 };
 
 /*
@@ -160,6 +161,17 @@ int saga_hip_bias_add(const SagaTensorView *y, const SagaTensorView *b, saga_str
 size_t saga_hip_bias_bwd_workspace_size(const SagaTensorView *dy);
 int saga_hip_bias_bwd(const SagaTensorView *dy, const SagaTensorView *db, float beta, void *workspace, size_t ws_bytes,
                       saga_stream_t stream);
+
+/* saga_hip_bias_bwd for callers that cannot allocate (code under HIP graph capture, serving loops and harnesses
+ * that forbid hipMalloc and so cannot provide a workspace).  No counterpart in the reference.  Same result as
+ * saga_hip_bias_bwd; the partial sums of the two-pass reduction live in a fixed array of
+ * SAGA_HIP_BIAS_BWD_NOALLOC_MAX_BYTES of device memory that every GPU the library runs on holds until the
+ * process ends.  Returns SAGA_HIP_ETOOLARGE, with nothing written, when saga_hip_bias_bwd_workspace_size(dy)
+ * exceeds that (channels-last tensors of more than 2048 channels once they have 2^20 elements).  The
+ * device the stream belongs to must be current.  All calls on one GPU share the array: calls that overlap
+ * on one GPU (two streams, two threads) race; calls in stream order do not. */
+#define SAGA_HIP_BIAS_BWD_NOALLOC_MAX_BYTES (4u << 20)
+int saga_hip_bias_bwd_noalloc(const SagaTensorView *dy, const SagaTensorView *db, float beta, saga_stream_t stream);
 
 /* ---- GEMM: cublasSgemm / cublasHgemm as used by the fc node (src/cuda/cuda_dnn.cpp:1001-1025).
  *      Row-major: C[M,N] = alpha * op(A) * op(B) + beta * C, op(A) is MxK, op(B) is KxN;

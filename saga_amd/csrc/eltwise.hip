@@ -2,6 +2,7 @@
 // All are HBM-bound: the fast paths move 16 bytes per lane per access and keep every
 // wavefront on consecutive addresses; odd layouts fall back to a strided gather.
 #include "common.hpp"
+#include <atomic>
 
 namespace {
 
@@ -632,8 +633,9 @@ size_t saga_hip_bias_bwd_workspace_size(const SagaTensorView *dy)
     return gx > 1 ? (size_t)gx * cl.C * sizeof(float) : 0;
 }
 
-int saga_hip_bias_bwd(const SagaTensorView *dy, const SagaTensorView *db, float beta, void *workspace, size_t ws_bytes,
-                      saga_stream_t stream)
+// Shared by saga_hip_bias_bwd (the caller's workspace) and saga_hip_bias_bwd_noalloc (the library's scratch array).
+static int bias_bwd_run(const SagaTensorView *dy, const SagaTensorView *db, float beta, void *workspace, size_t ws_bytes,
+                        saga_stream_t stream)
 {
     if(!valid_view(dy) || !valid_view(db))
         return SAGA_HIP_EINVAL;
@@ -681,6 +683,60 @@ int saga_hip_bias_bwd(const SagaTensorView *dy, const SagaTensorView *db, float 
     return 0;
 }
 
+int saga_hip_bias_bwd(const SagaTensorView *dy, const SagaTensorView *db, float beta, void *workspace, size_t ws_bytes,
+                      saga_stream_t stream)
+{
+    return bias_bwd_run(dy, db, beta, workspace, ws_bytes, stream);
+}
+
+// ---- the entry point that allocates nothing.  The per-block partial sums of the two-pass reduction go to a
+// fixed array in device memory instead of a workspace.  Every GPU holds its own copy of the array at its own
+// address, resolved once per device (saga_hip_init, or the first call on that device) and kept in
+// bias_scratch_ptr; host code passes that pointer, never the array's name, to the kernels.  The partial kernels
+// overwrite every [block][channel] entry the final kernel reads, so nothing has to be cleared between calls.
+static __device__ __align__(256) float scratch[SAGA_HIP_BIAS_BWD_NOALLOC_MAX_BYTES / sizeof(float)];
+static constexpr int MAX_SCRATCH_DEVICES = 64;
+static std::atomic<float *> bias_scratch_ptr[MAX_SCRATCH_DEVICES];
+
+// `device` must be the current device.
+static int resolve_bias_scratch(int device, float **out)
+{
+    if(device < 0 || device >= MAX_SCRATCH_DEVICES)
+        return SAGA_HIP_EINVAL;
+    float *p = bias_scratch_ptr[device].load(std::memory_order_acquire);
+    if(!p) {
+        const hipError_t e = hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch));
+        if(e != hipSuccess)
+            return (int)e;
+        if(!p)
+            return SAGA_HIP_EINVAL;
+        bias_scratch_ptr[device].store(p, std::memory_order_release);
+    }
+    if(out)
+        *out = p;
+    return 0;
+}
+
+int saga_hip_bias_bwd_noalloc(const SagaTensorView *dy, const SagaTensorView *db, float beta, saga_stream_t stream)
+{
+    if(!valid_view(dy) || !valid_view(db))
+        return SAGA_HIP_EINVAL;
+    const size_t need = saga_hip_bias_bwd_workspace_size(dy);
+    if(need > SAGA_HIP_BIAS_BWD_NOALLOC_MAX_BYTES)
+        return SAGA_HIP_ETOOLARGE;
+    float *ws = nullptr;
+    if(need) {
+        int device = -1;
+        const hipError_t e = hipGetDevice(&device);
+        if(e != hipSuccess)
+            return (int)e;
+        const int rc = resolve_bias_scratch(device, &ws);
+        if(rc)
+            return rc;
+    }
+    return bias_bwd_run(dy, db, beta, ws, need, stream);
+}
+
 int saga_hip_fill(void *ptr, int value, size_t bytes, saga_stream_t stream)
 {
     if(!ptr && bytes)
@@ -701,6 +757,7 @@ const char *saga_hip_error_string(int code)
     case SAGA_HIP_ESHAPE: return "operand shapes do not agree";
     case SAGA_HIP_EUNSUPPORTED: return "unsupported dtype or layout";
     case SAGA_HIP_EWORKSPACE: return "workspace missing or too small";
+    case SAGA_HIP_ETOOLARGE: return "operand needs more scratch than the entry point that allocates nothing holds";
     }
     if(code > 0)
         return hipGetErrorString((hipError_t)code);
@@ -718,7 +775,7 @@ int saga_hip_init(int device, int *cus)
         return (int)e;
     if(cus)
         *cus = prop.multiProcessorCount;
-    return 0;
+    return resolve_bias_scratch(device, nullptr);
 }
 
 int saga_hip_dropout_fwd(const SagaTensorView *x, const SagaTensorView *y, float prob, uint64_t seed, uint64_t offset,

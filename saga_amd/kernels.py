@@ -57,6 +57,7 @@ SIGNATURES = {
     "saga_hip_bias_add": (_I, [_TV, _TV, _VP]),
     "saga_hip_bias_bwd_workspace_size": (_SZ, [_TV]),
     "saga_hip_bias_bwd": (_I, [_TV, _TV, _F, _VP, _SZ, _VP]),
+    "saga_hip_bias_bwd_noalloc": (_I, [_TV, _TV, _F, _VP]),
     "saga_hip_gemm": (_I, [_I, _I, _I, _I, _I, _F, _VP, _I, _VP, _I, _F, _VP, _I, _I, _VP]),
     "saga_hip_bn_infer": (_I, [_TV, _TV, _TV, _VP, _VP, _VP, _VP, _F, _I, _VP]),
     "saga_hip_bn_workspace_size": (_SZ, [_TV]),
