@@ -9,6 +9,10 @@ fp16 (src/cuda/cuda_dnn.cpp:1297-1315), and the optimizer runs after backward
 (src/cuda/cuda_optimizer.cpp).  For fp16 networks every stored tensor is rounded to fp16 as
 the device does; arithmetic inside an operator stays in fp32/fp64.
 Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg import this module.
+
+Pinning: tests/test_oracle_net.py compares forward, every parameter gradient, the running statistics, the
+loss_scale/N factor, five fp32 training steps and an overflowing mixed-precision run (skipped elements, flags,
+loss-scale rule) with torch-CPU double autograd and a numpy Adam written from the reference kernel.
 """
 import numpy as np
 

@@ -15,6 +15,7 @@
  *   so_conv2d_fwd, so_bias_add     reference vectors test/test_ops.cpp:31-215, test_resnode
  *   so_conv2d_bwd_data             reference vectors test/test_resnode.cpp:104-134
  *   so_conv2d_bwd_filter           adjoint identity <conv(x,w),dy> = <w,bwd_filter(x,dy)>, torch-CPU
+ *   so_conv2d_* with dilation > 1  torch-CPU double conv2d and its autograd, dilation 2 and 3, with stride and groups
  *   so_bias_bwd                    closed form (plain sum)
  *   so_fc_*                        reference vectors test/test_ops.cpp:286-386 (fwd); adjoint (bwd)
  *   so_bn_infer                    reference vectors test/test_ops.cpp:438-470
@@ -24,7 +25,9 @@
  *   so_maxpool_*, so_avgpool_*     reference vectors test_ops.cpp:218-283 (fwd); brute force + sum
  *                                  conservation (bwd); max-pool tie break = first index, parity unpinned
  *   so_catclassifier_*             in-tree kernel src/cuda/cuda_kernels.cu:11-64 is the spec; closed forms
- *   so_adam_*                      in-tree kernel src/cuda/cuda_kernels.cu:159-230 is the spec; t=1 closed form
+ *   so_adam_*                      in-tree kernel src/cuda/cuda_kernels.cu:159-230 is the spec; t=1 closed form;
+ *                                  t > 1, weight decay and the fp16 skip / flag rules against a numpy restatement
+ *                                  of the kernel over several steps (tests/test_oracle_net.py)
  *   so_softmax                     closed form, rows sum to one
  *   so_loss_bwd, so_tensor_stats   in-tree kernels src/cuda/cuda_kernels.cu:252-473 are the spec (incl. the zeros their
  *                                  block reduction feeds into min / max); hand-computed case + numpy closed forms

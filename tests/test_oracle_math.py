@@ -16,37 +16,44 @@ def rnd(*shape):
 
 
 CONV_CASES = [
-    # N, C, H, W, K, R, pad, stride, group
+    # N, C, H, W, K, R, pad, stride, group[, dilation]
     (2, 8, 9, 9, 6, 3, 1, 1, 1),
     (2, 6, 11, 10, 4, 3, 1, 2, 1),
     (1, 3, 15, 15, 5, 7, 3, 2, 1),
     (2, 8, 8, 8, 8, 1, 0, 2, 1),
     (2, 8, 7, 7, 4, 3, 0, 1, 2),
     (1, 4, 6, 6, 4, 5, 2, 1, 1),
+    # dilated filters (shape rule src/node.cpp:50, 66-75): the GPU operator tests take the oracle's word for these
+    (2, 5, 11, 12, 4, 3, 2, 1, 1, 2),
+    (2, 4, 13, 13, 6, 3, 3, 2, 1, 3),
+    (1, 6, 12, 10, 4, 3, 1, 1, 2, 2),
+    (2, 3, 14, 14, 4, 5, 4, 2, 1, 2),
 ]
 
 
 @pytest.mark.parametrize("case", CONV_CASES)
 def test_conv_against_torch_and_adjoint(case):
-    N, C, H, W, K, R, pad, stride, group = case
+    N, C, H, W, K, R, pad, stride, group = case[:9]
+    dil = case[9] if len(case) > 9 else 1
     x, w = rnd(N, C, H, W), rnd(K, C // group, R, R)
-    y = ref.conv2d_fwd(x, w, pad, stride, 1, group)
-    yt = F.conv2d(torch.from_numpy(x).double(), torch.from_numpy(w).double(), None, stride, pad, 1, group)
+    y = ref.conv2d_fwd(x, w, pad, stride, dil, group)
+    yt = F.conv2d(torch.from_numpy(x).double(), torch.from_numpy(w).double(), None, stride, pad, dil, group)
+    assert y.shape == tuple(yt.shape)
     np.testing.assert_allclose(y, yt.numpy(), rtol=1e-5, atol=1e-5)
     dy = rnd(*y.shape)
-    dx = ref.conv2d_bwd_data(dy, w, x.shape, pad, stride, 1, group)
-    dw = ref.conv2d_bwd_filter(x, dy, w.shape, pad, stride, 1, group)
+    dx = ref.conv2d_bwd_data(dy, w, x.shape, pad, stride, dil, group)
+    dw = ref.conv2d_bwd_filter(x, dy, w.shape, pad, stride, dil, group)
     # <conv(x,w),dy> = <x,bwd_data(dy,w)> = <w,bwd_filter(x,dy)>
     lhs = float((y.astype(np.float64) * dy).sum())
     assert abs(lhs - float((x.astype(np.float64) * dx).sum())) <= 1e-4 * max(1, abs(lhs))
     assert abs(lhs - float((w.astype(np.float64) * dw).sum())) <= 1e-4 * max(1, abs(lhs))
     xt = torch.from_numpy(x).double().requires_grad_()
     wt = torch.from_numpy(w).double().requires_grad_()
-    F.conv2d(xt, wt, None, stride, pad, 1, group).backward(torch.from_numpy(dy).double())
+    F.conv2d(xt, wt, None, stride, pad, dil, group).backward(torch.from_numpy(dy).double())
     np.testing.assert_allclose(dx, xt.grad.numpy(), rtol=1e-5, atol=1e-5)
     np.testing.assert_allclose(dw, wt.grad.numpy(), rtol=1e-5, atol=1e-5)
     # beta = 1 accumulates
-    y2 = ref.conv2d_fwd(x, w, pad, stride, 1, group, y=y, beta=1.0)
+    y2 = ref.conv2d_fwd(x, w, pad, stride, dil, group, y=y, beta=1.0)
     np.testing.assert_allclose(y2, 2 * y, rtol=1e-6, atol=1e-6)
 
 
