@@ -658,6 +658,11 @@ void HipProgram::checkAnomaly(HipOperation &op, const HipOpArgs &tensors, const 
         if(bad) {
             fprintf(stderr, "\n\n *** Anomaly in tensor %s (%s)\n", t.second->info().c_str(), what);
             op.dump(stderr, true);
+            // the reference aborts (src/cuda/cuda_program.cpp:163-211); a host that wants to survive the report
+            // (a test, a service) asks for an exception instead
+            if(getenv("SAGA_HIP_ANOMALY_THROW"))
+                throw std::runtime_error(fmt("Anomaly in tensor %s (%s of %s)", t.second->info().c_str(), what,
+                                             op.name().c_str()));
             abort();
         }
     }

@@ -83,6 +83,104 @@ def test_conv_full_batch_properties(shape):
         assert_close(host(dx[:1]), 2 * dx_ref[:1], HALF, "dx beta=1")
 
 
+@pytest.mark.parametrize("shape", FULL_CONVS)
+def test_conv_bwd_filter_full_batch_elementwise(shape):
+    """Backward filter at the real launch geometry (the reduction over 256 images split over hundreds of blocks,
+    then the fixed-order second pass), compared element by element with the oracle.
+    1. dy is non-zero in two images only, so dw must equal the oracle's dw of those two images; three pairs that
+       fall into different parts of the split.  Every element of dw is checked, and blocks that see only zeros
+       must contribute nothing.
+    2. dy dense: dw[k0:k1, c0:c1] depends only on x[:, c0:c1] and dy[:, k0:k1], which the oracle handles over all
+       256 images; first, last and a middle block of channels."""
+    Cc, H, Kk, R, stride, pad = shape
+    g = torch.Generator(device="cuda").manual_seed(3 * Cc + Kk)
+    x = nhwc(torch.randn(N256, Cc, H, H, dtype=HALF, device="cuda", generator=g))
+    P = 1 + (H + 2 * pad - R) // stride
+    dy = nhwc(torch.randn(N256, Kk, P, P, dtype=HALF, device="cuda", generator=g))
+    dw = nhwc(torch.zeros(Kk, Cc, R, R, dtype=HALF, device="cuda"))
+    worst = 0.0
+    for pair in ((0, 255), (37, 128), (101, 202)):
+        sparse = torch.zeros_like(dy)
+        for n in pair:
+            sparse[n] = dy[n]
+        dw.fill_(7.0)  # beta = 0 must overwrite
+        K.conv2d(K.CONV_BWD_FILTER, x, sparse, dw, pad, stride)
+        idx = list(pair)
+        want = ref.conv2d_bwd_filter(host(x[idx]), host(dy[idx]), (Kk, Cc, R, R), pad, stride)
+        worst = max(worst, assert_close(host(dw), want, HALF, f"dw, dy non-zero in images {pair}", tol=2e-3))
+    K.conv2d(K.CONV_BWD_FILTER, x, dy, dw, pad, stride)
+    cb, kb = min(8, Cc), 8
+    for c0, k0 in ((0, 0), (Cc - cb, Kk - kb), ((Cc // 2 // cb) * cb, (Kk // 2 // kb) * kb + 3 if Kk > 16 else 0)):
+        k0 = min(k0, Kk - kb)
+        want = ref.conv2d_bwd_filter(host(x[:, c0:c0 + cb]), host(dy[:, k0:k0 + kb]), (kb, cb, R, R), pad, stride)
+        worst = max(worst, assert_close(host(dw[k0:k0 + kb, c0:c0 + cb]), want, HALF,
+                                        f"dw[{k0}:{k0 + kb}, {c0}:{c0 + cb}] over all images", tol=2e-3))
+    print(f"bwd-filter {shape}: worst element error {worst:.2e} of the largest element")
+
+
+def test_conv_fp32_nchw_full_batch():
+    """The fp32 NCHW half of the convolution microbenchmark at its real size (N=256, 64 -> 64, 56x56, 3x3):
+    the adjoint identity across the three passes, the first two images of forward and backward data against
+    the oracle, and backward filter element-wise with dy non-zero in two images."""
+    Cc, H, Kk, R, stride, pad = 64, 56, 64, 3, 1, 1
+    F32 = torch.float32
+    g = torch.Generator(device="cuda").manual_seed(77)
+    x = torch.randn(N256, Cc, H, H, dtype=F32, device="cuda", generator=g)
+    w = torch.randn(Kk, Cc, R, R, dtype=F32, device="cuda", generator=g) * (2.0 / (Cc * R * R)) ** 0.5
+    y = torch.zeros(N256, Kk, H, H, dtype=F32, device="cuda")
+    K.conv2d(K.CONV_FWD, x, w, y, pad, stride)
+    assert_close(host(y[:2]), ref.conv2d_fwd(host(x[:2]), host(w), pad, stride), F32, "y[:2]")
+    assert_close(host(y[-1:]), ref.conv2d_fwd(host(x[-1:]), host(w), pad, stride), F32, "y[-1]")
+    dy = torch.randn(N256, Kk, H, H, dtype=F32, device="cuda", generator=g)
+    dx, dw = torch.zeros_like(x), torch.zeros_like(w)
+    K.conv2d(K.CONV_BWD_DATA, dy, w, dx, pad, stride)
+    K.conv2d(K.CONV_BWD_FILTER, x, dy, dw, pad, stride)
+    lhs = dot(y, dy)
+    assert abs(dot(x, dx) - lhs) <= 1e-5 * abs(lhs)
+    assert abs(dot(w, dw) - lhs) <= 1e-5 * abs(lhs)
+    assert_close(host(dx[:2]), ref.conv2d_bwd_data(host(dy[:2]), host(w), (2, Cc, H, H), pad, stride), F32, "dx[:2]")
+    for pair in ((0, 255), (90, 171)):
+        sparse = torch.zeros_like(dy)
+        for n in pair:
+            sparse[n] = dy[n]
+        dw.fill_(7.0)
+        K.conv2d(K.CONV_BWD_FILTER, x, sparse, dw, pad, stride)
+        idx = list(pair)
+        want = ref.conv2d_bwd_filter(host(x[idx]), host(dy[idx]), (Kk, Cc, R, R), pad, stride)
+        assert_close(host(dw), want, F32, f"dw, dy non-zero in images {pair}")
+
+
+# the up-convolutions of the U-Net configuration at their real channel widths and sizes, one image:
+# Cin, H, Cout (2x2, stride 2)
+UNET_UPCONVS = [(1024, 16, 512), (512, 32, 256), (256, 64, 128), (128, 128, 64)]
+
+
+@pytest.mark.parametrize("shape", UNET_UPCONVS)
+def test_transposed_conv_real_widths(shape):
+    """Transposed convolution (src/cuda/cuda_dnn.cpp:542-574): forward = backward data with x in the dy role,
+    dW = backward filter with (dy, x) exchanged, dX = forward convolution of dy - each against the oracle."""
+    Cin, H, Cout = shape
+    rng = np.random.default_rng(Cin)
+    from tests.gpu_util import dev, rnd
+    x = rnd(rng, 1, Cin, H, H, dtype=HALF)
+    w = rnd(rng, Cin, Cout, 2, 2, dtype=HALF, scale=(2.0 / (Cout * 4)) ** 0.5)  # [Cx, Cy, R, S], src/node.cpp:99-110
+    Ho = ref.tconv_out(H, 2, 0, 2)
+    y_ref = ref.conv2d_bwd_data(x, w, (1, Cout, Ho, Ho), 0, 2)
+    xd, wd = dev(x, HALF, "nhwc"), dev(w, HALF, "nhwc")
+    yd = dev(np.zeros_like(y_ref), HALF, "nhwc")
+    K.conv2d(K.CONV_BWD_DATA, xd, wd, yd, 0, 2)
+    e1 = assert_close(host(yd), y_ref, HALF, "transposed conv y")
+    dy = rnd(rng, 1, Cout, Ho, Ho, dtype=HALF)
+    dyd = dev(dy, HALF, "nhwc")
+    dwd = dev(np.zeros_like(w), HALF, "nhwc")
+    K.conv2d(K.CONV_BWD_FILTER, dyd, xd, dwd, 0, 2)
+    e2 = assert_close(host(dwd), ref.conv2d_bwd_filter(dy, x, w.shape, 0, 2), HALF, "transposed conv dw")
+    dxd = dev(np.zeros_like(x), HALF, "nhwc")
+    K.conv2d(K.CONV_FWD, dyd, wd, dxd, 0, 2)
+    e3 = assert_close(host(dxd), ref.conv2d_fwd(dy, w, 0, 2), HALF, "transposed conv dx")
+    print(f"transposed conv {shape}: y {e1:.1e}, dw {e2:.1e}, dx {e3:.1e}")
+
+
 def test_batchnorm_full_size_invariants():
     Cc, H = 64, 112  # the largest batch-norm input of ResNet-50: 411 MB
     g = torch.Generator(device="cuda").manual_seed(7)

@@ -2,6 +2,9 @@
 batch / image size where the CPU oracle would take minutes) run on the hip engine and on the
 CPU oracle from identical seeded inputs and weights.  fp32 within 1e-4, fp16 within 2e-2 of the
 per-tensor max-abs value; predicted labels bit-exact."""
+import json
+import os
+
 import numpy as np
 import pytest
 
@@ -11,6 +14,23 @@ from saga_amd import networks as N
 from tests.gpu_util import rel_err
 
 pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+REPORT = os.path.join(ROOT, "gpurun_out", "network_parity.json")
+
+
+def record(test, rows):
+    """Keeps the achieved error of every checked tensor next to the bound it was held to
+    (gpurun_out/network_parity.json: {test: {tensor: [error, bound]}}), so that a reader can see how far inside
+    its bound each comparison sits."""
+    try:
+        os.makedirs(os.path.dirname(REPORT), exist_ok=True)
+        data = json.load(open(REPORT)) if os.path.exists(REPORT) else {}
+        data[test] = rows
+        with open(REPORT, "w") as f:
+            json.dump(data, f, indent=1, sort_keys=True)
+    except OSError:
+        pass
 
 
 def inputs(net, seed, uniform=False):
@@ -92,10 +112,12 @@ def run_training(net, seed, steps, lr, check_params, uniform=False, loss_scale=N
     o = OracleNet(net, lr=lr, loss_scale=loss_scale)
     tol = tol_of(net)
     bad = []
+    rows = {}
 
     def chk(name, got, want, bound):
         e = rel_err(got, want)
         print(f"  {name}: rel max-abs err {e:.3e} (bound {bound:.1e}, max |ref| {np.abs(want).max():.3e})")
+        rows[name if name not in rows else f"{name} (step {step})"] = [float(f"{e:.3e}"), float(f"{bound:.3e}")]
         if not e <= bound:
             bad.append(f"{name}: {e:.3e} > {bound:.1e}")
 
@@ -120,6 +142,7 @@ def run_training(net, seed, steps, lr, check_params, uniform=False, loss_scale=N
         # element whose tiny fp16 gradient flips sign lands 2*lr away: allow that on top of the bound
         slack = 2.5 * lr / max(float(np.abs(want).max()), 1e-30) if half else 0.0
         chk("weights " + k, got, want, (tol if half else 1e-5) + slack)
+    record(os.environ.get("PYTEST_CURRENT_TEST", net.name).split("::")[-1].split(" ")[0], rows)
     assert not bad, "; ".join(bad)
 
 
@@ -143,6 +166,64 @@ def test_resnet20_training_fp16(fusing):
 def test_resnet20_training_fp32():
     run_training(N.resnet20(8, dtype=S.FLOAT), 4, steps=2, lr=1e-3,
                  check_params=["s1-conv-w", "s3_0-conv-p-w", "fc-w", "s2_0-bn-1-s"])
+
+
+def test_resnet20_fp32_hundred_steps_weight_error_curve():
+    """Config 3 in fp32 (batch 8) for 100 Adam steps on a new batch every step, engine and oracle side by side:
+    the weight error after every tenth step.  Both sides compute from identical inputs; what separates them is
+    summation order (1e-7 per operator).  Training amplifies that: a relu input that rounds to the other side of
+    zero changes the gradients behind it, and Adam's normalised step turns any difference on a near-zero gradient
+    into a step of up to 2 lr.  How much is inherent is measured in the same test: a second ORACLE run whose
+    initial weights are perturbed by 1e-6 relative (fp32 rounding level) diverges from the first at the same
+    rate.  The engine must stay within 3x of that yardstick; the curves are recorded."""
+    net = N.resnet20(8, dtype=S.FLOAT)
+    lr = 1e-3
+    rng = np.random.default_rng(41)
+    x0, labels0 = inputs(net, 41)
+    ctx = S.Context()
+    g, t = N.build_graph(net, x0)
+    p = ctx.create_program(g, net.batch, training=True, learning_rate=lr)
+    xin, lab = ctx.resolve(t[net.input]), ctx.resolve(t["labels"])
+    names = ["s1-conv-w", "s2_1-conv-2-w", "s3_0-conv-p-w", "s4_2-conv-2-w", "fc-w", "s2_0-bn-1-s", "s4_2-bn-2-b"]
+    dev = {k: ctx.resolve(t[k]) for k in names}
+    o = OracleNet(net, lr=lr)
+    twin = N.resnet20(8, dtype=S.FLOAT)
+    prng = np.random.default_rng(0)
+    for k in twin.params:
+        if k.endswith("-w"):
+            twin.params[k] = (twin.params[k] * (1 + 1e-6 * prng.standard_normal(twin.params[k].shape))).astype(np.float32)
+    o2 = OracleNet(twin, lr=lr)
+
+    def errors(get):
+        d = {k: np.abs(get(k).astype(np.float64).reshape(o.p[k].shape) - o.p[k]) / np.abs(o.p[k]).max() for k in names}
+        return max(float(v.max()) for v in d.values()), float(np.median([np.median(v) for v in d.values()]))
+
+    rows, curve = {}, []
+    for step in range(1, 101):
+        x = rng.standard_normal(x0.shape).astype(np.float32)
+        labels = rng.integers(0, net.classes, (net.batch, 1)).astype(np.int32)
+        xin.write(x)
+        lab.write(labels)
+        p.run(1)
+        o.train_step(x, labels)
+        o2.train_step(x, labels)
+        if step == 1:
+            frac = float(np.mean(np.concatenate([
+                (np.abs(dev[k].read().astype(np.float64).reshape(o.p[k].shape) - o.p[k]) / np.abs(o.p[k]).max()).ravel()
+                for k in names]) <= 1e-5))
+            print(f"  step 1: {100 * frac:.2f}% of the checked weights within 1e-5")
+            assert frac >= 0.99
+        if step % 10 == 0:
+            (w, m), (yw, ym) = errors(lambda k: dev[k].read()), errors(lambda k: o2.p[k])
+            curve.append((step, w, m, yw, ym))
+            rows[f"step {step}: engine worst / median element"] = [float(f"{w:.3e}"), float(f"{m:.3e}")]
+            rows[f"step {step}: perturbed oracle worst / median element"] = [float(f"{yw:.3e}"), float(f"{ym:.3e}")]
+            print(f"  step {step}: engine vs oracle worst {w:.3e} median {m:.3e} | oracle perturbed by 1e-6 vs oracle "
+                  f"worst {yw:.3e} median {ym:.3e}")
+    record("test_resnet20_fp32_hundred_steps_weight_error_curve", rows)
+    for step, w, m, yw, ym in curve:
+        if step >= 30:
+            assert w <= 3 * yw and m <= 3 * ym, (step, w, m, yw, ym)
 
 
 def test_resnet50_inference_fp16():

@@ -1,11 +1,13 @@
 """The reference's own command-line harnesses (test/test_ops.cpp `ops`, `concat`;
-test/test_resnode.cpp `resnode`), compiled unmodified from the reference sources against this
+test/test_resnode.cpp `resnode`; test/test_mp.cpp `mp`; test/test_fc.cpp `fc`; test/test_conv.cpp `conv`;
+test/test_classifier.cpp `mnist`), compiled unmodified from the reference sources against this
 repository's hip engine (oracle/Makefile.ref -> oracle/_ref/saga_refhost), judge the backend
 with their own criterion (SSE <= 1e-4).  Skipped where the binary was not built (it needs the
 reference tree at build time; the prebuilt binary travels to the GPU box)."""
 import os
 import subprocess
 
+import numpy as np
 import pytest
 
 pytestmark = pytest.mark.gpu
@@ -49,6 +51,50 @@ def test_reference_concat():
     r = run("concat")
     assert r.returncode == 0
     assert "18.0" in r.stdout or "18" in r.stdout
+
+
+def test_reference_mixed_precision_overflow():
+    """`saga mp` (test/test_mp.cpp): fp16 fc + L2 loss against a target of 2e4 - the weight 0.1 moves to 0.11 by
+    Adam's first step; with a target beyond the fp16 range (-t 70000) the gradient is -inf, the optimizer skips
+    the element and the weight stays 0.1.  The harness prints, it asserts nothing itself."""
+    r = run("mp")
+    assert r.returncode == 0
+    assert "-2e+04" in r.stdout and "-2e+03" in r.stdout and "0.11" in r.stdout
+    r = run("mp", "-t", "40000")   # exponent 30: the range flag's territory, still finite
+    assert r.returncode == 0 and "-4e+04" in r.stdout and "0.11" in r.stdout
+    r = run("mp", "-t", "70000")
+    assert r.returncode == 0
+    lines = r.stdout.splitlines()
+    assert any(l.startswith("dy:") and "-inf" in l for l in lines)
+    w = [l for l in lines if l.startswith(" w: [")]
+    assert w and w[0].split()[-1] == "0.1", w
+
+
+@pytest.mark.parametrize("half", [False, True])
+def test_reference_fc_harness(half):
+    """`saga fc` (test/test_fc.cpp): one training step of a lone fc node, prints the program and its tensors."""
+    r = run("fc", *(["-h"] if half else []))
+    assert r.returncode == 0
+    assert ("adam-mixed" if half else "adam-f32") in r.stdout and "RESULT:" in r.stdout and "nan" not in r.stdout
+
+
+@pytest.mark.parametrize("half", [False, True])
+def test_reference_conv_training_loop(half):
+    """`saga conv` (test/test_conv.cpp): strided conv + bias -> relu -> fc -> relu -> reshape -> transposed conv
+    + bias -> L2 loss, trained in an endless loop that prints every 1000 steps; the test lets it run a few
+    seconds.  The target is the input pattern; the mean squared error it prints (last column of MMSS) must fall
+    well below the 0.2 of an untrained net and stay finite."""
+    if not os.path.exists(BIN):
+        pytest.skip("oracle/_ref/saga_refhost not built (make -C oracle -f Makefile.ref)")
+    r = subprocess.run(["timeout", "-s", "INT", "6", BIN, "conv", *(["-h"] if half else [])], capture_output=True,
+                       text=True, timeout=60)
+    rows = [l.split() for l in r.stdout.splitlines() if l.startswith("MMSS: [")]
+    assert len(rows) >= 4, r.stdout[-2000:]
+    rows = rows[:len(rows) // 2 * 2]  # the last block may have been cut by the signal
+    ms = [float(row[-1]) for row in rows]
+    print("mean squared error per print:", ms[:2], "...", ms[-2:])
+    assert all(np.isfinite(v) for v in ms)
+    assert max(ms[-2:]) <= 0.08 and sum(ms[-2:]) <= sum(ms[:2])
 
 
 def write_idx_dataset(path, n_train=6400, n_test=1280, seed=0):
