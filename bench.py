@@ -7,10 +7,11 @@ Saga Graph/Context/Program boundary on the hip engine.
 
 Prints ONE JSON line.  `value` is training images/sec over exactly K timed steps with the
 input batch already resident in HBM; `infer_images_per_sec` is the inference program on the
-same weights.  `roofline` describes the operation kind that takes the most GPU time in the
-training step (HIP-event timing of every operation on the engine's stream, taken in a second
-pass of K steps so that the events do not sit inside the timed region); `kernels` lists every
-operation kind the same way.  `cpu_baseline` is the CPU oracle (oracle/) running the same
+same weights.  `roofline` describes the kernel family that takes the most GPU time in the
+training step (the convolutions; HIP-event timing of every operation on the engine's stream, taken in a
+second pass of K steps so that the events do not sit inside the timed region), `roofline_hbm` the
+HBM-bound family with the most time (batch norm); `families` and `kernels` list every family and
+every operation kind the same way.  `cpu_baseline` is the CPU oracle (oracle/) running the same
 training step on a small batch on the host cores - a reported baseline, not a target.
 """
 import argparse
@@ -30,18 +31,25 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 MATRIX_KINDS = ("convfwd", "convbwddata", "convbwdfilter", "fc.")
 CONV_KINDS = ("convfwd", "convbwddata", "convbwdfilter")
 
-# HBM bytes per launch of each operation kind, averaged over the launches of one training step:
-# rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE over this benchmark, summed over the kernels an
-# operation launches, each counter scaled by what it reads for a plain copy of known size
-# (FETCH_SIZE reads 0.5 of the bytes a 1 GiB copy fetches, WRITE_SIZE 1.0).  The command lines and
-# the per-kernel table are in profiles/resnet50_b256_fp16_hbm_counters.txt.
-MEASURED_HBM_BYTES_PER_LAUNCH = {
-    # the counters cannot tell fused from plain batch-norm launches (same kernels): both kinds carry
-    # the average over all 53 batch-norm launches of a step
-    "bnbwd.fused": 635799930, "bnbwd": 635799930,
-    "bntrain.fused": 285296483, "bntrain": 285296483,
-    "convfwd": 264287030, "convbwddata": 283369189, "convbwdfilter": 309133801,
+# Operation kinds that share kernels and a roofline bound form a family; `roofline` describes the family with
+# the most GPU time in the training step.
+FAMILIES = {
+    "conv": ("convfwd", "convbwddata", "convbwdfilter"),
+    "batchnorm": ("bntrain", "bntrain.fused", "bnbwd", "bnbwd.fused"),
+    "pool": ("poolfwd", "poolbwd"),
 }
+
+# HBM bytes per launch of a family, averaged over ALL launches of that family in one training step (the same
+# population `algorithmic` is averaged over): rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE over
+# `bench.py --train-only --no-cpu --no-profile`, summed over the kernels the family's operations launch, each
+# counter scaled by what it reads for a plain copy of known size (`bench.py --copy-calibration`).  The command
+# lines, the per-kernel table and the commit the counters were taken at are in
+# profiles/resnet50_b256_fp16_hbm_counters.txt; they go stale when kernels change, hence the label.
+MEASURED_HBM_BYTES_PER_LAUNCH = {
+    "conv": None,
+    "batchnorm": None,
+}
+TRAFFIC_SOURCE = None
 
 
 def by_kind(rows):
@@ -107,6 +115,42 @@ def profile_rows(rows):
                        frac=round(a / PEAK_HBM_GBS, 4))
         out.append(row)
     out.sort(key=lambda r: -r["ms_total"])
+    return out
+
+
+def family_rows(rows, steps):
+    """Operation kinds grouped into families (FAMILIES; every other kind is its own family), most GPU time first.
+    achieved = algorithmic flops (matrix families) or bytes (the others) of all launches / their summed time,
+    both from this run; `algorithmic` and `traffic` are per launch, averaged over the same launches."""
+    fam_of = {k: f for f, kinds in FAMILIES.items() for k in kinds}
+    agg = {}
+    for r in rows:
+        if r["ms"] <= 0:
+            continue
+        f = fam_of.get(r["kind"], r["kind"])
+        a = agg.setdefault(f, {"kernel": f, "kinds": [], "launches": 0, "ms": 0.0, "flops": 0.0, "bytes": 0.0, "roof_ms": 0.0})
+        a["kinds"].append(r["kind"])
+        for k in ("launches", "ms", "flops", "bytes", "roof_ms"):
+            a[k] += r[k]
+    out = []
+    for a in agg.values():
+        matrix = a["kernel"] == "conv" or a["kernel"].startswith("fc.")
+        sec = a["ms"] * 1e-3
+        if matrix:
+            ach, peak, unit = a["flops"] / sec / 1e12, PEAK_FP16_TFLOPS, "TFLOP/s"
+            alg = a["flops"] / a["launches"]
+        else:
+            ach, peak, unit = a["bytes"] / sec / 1e9, PEAK_HBM_GBS, "GB/s"
+            alg = a["bytes"] / a["launches"]
+        out.append({"kernel": a["kernel"], "kinds": sorted(a["kinds"]), "bound": "mfma" if matrix else "hbm",
+                    "achieved": round(ach, 1), "peak": peak, "unit": unit, "frac": round(ach / peak, 4),
+                    "traffic": MEASURED_HBM_BYTES_PER_LAUNCH.get(a["kernel"]), "traffic_source": TRAFFIC_SOURCE,
+                    "algorithmic": round(alg), "algorithmic_unit": "flop/launch" if matrix else "byte/launch",
+                    "algorithmic_bytes": round(a["bytes"] / a["launches"]),
+                    "avg_launch_us": round(a["ms"] * 1e3 / a["launches"], 2), "launches": a["launches"],
+                    "ms_per_step": round(a["ms"] / steps, 3),
+                    "frac_of_own_roofline": round(a["roof_ms"] / a["ms"], 4)})
+    out.sort(key=lambda r: -r["ms_per_step"])
     return out
 
 
@@ -189,6 +233,8 @@ def main():
     ap.add_argument("--cpu-batch", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-profile", action="store_true")
+    ap.add_argument("--train-only", action="store_true",
+                    help="skip the inference program (counter runs that must see training launches only)")
     ap.add_argument("--per-op", metavar="FILE",
                     help="also write one line per operation of the training step (time, rate, own roofline bound)")
     ap.add_argument("--host-input", action="store_true",
@@ -215,12 +261,13 @@ def main():
     ctx = S.Context()
     graph, t = N.build_graph(net, x)
     train = ctx.create_program(graph, args.batch, training=True, learning_rate=1e-4, initial_loss_scale=1024.0)
-    infer = ctx.create_program(graph, args.batch, training=False)
+    infer = None if args.train_only else ctx.create_program(graph, args.batch, training=False)
     ctx.resolve(t["labels"]).write(labels)
     loss = ctx.resolve(t["loss"])
     pred = ctx.resolve(t["pred"])
     train.finalize()
-    infer.finalize()
+    if infer:
+        infer.finalize()
 
     import torch  # device-wide synchronisation around the timed regions
 
@@ -234,15 +281,17 @@ def main():
     mean_loss = float(loss.read().mean())
 
     # ---- inference on the same weights
-    infer.run(args.warmup)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    infer.run(args.steps)
-    torch.cuda.synchronize()
-    t_infer = time.perf_counter() - t0
-    pred.read()
+    t_infer = float("nan")
+    if not args.train_only:
+        infer.run(args.warmup)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        infer.run(args.steps)
+        torch.cuda.synchronize()
+        t_infer = time.perf_counter() - t0
+        pred.read()
 
-    kernels, roof, conv = [], None, None
+    kernels, roof, roof_hbm, conv, families = [], None, None, None, []
     if not args.no_profile:
         train.set_profiling(True)
         train.run(args.steps)
@@ -252,12 +301,11 @@ def main():
         rows = by_kind(raw)
         kernels = profile_rows(rows)
         train.set_profiling(False)
-        if kernels:
-            d = kernels[0]
-            roof = {"kernel": d["kind"], "bound": d["bound"], "achieved": d["achieved"], "peak": d["peak"],
-                    "unit": d["unit"], "frac": d["frac"],
-                    "traffic": MEASURED_HBM_BYTES_PER_LAUNCH.get(d["kind"]),
-                    "avg_launch_us": d["avg_us"], "launches": d["launches"]}
+        families = family_rows(rows, args.steps)
+        if families:
+            roof = families[0]
+            hbm = [f for f in families if f["bound"] == "hbm"]
+            roof_hbm = hbm[0] if hbm else None
         # the three convolution kinds together: the "conv MFMA util %" half of the metric
         cr = [r for r in rows if r["kind"] in CONV_KINDS and r["ms"] > 0]
         if cr:
@@ -286,14 +334,16 @@ def main():
         "config": {"workload": f"ResNet-50 v1.5 training step (fwd+bwd+Adam), fp16 NHWC, batch {args.batch}, "
                                f"{args.image}x{args.image}, 1000 classes", "global_batch": args.batch},
         "train_images_per_sec": round(ips, 1),
-        "infer_images_per_sec": round(args.batch * args.steps / t_infer, 1),
-        "infer_ms_per_batch": round(t_infer / args.steps * 1e3, 3),
+        "infer_images_per_sec": None if args.train_only else round(args.batch * args.steps / t_infer, 1),
+        "infer_ms_per_batch": None if args.train_only else round(t_infer / args.steps * 1e3, 3),
         "train_tflops": round(flops_step / (t_train / args.steps) / 1e12, 1),
-        "infer_tflops": round(net.flops_fwd * args.batch / (t_infer / args.steps) / 1e12, 1),
+        "infer_tflops": None if args.train_only else round(net.flops_fwd * args.batch / (t_infer / args.steps) / 1e12, 1),
         "loss_scale": train.loss_scale(),
         "mean_loss": round(mean_loss, 4),
         "roofline": roof,
+        "roofline_hbm": roof_hbm,
         "conv": conv,
+        "families": families,
         "kernels": kernels,
     }
     if not args.no_cpu:

@@ -6,7 +6,13 @@
 
 namespace {
 
-static int conv_dim(int in, int k, int pad, int stride, int dil) { return 1 + (in + 2 * pad - ((k - 1) * dil + 1)) / stride; }
+// 0 when the padded input is smaller than the dilated filter (C's division would truncate a negative
+// numerator toward zero and report one output position)
+static int conv_dim(int in, int k, int pad, int stride, int dil)
+{
+    const int span = in + 2 * pad - ((k - 1) * dil + 1);
+    return span < 0 ? 0 : 1 + span / stride;
+}
 
 // x: (N,C,H,W)  w: (K,C/group,R,S)  y: (N,K,P,Q)
 static int geometry(const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y, const SagaConvParams *p,

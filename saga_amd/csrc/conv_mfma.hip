@@ -329,6 +329,185 @@ __device__ __forceinline__ void halve_exchange(float (&a)[NV], float (&b)[NV], i
     }
 }
 
+// Everything the gather kernels do after their main loop: alpha / beta, the optional batch-norm
+// inference fold (+ residual + relu), the 16-byte channel-vector stores and the optional per-channel
+// statistics of the stored values.  acc[i][j][v] belongs to row wm + 32*i + lane%32 of the block tile
+// and channel n0 + wn + 32*j + 8*(v/4) + 4*(lane/32) + v%4; rowpix(i, ok, pix) names the output pixel of
+// this lane's row in M-subtile i (ok false: nothing is stored).  MASK: rows that are not ok may hold
+// non-zero accumulators and have to be kept out of the statistics.  smem: the block's LDS, free for
+// reuse once every wavefront has left the main loop (the barriers inside see to that).
+template <int TM, int TN, int WGM, int WGN, int BN, bool BWD, bool MASK, typename RowPix>
+__device__ __forceinline__ void gather_epilogue(const GatherArgs &g, float16_t (&acc)[TM][TN], char *smem, int tid, int lane,
+                                                int wave, int wm, int wn, int n0, int stats_row, RowPix rowpix)
+{
+    // Inference with a folded batch norm: scale = s/sqrt(v+eps) and shift = b - m*scale of the
+    // block's BN channels go into LDS once (the stage memory is free after the last slice).
+    float *bnp = (float *)smem;
+    if constexpr(!BWD) {
+        if(g.bn_s) {
+            __syncthreads(); // every wavefront is done reading the last slice
+            if(tid < BN) {
+                const int n = n0 + tid;
+                float sc = 0.0f, sh = 0.0f;
+                if(n < g.Ngemm) {
+                    sc = g.bn_s[n] * rsqrtf(g.bn_v[n] + g.bn_eps);
+                    sh = g.bn_b[n] - g.bn_m[n] * sc;
+                }
+                bnp[tid] = sc;
+                bnp[BN + tid] = sh;
+            }
+            __syncthreads();
+        }
+    }
+    // acc[i][j][v]: pixel wm + 32*i + lane%32, channel wn + 32*j + 8*(v/4) + 4*(lane/32) + v%4
+    const int hi = lane >> 5;
+    bool okr[TM];
+    const bool vec_ok = (g.ldo & 7) == 0 && (g.Ngemm & 7) == 0 && ((uintptr_t)g.out & 15) == 0;
+#pragma unroll
+    for(int i = 0; i < TM; i++) {
+        bool ok;
+        int64_t pix;
+        rowpix(i, ok, pix);
+        okr[i] = ok;
+        half_t *orow = g.out + pix * g.ldo;
+#pragma unroll
+        for(int j = 0; j < TN; j++) {
+            const int nb = n0 + wn + j * 32;
+            if(vec_ok) {
+                float f[16];
+#pragma unroll
+                for(int v = 0; v < 16; v++)
+                    f[v] = g.alpha * acc[i][j][v];
+                typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+                if(g.beta != 0.0f) {
+                    float old[16];
+                    load_row32(orow, ok, nb, g.Ngemm, hi, old);
+#pragma unroll
+                    for(int v = 0; v < 16; v++)
+                        f[v] += g.beta * old[v];
+                }
+                if constexpr(!BWD) {
+                    if(g.bn_s) {
+                        float zz[16];
+                        if(g.bn_flags & SAGA_BN_ADD)
+                            load_row32(g.z + pix * g.ldz, ok, nb, g.Ngemm, hi, zz);
+#pragma unroll
+                        for(int q = 0; q < 4; q++) {
+                            // scale and shift of the block's channels were put into LDS after the main loop
+                            const int cl = wn + j * 32 + 8 * q + 4 * hi;
+                            const float4_t sc = *(const float4_t *)(bnp + cl), sh = *(const float4_t *)(bnp + BN + cl);
+#pragma unroll
+                            for(int e = 0; e < 4; e++) {
+                                float t = __builtin_fmaf(f[4 * q + e], sc[e], sh[e]);
+                                if(g.bn_flags & SAGA_BN_ADD)
+                                    t += zz[4 * q + e];
+                                if(g.bn_flags & SAGA_BN_RELU)
+                                    t = (t != t) ? t : fmaxf(t, 0.0f);
+                                f[4 * q + e] = t;
+                            }
+                        }
+                    }
+                }
+                // after the swaps: lower half-wave holds channels 0..7 (then 16..23) of the tile,
+                // upper half-wave 8..15 (24..31): one store covers 32 contiguous bytes per pixel
+#pragma unroll
+                for(int q = 0; q < 2; q++) {
+                    const unsigned x0 = pack2(f[8 * q + 0], f[8 * q + 1]), x1 = pack2(f[8 * q + 2], f[8 * q + 3]);
+                    const unsigned y0 = pack2(f[8 * q + 4], f[8 * q + 5]), y1 = pack2(f[8 * q + 6], f[8 * q + 7]);
+                    const auto s0_ = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+                    const auto s1_ = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+                    const int n = nb + 16 * q + 8 * hi;
+                    if(ok && n < g.Ngemm) {
+                        typedef unsigned u4 __attribute__((ext_vector_type(4)));
+                        const u4 o = {s0_[0], s1_[0], s0_[1], s1_[1]};
+                        *(u4 *)(orow + n) = o;
+                    }
+                }
+            } else if(ok) {
+#pragma unroll
+                for(int v = 0; v < 16; v++) {
+                    const int n = nb + (v >> 2) * 8 + hi * 4 + (v & 3);
+                    if(n >= g.Ngemm)
+                        continue;
+                    float val = g.alpha * acc[i][j][v];
+                    if(g.beta != 0.0f)
+                        val += g.beta * (float)orow[n];
+                    if constexpr(!BWD) {
+                        if(g.bn_s) {
+                            const float sc = g.bn_s[n] * rsqrtf(g.bn_v[n] + g.bn_eps);
+                            val = __builtin_fmaf(val, sc, g.bn_b[n] - g.bn_m[n] * sc);
+                            if(g.bn_flags & SAGA_BN_ADD)
+                                val += (float)g.z[pix * g.ldz + n];
+                            if(g.bn_flags & SAGA_BN_RELU)
+                                val = (val != val) ? val : fmaxf(val, 0.0f);
+                        }
+                    }
+                    orow[n] = (half_t)val;
+                }
+            }
+        }
+    }
+    // Optional: per-channel sum and sum of squares of this block's outputs (as stored, i.e.
+    // rounded to fp16), for a batch normalisation that follows.  Columns past Ngemm hold zeros in
+    // the accumulators and add nothing; so do rows that are not ok unless MASK says they may hold
+    // anything, in which case they are left out here.  Lanes of one half-wave hold
+    // different pixels of the same channels: a halving exchange (each step swaps half of the
+    // values with the lane 16, 8, .. 1 away) leaves every lane with the total of one channel;
+    // the wavefronts stacked along M are then added through LDS in a fixed order.
+    if constexpr(!BWD) {
+        if(g.stats) {
+            constexpr int NV = TN * 16;
+            static_assert(NV == 16 || NV == 32, "stats layout");
+            float sv[NV], qv[NV];
+#pragma unroll
+            for(int j = 0; j < TN; j++)
+#pragma unroll
+                for(int v = 0; v < 16; v++) {
+                    float a = 0.0f, q = 0.0f;
+#pragma unroll
+                    for(int i = 0; i < TM; i++) {
+                        const float r = (!MASK || okr[i]) ? (float)(half_t)(g.alpha * acc[i][j][v]) : 0.0f;
+                        a += r;
+                        q += r * r;
+                    }
+                    sv[j * 16 + v] = a;
+                    qv[j * 16 + v] = q;
+                }
+            if constexpr(NV == 32) {
+                halve_exchange<32>(sv, qv, lane, 16);
+                halve_exchange<16>(sv, qv, lane, 8);
+                halve_exchange<8>(sv, qv, lane, 4);
+                halve_exchange<4>(sv, qv, lane, 2);
+                halve_exchange<2>(sv, qv, lane, 1);
+            } else {
+                halve_exchange<16>(sv, qv, lane, 16);
+                halve_exchange<8>(sv, qv, lane, 8);
+                halve_exchange<4>(sv, qv, lane, 4);
+                halve_exchange<2>(sv, qv, lane, 2);
+                sv[0] += __shfl_xor(sv[0], 1, 64);
+                qv[0] += __shfl_xor(qv[0], 1, 64);
+            }
+            const int idx = NV == 32 ? (lane & 31) : (lane & 31) >> 1;
+            const int chl = 32 * (idx >> 4) + 8 * ((idx & 15) >> 2) + 4 * hi + (idx & 3); // channel inside the wave tile
+            typedef float float2_t __attribute__((ext_vector_type(2)));
+            float2_t *red = (float2_t *)smem;
+            __syncthreads(); // every wavefront is done reading the last slice
+            if(NV == 32 || (lane & 1) == 0) {
+                float2_t v2 = {sv[0], qv[0]};
+                red[(wave / WGN) * BN + wn + chl] = v2;
+            }
+            __syncthreads();
+            if(tid < BN && n0 + tid < g.Ngemm) {
+                float2_t t = red[tid];
+#pragma unroll
+                for(int wy = 1; wy < WGM; wy++)
+                    t += red[wy * BN + tid];
+                *(float2_t *)(g.stats + ((int64_t)stats_row * g.Ngemm + n0 + tid) * 2) = t;
+            }
+        }
+    }
+}
+
 template <int BM, int BN, int WGM, int WGN, int STAGES, int BKT, bool BWD, int PROD = 0>
 __global__ void __launch_bounds__(64 * (WGM * WGN + PROD), PROD ? (WGM * WGN + PROD + 3) / 4 : 1) conv_gather_gemm_dma(GatherArgs g)
 {
@@ -680,33 +859,10 @@ __global__ void __launch_bounds__(64 * (WGM * WGN + PROD), PROD ? (WGM * WGN + P
         }
     }
 
-    // Inference with a folded batch norm: scale = s/sqrt(v+eps) and shift = b - m*scale of the
-    // block's BN channels go into LDS once (the stage memory is free after the last slice).
-    float *bnp = (float *)smem;
-    if constexpr(!BWD) {
-        if(g.bn_s) {
-            __syncthreads(); // every wavefront is done reading the last slice
-            if(tid < BN) {
-                const int n = n0 + tid;
-                float sc = 0.0f, sh = 0.0f;
-                if(n < g.Ngemm) {
-                    sc = g.bn_s[n] * rsqrtf(g.bn_v[n] + g.bn_eps);
-                    sh = g.bn_b[n] - g.bn_m[n] * sc;
-                }
-                bnp[tid] = sc;
-                bnp[BN + tid] = sh;
-            }
-            __syncthreads();
-        }
-    }
-    // acc[i][j][v]: pixel wm + 32*i + lane%32, channel wn + 32*j + 8*(v/4) + 4*(lane/32) + v%4
-    const int hi = lane >> 5;
-    const bool vec_ok = (g.ldo & 7) == 0 && (g.Ngemm & 7) == 0 && ((uintptr_t)g.out & 15) == 0;
-#pragma unroll
-    for(int i = 0; i < TM; i++) {
+    gather_epilogue<TM, TN, WGM, WGN, BN, BWD, false>(g, acc, smem, tid, lane, wave, wm, wn, n0, bm, [&](int i, bool &ok, int64_t &pix) {
         const int m = m0 + wm + i * 32 + (lane & 31);
-        bool ok = m < Mloc;
-        int64_t pix = m;
+        ok = m < Mloc;
+        pix = m;
         if(BWD && g.classes > 1) {
             const int mm = ok ? m : 0;
             const int ox = mm % PW;
@@ -717,142 +873,7 @@ __global__ void __launch_bounds__(64 * (WGM * WGN + PROD), PROD ? (WGM * WGN + P
             ok = ok && y < g.OH && x < g.OW;
             pix = ((int64_t)n * g.OH + y) * g.OW + x;
         }
-        half_t *orow = g.out + pix * g.ldo;
-#pragma unroll
-        for(int j = 0; j < TN; j++) {
-            const int nb = n0 + wn + j * 32;
-            if(vec_ok) {
-                float f[16];
-#pragma unroll
-                for(int v = 0; v < 16; v++)
-                    f[v] = g.alpha * acc[i][j][v];
-                typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
-                if(g.beta != 0.0f) {
-                    float old[16];
-                    load_row32(orow, ok, nb, g.Ngemm, hi, old);
-#pragma unroll
-                    for(int v = 0; v < 16; v++)
-                        f[v] += g.beta * old[v];
-                }
-                if constexpr(!BWD) {
-                    if(g.bn_s) {
-                        float zz[16];
-                        if(g.bn_flags & SAGA_BN_ADD)
-                            load_row32(g.z + pix * g.ldz, ok, nb, g.Ngemm, hi, zz);
-#pragma unroll
-                        for(int q = 0; q < 4; q++) {
-                            // scale and shift of the block's channels were put into LDS after the main loop
-                            const int cl = wn + j * 32 + 8 * q + 4 * hi;
-                            const float4_t sc = *(const float4_t *)(bnp + cl), sh = *(const float4_t *)(bnp + BN + cl);
-#pragma unroll
-                            for(int e = 0; e < 4; e++) {
-                                float t = __builtin_fmaf(f[4 * q + e], sc[e], sh[e]);
-                                if(g.bn_flags & SAGA_BN_ADD)
-                                    t += zz[4 * q + e];
-                                if(g.bn_flags & SAGA_BN_RELU)
-                                    t = (t != t) ? t : fmaxf(t, 0.0f);
-                                f[4 * q + e] = t;
-                            }
-                        }
-                    }
-                }
-                // after the swaps: lower half-wave holds channels 0..7 (then 16..23) of the tile,
-                // upper half-wave 8..15 (24..31): one store covers 32 contiguous bytes per pixel
-#pragma unroll
-                for(int q = 0; q < 2; q++) {
-                    const unsigned x0 = pack2(f[8 * q + 0], f[8 * q + 1]), x1 = pack2(f[8 * q + 2], f[8 * q + 3]);
-                    const unsigned y0 = pack2(f[8 * q + 4], f[8 * q + 5]), y1 = pack2(f[8 * q + 6], f[8 * q + 7]);
-                    const auto s0_ = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
-                    const auto s1_ = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
-                    const int n = nb + 16 * q + 8 * hi;
-                    if(ok && n < g.Ngemm) {
-                        typedef unsigned u4 __attribute__((ext_vector_type(4)));
-                        const u4 o = {s0_[0], s1_[0], s0_[1], s1_[1]};
-                        *(u4 *)(orow + n) = o;
-                    }
-                }
-            } else if(ok) {
-#pragma unroll
-                for(int v = 0; v < 16; v++) {
-                    const int n = nb + (v >> 2) * 8 + hi * 4 + (v & 3);
-                    if(n >= g.Ngemm)
-                        continue;
-                    float val = g.alpha * acc[i][j][v];
-                    if(g.beta != 0.0f)
-                        val += g.beta * (float)orow[n];
-                    if constexpr(!BWD) {
-                        if(g.bn_s) {
-                            const float sc = g.bn_s[n] * rsqrtf(g.bn_v[n] + g.bn_eps);
-                            val = __builtin_fmaf(val, sc, g.bn_b[n] - g.bn_m[n] * sc);
-                            if(g.bn_flags & SAGA_BN_ADD)
-                                val += (float)g.z[pix * g.ldz + n];
-                            if(g.bn_flags & SAGA_BN_RELU)
-                                val = (val != val) ? val : fmaxf(val, 0.0f);
-                        }
-                    }
-                    orow[n] = (half_t)val;
-                }
-            }
-        }
-    }
-    // Optional: per-channel sum and sum of squares of this block's outputs (as stored, i.e.
-    // rounded to fp16), for a batch normalisation that follows.  Rows past M and columns past
-    // Ngemm hold zeros in the accumulators and add nothing.  Lanes of one half-wave hold
-    // different pixels of the same channels: a halving exchange (each step swaps half of the
-    // values with the lane 16, 8, .. 1 away) leaves every lane with the total of one channel;
-    // the wavefronts stacked along M are then added through LDS in a fixed order.
-    if constexpr(!BWD) {
-        if(g.stats) {
-            constexpr int NV = TN * 16;
-            static_assert(NV == 16 || NV == 32, "stats layout");
-            float sv[NV], qv[NV];
-#pragma unroll
-            for(int j = 0; j < TN; j++)
-#pragma unroll
-                for(int v = 0; v < 16; v++) {
-                    float a = 0.0f, q = 0.0f;
-#pragma unroll
-                    for(int i = 0; i < TM; i++) {
-                        const float r = (float)(half_t)(g.alpha * acc[i][j][v]);
-                        a += r;
-                        q += r * r;
-                    }
-                    sv[j * 16 + v] = a;
-                    qv[j * 16 + v] = q;
-                }
-            if constexpr(NV == 32) {
-                halve_exchange<32>(sv, qv, lane, 16);
-                halve_exchange<16>(sv, qv, lane, 8);
-                halve_exchange<8>(sv, qv, lane, 4);
-                halve_exchange<4>(sv, qv, lane, 2);
-                halve_exchange<2>(sv, qv, lane, 1);
-            } else {
-                halve_exchange<16>(sv, qv, lane, 16);
-                halve_exchange<8>(sv, qv, lane, 8);
-                halve_exchange<4>(sv, qv, lane, 4);
-                halve_exchange<2>(sv, qv, lane, 2);
-                sv[0] += __shfl_xor(sv[0], 1, 64);
-                qv[0] += __shfl_xor(qv[0], 1, 64);
-            }
-            const int idx = NV == 32 ? (lane & 31) : (lane & 31) >> 1;
-            const int chl = 32 * (idx >> 4) + 8 * ((idx & 15) >> 2) + 4 * hi + (idx & 3); // channel inside the wave tile
-            typedef float float2_t __attribute__((ext_vector_type(2)));
-            float2_t *red = (float2_t *)smem;
-            __syncthreads(); // every wavefront is done reading the last slice
-            if(NV == 32 || (lane & 1) == 0) {
-                float2_t v2 = {sv[0], qv[0]};
-                red[(wave / WGN) * BN + wn + chl] = v2;
-            }
-            __syncthreads();
-            if(tid < BN && n0 + tid < g.Ngemm) {
-                float2_t t = red[tid];
-#pragma unroll
-                for(int wy = 1; wy < WGM; wy++)
-                    t += red[wy * BN + tid];
-                *(float2_t *)(g.stats + ((int64_t)bm * g.Ngemm + n0 + tid) * 2) = t;
-            }
-        }
-    }
+    });
 }
 
 // Many filters in one launch: job j owns the blocks first_block[j] .. first_block[j+1]-1, one block per

@@ -301,6 +301,7 @@ struct BiasAdd : public HipOperation {
     }
     HipOpArgs listInputs() const override { return {{"b", b_}, {"y", y_}}; }
     HipOpArgs listOutputs() const override { return {{"y", y_}}; }
+    double bytes() const override { return 2 * nbytes(y_); }
     // the output is read as well as written; report it as accumulating so that liveness sees the read
     float one_ = 1.0f;
     float *getBeta(const T &t) override { return t == y_ ? &one_ : nullptr; }
@@ -321,6 +322,7 @@ struct BiasBwd : public HipOperation {
     }
     HipOpArgs listInputs() const override { return {{"dy", dy_}}; }
     HipOpArgs listOutputs() const override { return {{"db", db_}}; }
+    double bytes() const override { return nbytes(dy_); }
     float *getBeta(const T &t) override { return t == db_ ? &beta_ : nullptr; }
 };
 
@@ -719,6 +721,7 @@ struct CatClassifierFwd : public HipOperation {
     }
     HipOpArgs listInputs() const override { return {{"x", x_}}; }
     HipOpArgs listOutputs() const override { return {{"y", y_}}; }
+    double bytes() const override { return nbytes(x_); }
 };
 
 struct CatClassifierBwd : public HipOperation {
@@ -739,6 +742,7 @@ struct CatClassifierBwd : public HipOperation {
                                            (const int32_t *)dy_->deviceMem(),
                                            loss_ ? (float *)loss_->deviceMem() : nullptr, scale, S(p)));
     }
+    double bytes() const override { return nbytes(x_) + nbytes(dx_); }
     // the loss scale is a launch argument and changes every step
     bool graphSafe() const override { return x_->m_data_type != Tensor::DataType::HALF; }
     HipOpArgs listInputs() const override { return {{"x", x_}, {"y", y_}, {"dy", dy_}}; }

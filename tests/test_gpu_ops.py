@@ -112,7 +112,9 @@ def test_conv_nonsquare_filter(R, S, layout, dtype):
 
 
 @pytest.mark.parametrize("case", [(2, 64, 14, 64, 3, 1, 1, 3), (3, 32, 9, 160, 1, 0, 1, 1), (2, 128, 13, 24, 3, 1, 2, 0),
-                                  (2, 3, 30, 64, 7, 3, 2, 3), (2, 16, 8, 20, 3, 1, 1, 3)])
+                                  (2, 3, 30, 64, 7, 3, 2, 3), (2, 16, 8, 20, 3, 1, 1, 3),
+                                  # 3x3 layers of the last stages: many channels, tiles with dead rows, 7x7 images
+                                  (3, 128, 14, 256, 3, 1, 1, 3), (6, 64, 7, 136, 3, 1, 1, 1), (2, 64, 28, 64, 3, 1, 1, 2)])
 def test_conv_with_folded_bn_inference(case):
     """Convolution with the inference batch norm (+ residual + relu) in its epilogue against the two
     separate operators of the oracle."""
@@ -150,6 +152,10 @@ BNSTATS_CASES = [
     (3, 32, 9, 160, 1, 0, 1, True),
     (2, 128, 13, 24, 3, 1, 2, True),
     (2, 3, 30, 64, 7, 3, 2, False),
+    # 3x3 layers of the last stages: row counts that are no multiple of the tile, 7x7 images, 56x56 at 64 channels
+    (3, 128, 14, 256, 3, 1, 1, True),
+    (6, 64, 7, 136, 3, 1, 1, False),
+    (2, 64, 56, 64, 3, 1, 1, True),
 ]
 
 
@@ -752,6 +758,12 @@ def test_rejects_bad_arguments():
     w = dev(np.zeros((4, 4, 3, 3), np.float32))
     with pytest.raises(K.SagaHipError):
         K.conv2d(K.CONV_FWD, x, w, y, pad=0)  # y should be 2x2
+    # an input smaller than the dilated filter has no output position at all: 4 + 0 < (3 - 1) * 3 + 1 with
+    # stride 2 would come out as one position if the shape rule's division truncated toward zero
+    y1 = dev(np.zeros((1, 4, 1, 1), np.float32))
+    p = K.ConvParams(0, 2, 3, 1)
+    assert K.lib().saga_hip_conv2d_fwd(C.byref(K.view(x)), C.byref(K.view(w)), C.byref(K.view(y1)), C.byref(p), 1.0, 0.0,
+                                       None, 0, S()) == -2
     assert K.lib().saga_hip_act_fwd(99, 0.0, C.byref(K.view(x)), C.byref(K.view(x)), 0.0, S()) == -1
 
 
@@ -767,6 +779,47 @@ RESNET_SHAPES = [
     (16, 32, 16, 3, 1, 1),
     (24, 9, 40, 3, 1, 1),
 ]
+
+
+# N, C, H, W, K: 3x3 / stride 1 / pad 1 problems at the image sizes and channel counts of the residual stages
+# (whole small images, ragged batches, output channels beyond / short of whole tiles, non-square images),
+# forward and backward data with beta 0 and 1, dense and as channel slices
+PATCH_CASES = [
+    (3, 64, 56, 56, 64),
+    (2, 128, 28, 28, 128),
+    (3, 256, 14, 14, 256),
+    (6, 512, 7, 7, 512),
+    (5, 64, 7, 7, 72),
+    (2, 64, 32, 32, 96),
+    (2, 128, 16, 16, 264),
+    (1, 192, 14, 14, 40),
+    (2, 64, 28, 56, 64),
+]
+
+
+@pytest.mark.parametrize("padc", [0, 8])
+@pytest.mark.parametrize("case", PATCH_CASES)
+def test_conv3x3_stage_shapes(case, padc):
+    N, Cc, H, W, Kk = case
+    dtype = torch.float16
+    rng = np.random.default_rng(N * 1000 + Cc + Kk + H)
+    x = rnd(rng, N, Cc, H, W, dtype=dtype)
+    w = rnd(rng, Kk, Cc, 3, 3, dtype=dtype, scale=(2.0 / (Cc * 9)) ** 0.5)
+    y_ref = ref.conv2d_fwd(x, w, 1, 1)
+    xd, wd = dev(x, dtype, "nhwc", padc), dev(w, dtype, "nhwc")
+    yd = dev(np.full_like(y_ref, 7.0), dtype, "nhwc", padc)
+    K.conv2d(K.CONV_FWD, xd, wd, yd, 1, 1)
+    assert_close(host(yd), y_ref, dtype, "y", tol=2e-3)
+    K.conv2d(K.CONV_FWD, xd, wd, yd, 1, 1, 1, 1, 1.0, 1.0)
+    assert_close(host(yd), 2 * y_ref, dtype, "y beta=1", tol=3e-3)
+    dy = rnd(rng, *y_ref.shape, dtype=dtype)
+    dyd = dev(dy, dtype, "nhwc", padc)
+    dxd = dev(np.full_like(x, 7.0), dtype, "nhwc", padc)
+    K.conv2d(K.CONV_BWD_DATA, dyd, wd, dxd, 1, 1)
+    dx_ref = ref.conv2d_bwd_data(dy, w, x.shape, 1, 1)
+    assert_close(host(dxd), dx_ref, dtype, "dx", tol=2e-3)
+    K.conv2d(K.CONV_BWD_DATA, dyd, wd, dxd, 1, 1, 1, 1, 1.0, 1.0)
+    assert_close(host(dxd), 2 * dx_ref, dtype, "dx beta=1", tol=3e-3)
 
 
 @pytest.mark.parametrize("shape", RESNET_SHAPES)
