@@ -46,10 +46,10 @@ FAMILIES = {
 # lines, the per-kernel table and the commit the counters were taken at are in
 # profiles/resnet50_b256_fp16_hbm_counters.txt; they go stale when kernels change, hence the label.
 MEASURED_HBM_BYTES_PER_LAUNCH = {
-    "conv": None,
-    "batchnorm": None,
+    "conv": 275571868,
+    "batchnorm": 460542165,
 }
-TRAFFIC_SOURCE = None
+TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE snapshot at commit 92e6e3e (profiles/resnet50_b256_fp16_hbm_counters.txt)"
 
 
 def by_kind(rows):
