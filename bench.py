@@ -220,6 +220,41 @@ def copy_calibration():
     print(json.dumps({"copy_bytes": n * 4, "launches": 5}))
 
 
+def conv_microbench(args):
+    """The single-layer convolution microbenchmark (N=256, 56x56, 64 -> 64 channels, 3x3, stride 1, pad 1) in fp16
+    NHWC and fp32 NCHW through the C ABI: forward, backward data and backward filter, inputs N(0,1), He-normal
+    filter, 59.19 GFLOP per pass.  HIP events on the launch stream, `steps` launches per pass after 3 warm-ups."""
+    import torch
+    from saga_amd import kernels as K
+
+    N, Cc, H, Kk, R = 256, 64, 56, 64, 3
+    flops = 2.0 * N * Kk * H * H * Cc * R * R
+    out = {}
+    for name, dt, cl in (("fp16_nhwc", torch.float16, True), ("fp32_nchw", torch.float32, False)):
+        g = torch.Generator(device="cuda").manual_seed(2)
+        mk = lambda *shape: torch.randn(*shape, dtype=dt, device="cuda", generator=g)
+        fmt = (lambda t: t.contiguous(memory_format=torch.channels_last)) if cl else (lambda t: t)
+        x, dy = fmt(mk(N, Cc, H, H)), fmt(mk(N, Kk, H, H))
+        w = fmt(mk(Kk, Cc, R, R) * (2.0 / (Cc * R * R)) ** 0.5)
+        y, dx, dw = torch.zeros_like(dy), torch.zeros_like(x), torch.zeros_like(w)
+        res = {}
+        for kind, a in (("fwd", (K.CONV_FWD, x, w, y)), ("bwd_data", (K.CONV_BWD_DATA, dy, w, dx)),
+                        ("bwd_filter", (K.CONV_BWD_FILTER, x, dy, dw))):
+            for _ in range(3):
+                K.conv2d(*a, 1, 1)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(args.steps):
+                K.conv2d(*a, 1, 1)
+            e1.record()
+            e1.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / args.steps
+            res[kind] = {"us": round(us, 1), "tflops": round(flops / us / 1e6, 1)}
+        out[name] = res
+    print(json.dumps({"conv_microbench": {"shape": "N256 C64 56x56 K64 3x3 s1 p1", "gflop_per_pass": round(flops / 1e9, 2),
+                                          "peak_tflops": {"fp16_nhwc": PEAK_FP16_TFLOPS, "fp32_nchw": 157.3}, **out}}))
+
+
 def host_input_rate(args):
     """The same two programs with the image batch and the labels declared as batched tensors: every step the
     engine uploads the host's back buffers (pinned memory, hipMemcpyAsync on the program's stream) before it
@@ -268,6 +303,8 @@ def main():
                     help="also write one line per operation of the training step (time, rate, own roofline bound)")
     ap.add_argument("--host-input", action="store_true",
                     help="time the programs with the batch handed over from host memory every step (PCIe included) and exit")
+    ap.add_argument("--conv-microbench", action="store_true",
+                    help="time the single-layer convolution microbenchmark (fp16 NHWC and fp32 NCHW) and exit")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run a plain 1 GiB device copy five times and exit (reference for the HBM counters)")
     args = ap.parse_args()
@@ -277,6 +314,8 @@ def main():
         return copy_calibration()
     if args.host_input:
         return host_input_rate(args)
+    if args.conv_microbench:
+        return conv_microbench(args)
 
     os.environ.setdefault("SAGA_HIP_PROFILE_PER_OP", "1")  # profile rows per operation, see by_kind()
     from saga_amd import api as S

@@ -85,6 +85,11 @@ class OracleNet:
                 y = fn(x_, k, at.get("pad", 0), at.get("stride", 1))
             elif ty == "sum":
                 y = get(i["x0"]) + get(i["x1"])
+            elif ty == "softmax":
+                # over the channels at every pixel, inference only (src/cuda/cuda_dnn.cpp:1928-1964)
+                if training:
+                    raise NotImplementedError("softmax has no backward pass in the reference")
+                y = ref.softmax(get(i["x"]))
             elif ty == "concat":
                 y = np.concatenate([get(i[f"x{j}"]) for j in range(len(i))], axis=at.get("axis", 1))
             elif ty == "fc":

@@ -203,10 +203,13 @@ def resnet50(batch=256, seed=4, dtype=S.HALF, image=224, classes=1000):
     return net
 
 
-def unet(batch=16, seed=5, dtype=S.HALF, image=256, classes=8, widths=(64, 128, 256, 512), bottleneck=1024):
+def unet(batch=16, seed=5, dtype=S.HALF, image=256, classes=8, widths=(64, 128, 256, 512), bottleneck=1024,
+         softmax=False):
     """U-Net-style encoder-decoder (config 5): 4 down stages (2 x conv3x3+bn+relu, maxpool 2), a
     bottleneck, 4 up stages (2x2/2 transposed conv, skip concat, 2 x conv3x3+bn+relu), 1x1 conv to
-    `classes` channels.  The skip concats are realised by the engine as strided outputs."""
+    `classes` channels.  The skip concats are realised by the engine as strided outputs.
+    softmax: the per-pixel softmax over the classes on top (an inference-only node in the reference,
+    src/cuda/cuda_dnn.cpp:1928-1964); net.output stays the class scores, net.softmax names the probabilities."""
     net = Net("unet", batch, (3, image, image), classes, dtype)
     b = Builder(net, seed)
 
@@ -225,6 +228,7 @@ def unet(batch=16, seed=5, dtype=S.HALF, image=256, classes=8, widths=(64, 128, 
         up = b.conv(x, f"up{i}-t", ch, 2, 2, 0, bias=True, transpose=True)
         x = double(b.concat([skips[i], up]), ch, f"up{i}")
     net.output = b.conv(x, "head", classes, 1, 1, 0, bias=True)
+    net.softmax = b.unary("softmax", net.output) if softmax else None
     return net
 
 

@@ -248,6 +248,44 @@ def test_unet_training_fp16():
                  check_params=["down0a-w", "up3-t-w", "up0-t-w", "up0a-w", "head-w", "up2-t-b"])
 
 
+def test_unet_real_widths_inference_with_per_pixel_softmax():
+    """Config 5 at its real widths (64 .. 1024 channels) and resolution (256 x 256), one image, inference with
+    the per-pixel softmax over the 8 classes: class scores and probabilities against the oracle network, the
+    per-pixel arg-max on all pixels where the oracle's two best classes are not within rounding of each other.
+    (Training goes through a pooled classifier head in test_unet_training_fp16: the reference's softmax node
+    has no backward pass and its catclassifier takes [N, C] scores.)"""
+    net = N.unet(1, image=256, softmax=True)
+    rng = np.random.default_rng(17)
+    # inference batch norm with non-trivial running statistics
+    for k in net.params:
+        if k.endswith("-m"):
+            net.params[k] = (rng.standard_normal(net.params[k].shape) * 0.1).astype(np.float32)
+        elif k.endswith("-v"):
+            net.params[k] = rng.uniform(0.5, 1.5, net.params[k].shape).astype(np.float32)
+    x, _ = inputs(net, 17)
+    ctx = S.Context()
+    g, t = N.build_graph(net, x, with_classifier=False)
+    p = ctx.create_program(g, 1, training=False)
+    scores, prob = ctx.resolve(t[net.output]), ctx.resolve(t[net.softmax])
+    p.run(1)
+    o = OracleNet(net)
+    o.forward(x, training=False)
+    want_s, want_p = o.acts[net.output], o.acts[net.softmax]
+    got_s, got_p = scores.read().astype(np.float32), prob.read().astype(np.float32)
+    rows = {}
+    for name, got, want in (("class scores", got_s, want_s), ("probabilities", got_p, want_p)):
+        e = rel_err(got, want)
+        rows[name] = [float(f"{e:.3e}"), 2e-2]
+        print(f"  {name}: rel max-abs err {e:.3e}")
+        assert e <= 2e-2, name
+    np.testing.assert_allclose(got_p.sum(1), 1.0, atol=4e-3)
+    top2 = np.sort(want_s, axis=1)[:, -2:]
+    clear = (top2[:, 1] - top2[:, 0]) > 4e-2 * np.abs(want_s).max()
+    assert clear.mean() > 0.5
+    assert np.array_equal(got_s.argmax(1)[clear], want_s.argmax(1)[clear])
+    record("test_unet_real_widths_inference_with_per_pixel_softmax", rows)
+
+
 def test_storage_reuse_arena():
     """Activations and gradients that live only within a step share one arena (the role of the
     reference's liveness + best-fit layout, src/cuda/cuda_analysis.cpp:194-547): it is smaller

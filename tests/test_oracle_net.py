@@ -308,3 +308,17 @@ def test_mixed_precision_steps_overflow_skips_and_loss_scale_rule():
             grown += 1
         assert o.loss_scale == scale, (step, o.loss_scale, scale)
     assert halved >= 2 and grown >= 2, (halved, grown)
+
+
+def test_per_pixel_softmax_head_against_torch():
+    """The `softmax` node (over the channels at every pixel, inference only) on top of a convolution."""
+    net = N.Net("head", 2, (4, 6, 5), 3, S.FLOAT)
+    b = N.Builder(net, 5)
+    net.output = b.unary("softmax", b.conv(net.input, "c", 3, 1, 1, 0, bias=True))
+    net.params["c-bt"] = (b.rng.standard_normal((1, 3)) * 0.5).astype(np.float32)
+    x, _ = batch(net, 9)
+    got = OracleNet(net).forward(x, training=False)
+    w = torch.tensor(net.params["c-w"].astype(np.float64))
+    want = torch.softmax(F.conv2d(torch.tensor(x.astype(np.float64)), w, torch.tensor(net.params["c-bt"].astype(np.float64)).reshape(-1)), 1)
+    assert worst(got, want.numpy()) <= 1e-6
+    np.testing.assert_allclose(got.sum(1), 1.0, atol=1e-6)
