@@ -29,13 +29,13 @@ PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 matrix
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
 MATRIX_KINDS = ("convfwd", "convbwddata", "convbwdfilter", "fc.")
-CONV_KINDS = ("convfwd", "convbwddata", "convbwdfilter")
+CONV_KINDS = ("convfwd", "convbwddata", "convbwddata.bn", "convbwdfilter")
 
 # Operation kinds that share kernels and a roofline bound form a family; `roofline` describes the family with
 # the most GPU time in the training step.
 FAMILIES = {
-    "conv": ("convfwd", "convbwddata", "convbwdfilter"),
-    "batchnorm": ("bntrain", "bntrain.fused", "bnbwd", "bnbwd.fused"),
+    "conv": ("convfwd", "convbwddata", "convbwddata.bn", "convbwdfilter"),
+    "batchnorm": ("bntrain", "bntrain.fused", "bnbwd", "bnbwd.fused", "bnbwd.linked"),
     "pool": ("poolfwd", "poolbwd"),
 }
 

@@ -155,6 +155,35 @@ int saga_hip_conv2d_fwd_bn_infer(const SagaTensorView *x, const SagaTensorView *
                                  const float *m, const float *v, float eps, int flags, void *workspace,
                                  size_t ws_bytes, saga_stream_t stream);
 
+/* ---- backward data of the convolution that consumes a batch norm's (+ relu) output, with the first pass
+ *      of that norm's backward done in the epilogue.  The reference runs cudnnConvolutionBackwardData
+ *      (src/cuda/cuda_dnn.cpp:467-476) and then cudnnBatchNormalizationBackwardEx (:2138-2163), whose first
+ *      pass reads the gradient and the norm's input again for two per-channel sums.  Here dx - which is
+ *      the gradient of the norm's result y = act(bn(link->x)) - is stored already masked by y > 0
+ *      (link->flags & SAGA_BN_RELU; the mask is recomputed from link->x with the forward's own expression)
+ *      and link->partial[link->partial_rows][C][2] receives, per block of pixels and channel, the sums of
+ *      the masked gradient and of masked gradient * (x - save_mean).  saga_hip_bn_bwd_linked then finishes
+ *      the norm's backward from dx and those sums.  This launch must be the only writer of dx that the
+ *      norm sees after it (beta != 0 accumulates onto earlier writers as usual).  wt: the transposed filter
+ *      of saga_hip_conv2d_bwd_data_wt, or NULL.  Returns SAGA_HIP_EUNSUPPORTED, with nothing written to dx,
+ *      outside the fp16 channels-last MFMA path (C % 8 == 0, stride 1, 2 or 4, dilation 1): run
+ *      saga_hip_conv2d_bwd_data(_wt) and saga_hip_bn_bwd_ex instead.  _size: bytes link->partial must
+ *      hold (0: never supported for these operands). */
+typedef struct SagaBnBwdLink {
+    const SagaTensorView *x;  /* the norm's input: dims of dx, fp16 channels-last, not dx itself */
+    const float *s, *b;       /* scale and bias; read only with SAGA_BN_RELU */
+    const float *save_mean, *save_invstd;
+    int32_t flags;            /* SAGA_BN_RELU or 0 */
+    int32_t partial_rows;     /* out */
+    float *partial;
+    size_t partial_bytes;
+} SagaBnBwdLink;
+size_t saga_hip_conv2d_bwd_data_bnbwd_size(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx,
+                                           const SagaConvParams *p);
+int saga_hip_conv2d_bwd_data_bnbwd(const SagaTensorView *dy, const SagaTensorView *w, const void *wt,
+                                   const SagaTensorView *dx, const SagaConvParams *p, float alpha, float beta,
+                                   void *workspace, size_t ws_bytes, SagaBnBwdLink *link, saga_stream_t stream);
+
 /* y[n,c,:,:] += b[c] : cudnnAddTensor of a {1,C,1,1} bias (src/cuda/cuda_dnn.cpp:39-68). b is fp32 or y's type. */
 int saga_hip_bias_add(const SagaTensorView *y, const SagaTensorView *b, saga_stream_t stream);
 /* db[c] = beta*db + sum_{n,h,w} dy : cudnnConvolutionBackwardBias (src/cuda/cuda_dnn.cpp:378-385). */
@@ -221,6 +250,16 @@ int saga_hip_bn_bwd_ex(const SagaTensorView *x, const SagaTensorView *y, const S
                        const float *save_mean, const float *save_invstd, float *ds, float *db, float beta_dx,
                        float beta_dz, float beta_p, int flags, const uint8_t *relu_mask, void *workspace,
                        size_t ws_bytes, saga_stream_t stream);
+
+/* second half of cudnnBatchNormalizationBackwardEx (src/cuda/cuda_dnn.cpp:2138-2163) for a norm whose
+ * first pass saga_hip_conv2d_bwd_data_bnbwd performed: g is the masked gradient that launch stored,
+ * partial[partial_rows][C][2] its sums.  Writes ds, db (beta_p as in saga_hip_bn_bwd) and
+ * dx = s*invstd*(g - db/M - (x - mean)*invstd*ds/M) + beta_dx*dx.  fp16 or fp32 channels-last tensors.
+ * workspace: saga_hip_bn_workspace_size(x). */
+int saga_hip_bn_bwd_linked(const SagaTensorView *x, const SagaTensorView *g, const SagaTensorView *dx, const float *s,
+                           const float *save_mean, const float *save_invstd, float *ds, float *db, float beta_dx,
+                           float beta_p, const float *partial, int partial_rows, void *workspace, size_t ws_bytes,
+                           saga_stream_t stream);
 
 /* ---- activations: cudnnActivationForward / Backward (src/cuda/cuda_dnn.cpp:631-638, :668-676),
  *      leaky relu kernel (src/cuda/cuda_kernels.cu:478-495).  y = act(x) + beta*y ; dx = dy*act'(x) + beta*dx. */

@@ -975,4 +975,43 @@ int saga_hip_bn_bwd_ex(const SagaTensorView *x, const SagaTensorView *y, const S
     return 0;
 }
 
+int saga_hip_bn_bwd_linked(const SagaTensorView *x, const SagaTensorView *g, const SagaTensorView *dx, const float *s,
+                           const float *save_mean, const float *save_invstd, float *ds, float *db, float beta_dx,
+                           float beta_p, const float *partial, int partial_rows, void *workspace, size_t ws_bytes,
+                           saga_stream_t stream)
+{
+    if(!valid_view(x) || !valid_view(g) || !valid_view(dx) || !s || !save_mean || !save_invstd || !ds || !db || !partial ||
+       partial_rows < 1)
+        return SAGA_HIP_EINVAL;
+    if(!same_dims(x, g) || !same_dims(x, dx))
+        return SAGA_HIP_ESHAPE;
+    const int dt = x->dtype;
+    if((dt != SAGA_HALF && dt != SAGA_FLOAT) || g->dtype != dt || dx->dtype != dt)
+        return SAGA_HIP_EUNSUPPORTED;
+    CLInfo lx, lg, ldx;
+    if(!as_channels_last(x, &lx) || !as_channels_last(g, &lg) || !as_channels_last(dx, &ldx))
+        return SAGA_HIP_EUNSUPPORTED;
+    const int C = lx.C;
+    if(!workspace || ws_bytes < 3 * (size_t)C * sizeof(float))
+        return SAGA_HIP_EWORKSPACE;
+    hipStream_t st = as_stream(stream);
+    float *coef = (float *)workspace;
+    const int vn = vec_width(dt, C, {x, g, dx}, {lx.pitch, lg.pitch, ldx.pitch});
+    const Shape sh = plan(lx.rows, C / vn);
+    const dim3 grid(sh.gx, sh.gy);
+    bn_bwd_finalize<<<C, 256, 0, st>>>(partial, partial_rows, s, save_invstd, ds, db, coef, (double)lx.rows, C, beta_p);
+#define GO(T, VN)                                                                                                     \
+    bn_bwd_apply_cl<T, VN, false><<<grid, 256, 0, st>>>((const T *)x->ptr, lx.pitch, nullptr, 0, (const T *)g->ptr,    \
+                                                        lg.pitch, (T *)dx->ptr, ldx.pitch, nullptr, 0, save_mean, coef, \
+                                                        lx.rows, C, sh.cvb, 0, beta_dx, 0.0f, nullptr)
+    if(dt == SAGA_HALF) {
+        if(vn == 8) GO(half_t, 8); else GO(half_t, 1);
+    } else {
+        if(vn == 4) GO(float, 4); else GO(float, 1);
+    }
+#undef GO
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
 } // extern "C"

@@ -178,6 +178,39 @@ int saga_hip_conv2d_bwd_data_wt(const SagaTensorView *dy, const SagaTensorView *
     return conv_mfma_bwd_data(dy, w, dx, g, alpha, beta, workspace, ws_bytes, as_stream(stream), wt);
 }
 
+size_t saga_hip_conv2d_bwd_data_bnbwd_size(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx,
+                                           const SagaConvParams *p)
+{
+    ConvGeom g;
+    if(geometry(dx, w, dy, p, &g) || force_direct() || !conv_mfma_bwd_data_ok(dy, w, dx, g) || g.C % 8 || g.dil != 1 ||
+       g.stride > 4)
+        return 0;
+    return conv_mfma_bnbwd_floats(g) * sizeof(float);
+}
+
+int saga_hip_conv2d_bwd_data_bnbwd(const SagaTensorView *dy, const SagaTensorView *w, const void *wt,
+                                   const SagaTensorView *dx, const SagaConvParams *p, float alpha, float beta,
+                                   void *workspace, size_t ws_bytes, SagaBnBwdLink *link, saga_stream_t stream)
+{
+    if(!link || !valid_view(link->x) || !link->save_mean || !link->partial)
+        return SAGA_HIP_EINVAL;
+    if((link->flags & ~SAGA_BN_RELU) || ((link->flags & SAGA_BN_RELU) && (!link->s || !link->b || !link->save_invstd)))
+        return SAGA_HIP_EINVAL;
+    ConvGeom g;
+    int r = geometry(dx, w, dy, p, &g);
+    if(r)
+        return r;
+    if(force_direct() || !conv_mfma_bwd_data_ok(dy, w, dx, g))
+        return SAGA_HIP_EUNSUPPORTED;
+    int rows = 0;
+    const ConvBnBwdLink l = {link->x, link->save_mean, link->save_invstd, link->s, link->b, link->flags & SAGA_BN_RELU,
+                             link->partial, link->partial_bytes / sizeof(float), &rows};
+    r = conv_mfma_bwd_data(dy, w, dx, g, alpha, beta, workspace, ws_bytes, as_stream(stream), wt, &l);
+    if(r == 0)
+        link->partial_rows = rows;
+    return r;
+}
+
 int saga_hip_conv2d_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, const SagaTensorView *dw,
                                const SagaConvParams *p, float alpha, float beta, void *workspace,
                                size_t ws_bytes, saga_stream_t stream)

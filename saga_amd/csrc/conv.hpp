@@ -34,9 +34,22 @@ struct ConvBnFold {
 int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTensorView *y, const ConvGeom &g,
                   float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st, float *stats = nullptr,
                   size_t stats_floats = 0, int *stats_rows = nullptr, const ConvBnFold *bn = nullptr);
+// backward data whose result dx is the gradient of a batch norm's (+ relu) output, with that norm's first
+// backward pass done in the epilogue: dx is stored masked by the relu and partial[*partial_rows][C][2]
+// receives sum(dx) and sum(dx * (x - mean)) per block row and channel.  EUNSUPPORTED (nothing written)
+// outside the pipelined kernel with 16-byte channel vectors.
+struct ConvBnBwdLink {
+    const SagaTensorView *x;               // the norm's input, dims of dx
+    const float *mean, *invstd, *s, *b;    // invstd, s, b only for relu
+    int relu;
+    float *partial;
+    size_t partial_floats;                 // at least conv_mfma_bnbwd_floats(g)
+    int *partial_rows;
+};
+size_t conv_mfma_bnbwd_floats(const ConvGeom &g);
 int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx,
                        const ConvGeom &g, float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st,
-                       const void *wt_ready = nullptr);
+                       const void *wt_ready = nullptr, const ConvBnBwdLink *link = nullptr);
 bool conv_mfma_bwd_data_ok(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx, const ConvGeom &g);
 int conv_mfma_transpose_blocks(int K, int C, int RS);
 int conv_mfma_transpose_batched(const SagaFilterTransposeJob *jobs, int njobs, int total_blocks, hipStream_t st);

@@ -59,6 +59,16 @@ struct GatherArgs {
     int bn_flags;      // SAGA_BN_RELU | SAGA_BN_ADD
     const half_t *z;   // residual, [M][ldz]
     int ldz;
+    // backward data only, optional (kernels instantiated with BQ): the output is the gradient of a batch norm's
+    // (+ relu) result and this launch is its only writer.  The epilogue masks it with that relu (recomputed from
+    // the norm's input as half(fma(x, s*invstd, b - mean*s*invstd)) > 0, what the forward stored), stores the
+    // masked gradient and leaves, per block row and channel, sum(g) and sum(g * (x - mean)) in
+    // bq_partial[stats_rows][Ngemm][2]: the first pass of the batch norm's backward.
+    const half_t *bq_x; // the norm's input, [M][bq_ldx]
+    int bq_ldx;
+    const float *bq_mean, *bq_s, *bq_invstd, *bq_b;
+    int bq_relu;
+    float *bq_partial;  // null: no link
     float *stats;      // forward only, optional: per block row and output channel, sum and sum of
                        // squares of the stored outputs, [ceil(M / BM)][Ngemm][2]
     int stats_rows;    // out: block rows the launch wrote
@@ -508,8 +518,227 @@ __device__ __forceinline__ void gather_epilogue(const GatherArgs &g, float16_t (
     }
 }
 
-template <int BM, int BN, int WGM, int WGN, int STAGES, int BKT, bool BWD, int PROD = 0>
-__global__ void __launch_bounds__(64 * (WGM * WGN + PROD), PROD ? (WGM * WGN + PROD + 3) / 4 : 1) conv_gather_gemm_dma(GatherArgs g)
+// The epilogue of a backward-data launch linked to a batch norm's backward (GatherArgs::bq_*): alpha / beta,
+// the norm's relu mask, the 16-byte channel-vector stores of the masked gradient and, per channel, the sums
+// of that gradient and of gradient * (x - mean) over the block's rows.  Arguments as in gather_epilogue; the
+// output must allow the vector stores.
+// Registers decide how many blocks a CU holds, so the work is laid out to need few of them: first every
+// accumulator is turned into the fp16 value an unlinked launch would store (two per register, half the
+// accumulators' footprint); then the wave tile is walked one 32x32 sub-tile at a time, rows inside
+// 32-channel columns, eight elements at a time, and the running sums are kept after the first step of the
+// halving exchange (8 per lane and sum instead of 16).  okr / pixr: validity and pixel index of this lane's row
+// in row block i (rows * pitch of either tensor fits 31 bits, checked on the host); xraw: bnbwd_prefetch's;
+// bnp: bnbwd_table's.
+typedef unsigned uint4_t __attribute__((ext_vector_type(4)));
+
+// Mean, and the forward's scale and shift for the relu recompute, of the block's BN channels: written to LDS
+// (behind the stage memory) by the first BN threads before the main loop, whose barriers publish it.
+template <int BN> __device__ __forceinline__ void bnbwd_table(const GatherArgs &g, float *bnp, int tid, int n0)
+{
+    if(tid < BN) {
+        const int n = n0 + tid;
+        float mean = 0.0f, sc = 0.0f, sh = 0.0f;
+        if(n < g.Ngemm) {
+            mean = g.bq_mean[n];
+            if(g.bq_relu) {
+                sc = g.bq_s[n] * g.bq_invstd[n];
+                sh = __builtin_fmaf(-mean, sc, g.bq_b[n]); // the forward's own expression
+            }
+        }
+        bnp[tid] = mean;
+        bnp[BN + tid] = sc;
+        bnp[2 * BN + tid] = sh;
+    }
+}
+
+// The norm's input for the linked epilogue below, fetched by the wavefront before its main loop so that the
+// data is in registers when the epilogue starts (four dependent trips to memory per block otherwise, which
+// nothing hides once every block of a CU reaches its epilogue at the same time): sub-tile t = j*TM + i
+// (row block i, 32-channel column j), two 16-byte vectors each, as the stores of the epilogue are laid out.
+template <int TM, int TN, int T0, int T1>
+__device__ __forceinline__ void bnbwd_prefetch(const GatherArgs &g, int lane, int wn, int n0, const bool (&okr)[TM],
+                                               const int (&pixr)[TM], uint4_t (&xraw)[TM * TN][2])
+{
+    const int hi = lane >> 5;
+#pragma unroll
+    for(int t = T0; t < T1; t++) {
+        const int j = t / TM, i = t % TM;
+        const half_t *row = g.bq_x + pixr[i] * g.bq_ldx;
+#pragma unroll
+        for(int q = 0; q < 2; q++) {
+            const int n = n0 + wn + j * 32 + 16 * q + 8 * hi;
+            const uint4_t z = {0, 0, 0, 0};
+            xraw[t][q] = z;
+            if(okr[i] && n < g.Ngemm)
+                xraw[t][q] = *(const uint4_t *)(row + n);
+        }
+    }
+}
+
+template <int TM, int TN, int WGM, int WGN, int BN>
+__device__ __forceinline__ void gather_epilogue_bnbwd(const GatherArgs &g, float16_t (&acc)[TM][TN], char *smem, int tid,
+                                                      int lane, int wave, int wm, int wn, int n0, int stats_row,
+                                                      const bool (&okr)[TM], const int (&pixr)[TM],
+                                                      uint4_t (&xraw)[TM * TN][2], const float *bnp)
+{
+    typedef uint4_t u4;
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    const int hi = lane >> 5;
+    // phase 1: pk[i][j][4q .. 4q+3] = channels 8q .. 8q+7 of this lane's accumulator elements, as stored
+    unsigned pk[TM][TN][8];
+#pragma unroll
+    for(int j = 0; j < TN; j++)
+#pragma unroll
+        for(int i = 0; i < TM; i++) {
+            float f[16];
+#pragma unroll
+            for(int v = 0; v < 16; v++)
+                f[v] = g.alpha * acc[i][j][v];
+            if(g.beta != 0.0f) {
+                float old[16];
+                load_row32(g.out + pixr[i] * g.ldo, okr[i], n0 + wn + j * 32, g.Ngemm, hi, old);
+#pragma unroll
+                for(int v = 0; v < 16; v++)
+                    f[v] += g.beta * old[v];
+            }
+#pragma unroll
+            for(int e = 0; e < 8; e++) {
+                pk[i][j][e] = pack2(f[2 * e], f[2 * e + 1]);
+                asm volatile("" : "+v"(pk[i][j][e])); // converted here and now: the accumulator is dead from here on
+            }
+        }
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads(); // the parameter table is complete (a block may have had no main-loop barrier to publish it)
+    // phase 2
+    float sres[TN], qres[TN];
+    float sv[8], qv[8];
+#pragma unroll
+    for(int t = 0; t < TM * TN; t++) {
+        const int j = t / TM, i = t % TM;
+        const int nb = n0 + wn + j * 32;
+        const bool ok = okr[i];
+        const u4 (&cur)[2] = xraw[t];
+        if(i == 0) {
+#pragma unroll
+            for(int v = 0; v < 8; v++)
+                sv[v] = qv[v] = 0.0f;
+        }
+        // the norm's input in accumulator order (the same half-wave swap as on the way out, undone):
+        // wx[c][2*(e/2) .. ] holds elements 8c + 2*ee, 8c + 2*ee + 1 in word ee
+        unsigned wx[2][4];
+#pragma unroll
+        for(int c = 0; c < 2; c++) {
+            const auto s0 = __builtin_amdgcn_permlane32_swap(cur[c][0], cur[c][2], false, false);
+            const auto s1 = __builtin_amdgcn_permlane32_swap(cur[c][1], cur[c][3], false, false);
+            wx[c][0] = s0[0]; wx[c][1] = s1[0]; wx[c][2] = s0[1]; wx[c][3] = s1[1];
+        }
+        // Elements are handled eight at a time: the four of channel group q = half and the four of group
+        // q + 2, which are the partners of the first step of the halving exchange (element k with k + 8; the
+        // lane with bit 16 set keeps the upper one, its partner 16 lanes away the lower one) - that step is
+        // folded into the running sums right away, so only eight gradients and products are live at a time.
+#pragma unroll
+        for(int half = 0; half < 2; half++) {
+            float gf[2][4], gq[2][4];
+#pragma unroll
+            for(int side = 0; side < 2; side++) {
+                const int q = half + 2 * side;
+                // the table is read again for every sub-tile (the opaque index keeps the compiler from holding
+                // a column's 48 parameters in registers across its rows)
+                int cl = wn + j * 32 + 8 * q + 4 * hi;
+                asm volatile("" : "+v"(cl));
+                const float4_t mean = *(const float4_t *)(bnp + cl), sc = *(const float4_t *)(bnp + BN + cl),
+                               sh = *(const float4_t *)(bnp + 2 * BN + cl);
+#pragma unroll
+                for(int e2 = 0; e2 < 2; e2++) {
+                    const unsigned word = pk[i][j][2 * q + e2];
+                    const h2 hv = __builtin_bit_cast(h2, word), xv = __builtin_bit_cast(h2, wx[side][2 * half + e2]);
+                    unsigned keep = 0;
+#pragma unroll
+                    for(int h = 0; h < 2; h++) {
+                        const int e = 2 * e2 + h;
+                        const float xe = (float)xv[h];
+                        const bool pos = !g.bq_relu || (float)(half_t)__builtin_fmaf(xe, sc[e], sh[e]) > 0.0f;
+                        const bool on = ok && pos;
+                        keep |= on ? (h ? 0xffff0000u : 0x0000ffffu) : 0u;
+                        const float gv = on ? (float)hv[h] : 0.0f;
+                        gf[side][e] = gv;
+                        gq[side][e] = gv * (xe - mean[e]);
+                    }
+                    pk[i][j][2 * q + e2] = word & keep;
+                }
+            }
+            // v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even rows of the
+            // second: afterwards the two operands of a lane add up to what it keeps plus what its partner sent
+#pragma unroll
+            for(int e = 0; e < 4; e++) {
+                const auto a = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, gf[0][e]),
+                                                                __builtin_bit_cast(unsigned, gf[1][e]), false, false);
+                const auto b = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, gq[0][e]),
+                                                                __builtin_bit_cast(unsigned, gq[1][e]), false, false);
+                // (the four results go through an opaque statement: hipcc 7.2 otherwise folds the sum of the
+                // two results of one swap into twice the first)
+                unsigned a0 = a[0], a1 = a[1], b0 = b[0], b1 = b[1];
+                asm volatile("" : "+v"(a0), "+v"(a1), "+v"(b0), "+v"(b1));
+                sv[4 * half + e] += __builtin_bit_cast(float, a0) + __builtin_bit_cast(float, a1);
+                qv[4 * half + e] += __builtin_bit_cast(float, b0) + __builtin_bit_cast(float, b1);
+            }
+            // added here and now (left to itself the compiler postpones the additions to the end of the column
+            // and keeps every exchanged value in a register until then)
+#pragma unroll
+            for(int e = 0; e < 4; e++)
+                asm volatile("" : "+v"(sv[4 * half + e]), "+v"(qv[4 * half + e]));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // after the swaps: lower half-wave holds channels 0..7 (then 16..23) of the tile,
+        // upper half-wave 8..15 (24..31): one store covers 32 contiguous bytes per pixel
+        half_t *orow = g.out + pixr[i] * g.ldo;
+#pragma unroll
+        for(int q = 0; q < 2; q++) {
+            const auto s0_ = __builtin_amdgcn_permlane32_swap(pk[i][j][4 * q + 0], pk[i][j][4 * q + 2], false, false);
+            const auto s1_ = __builtin_amdgcn_permlane32_swap(pk[i][j][4 * q + 1], pk[i][j][4 * q + 3], false, false);
+            const int n = nb + 16 * q + 8 * hi;
+            if(ok && n < g.Ngemm) {
+                const u4 o = {s0_[0], s1_[0], s0_[1], s1_[1]};
+                *(u4 *)(orow + n) = o;
+            }
+        }
+        if(i == TM - 1) {
+            // lanes of a half-wave hold different pixels of the same 16 channels: after the remaining halving
+            // exchanges each pair of lanes holds one channel's total over the wave tile's rows
+            halve_exchange<8>(sv, qv, lane, 8);
+            halve_exchange<4>(sv, qv, lane, 4);
+            halve_exchange<2>(sv, qv, lane, 2);
+            sres[j] = sv[0] + __shfl_xor(sv[0], 1, 64);
+            qres[j] = qv[0] + __shfl_xor(qv[0], 1, 64);
+        }
+        __builtin_amdgcn_sched_barrier(0); // one sub-tile at a time: interleaving them costs registers
+    }
+    // pair p = (lane%32)/2 holds, per column j, channel 32*j + 8*(p/4) + 4*hi + p%4 of the wave tile;
+    // the wavefronts stacked along M are added through LDS in a fixed order
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    float2_t *red = (float2_t *)smem;
+    const int p = (lane & 31) >> 1;
+    __syncthreads(); // every wavefront is done reading the last slice, which the sums below overwrite
+    if((lane & 1) == 0) {
+#pragma unroll
+        for(int j = 0; j < TN; j++) {
+            const float2_t v2 = {sres[j], qres[j]};
+            red[(wave / WGN) * BN + wn + 32 * j + 8 * (p >> 2) + 4 * hi + (p & 3)] = v2;
+        }
+    }
+    __syncthreads();
+    if(tid < BN && n0 + tid < g.Ngemm) {
+        float2_t t = red[tid];
+#pragma unroll
+        for(int wy = 1; wy < WGM; wy++)
+            t += red[wy * BN + tid];
+        *(float2_t *)(g.bq_partial + ((int64_t)stats_row * g.Ngemm + n0 + tid) * 2) = t;
+    }
+}
+
+template <int BM, int BN, int WGM, int WGN, int STAGES, int BKT, bool BWD, int PROD = 0, bool BQ = false>
+__global__ void __launch_bounds__(64 * (WGM * WGN + PROD), (BQ && WGM * WGN + PROD == 8) ? 4 : PROD ? (WGM * WGN + PROD + 3) / 4 : 1)
+    conv_gather_gemm_dma(GatherArgs g)
 {
     constexpr int NW = WGM * WGN;                      // wavefronts per block
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
@@ -534,12 +763,14 @@ __global__ void __launch_bounds__(64 * (WGM * WGN + PROD), PROD ? (WGM * WGN + P
     int bid = xcd_remap(blockIdx.x, g.nblocks);
     int py = 0, px = 0, r0 = 0, s0 = 0, nr = g.R, ns = g.S, rstep = 1;
     int PH = g.OH, PW = g.OW; // pixel grid this block's rows are numbered over
+    int srow0 = 0;            // first row of this block's class in the per-row sums
     if(BWD && g.classes > 1) {
         // the classes of one tile position are neighbours in block order: they read the same
         // rows of dy and write interleaved pixels of the same rows of dx, which L2 then shares
         const int ci = bid % g.nactive;
         bid /= g.nactive;
         const int cls = g.cls_ids[ci];
+        srow0 = ci * (g.blocks_per_class / g.nblk_n);
         py = cls >> g.sshift;
         px = cls & (g.stride - 1);
         r0 = (py + g.pad) & (g.stride - 1);
@@ -705,6 +936,11 @@ __global__ void __launch_bounds__(64 * (WGM * WGN + PROD), PROD ? (WGM * WGN + P
                     __syncthreads();
                 }
             }
+            if constexpr(BQ) { // the parameter table's barrier and the two of the sums
+                __syncthreads();
+                __syncthreads();
+                __syncthreads();
+            }
             return;
         }
     }
@@ -790,6 +1026,39 @@ __global__ void __launch_bounds__(64 * (WGM * WGN + PROD), PROD ? (WGM * WGN + P
                 acc[i][j][v] = 0.0f;
 
     const int wm = (wave / WGN) * WTM, wn = (wave % WGN) * WTN;
+    auto rowpix = [&](int i, bool &ok, int64_t &pix) {
+        const int m = m0 + wm + i * 32 + (lane & 31);
+        ok = m < Mloc;
+        pix = m;
+        if(BWD && g.classes > 1) {
+            const int mm = ok ? m : 0;
+            const int ox = mm % PW;
+            const int t = mm / PW;
+            const int oy = t % PH;
+            const int n = t / PH;
+            const int y = oy * rstep + py, x = ox * rstep + px;
+            ok = ok && y < g.OH && x < g.OW;
+            pix = ((int64_t)n * g.OH + y) * g.OW + x;
+        }
+    };
+    // linked to a batch norm's backward: that norm's input for this wavefront's tile is requested now and
+    // arrives while the main loop runs
+    bool bq_ok[BQ ? TM : 1];
+    int bq_pix[BQ ? TM : 1];
+    uint4_t bq_x[BQ ? TM * TN : 1][2];
+    float *bq_tab = (float *)(smem + STAGES * (BM + BN) * BKT * 2);
+    if constexpr(BQ) {
+#pragma unroll
+        for(int i = 0; i < TM; i++) {
+            int64_t pix;
+            rowpix(i, bq_ok[i], pix);
+            bq_pix[i] = (int)pix;
+        }
+        bnbwd_table<BN>(g, bq_tab, tid, n0);
+        // (wavefronts that also issue the main loop's loads have no registers to spare: they ask after the loop)
+        if constexpr(PROD > 0)
+            bnbwd_prefetch<TM, TN, 0, TM * TN>(g, lane, wn, n0, bq_ok, bq_pix, bq_x);
+    }
     const int frow = lane & 31;
     const int swz = swz_of(frow);
     // byte offset inside a row of this lane's fragment vector for MFMA step kk (k = 16*kk ..)
@@ -859,21 +1128,13 @@ __global__ void __launch_bounds__(64 * (WGM * WGN + PROD), PROD ? (WGM * WGN + P
         }
     }
 
-    gather_epilogue<TM, TN, WGM, WGN, BN, BWD, false>(g, acc, smem, tid, lane, wave, wm, wn, n0, bm, [&](int i, bool &ok, int64_t &pix) {
-        const int m = m0 + wm + i * 32 + (lane & 31);
-        ok = m < Mloc;
-        pix = m;
-        if(BWD && g.classes > 1) {
-            const int mm = ok ? m : 0;
-            const int ox = mm % PW;
-            const int t = mm / PW;
-            const int oy = t % PH;
-            const int n = t / PH;
-            const int y = oy * rstep + py, x = ox * rstep + px;
-            ok = ok && y < g.OH && x < g.OW;
-            pix = ((int64_t)n * g.OH + y) * g.OW + x;
-        }
-    });
+    if constexpr(BQ && PROD == 0)
+        bnbwd_prefetch<TM, TN, 0, TM * TN>(g, lane, wn, n0, bq_ok, bq_pix, bq_x);
+    if constexpr(BQ)
+        gather_epilogue_bnbwd<TM, TN, WGM, WGN, BN>(g, acc, smem, tid, lane, wave, wm, wn, n0, srow0 + bm, bq_ok, bq_pix,
+                                                    bq_x, bq_tab);
+    else
+        gather_epilogue<TM, TN, WGM, WGN, BN, BWD, false>(g, acc, smem, tid, lane, wave, wm, wn, n0, bm, rowpix);
 }
 
 // Many filters in one launch: job j owns the blocks first_block[j] .. first_block[j+1]-1, one block per
@@ -1626,7 +1887,8 @@ template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
             // classes that no tap reaches produce beta*out: nothing to do for beta == 1, one
             // coalesced fill for beta == 0 (a vectorisable output; otherwise they keep their blocks)
             const bool can_fill = (g.ldo & 7) == 0 && (g.Ngemm & 7) == 0 && ((uintptr_t)g.out & 15) == 0;
-            const bool drop = g.beta == 1.0f || (g.beta == 0.0f && can_fill);
+            // (linked to a batch norm's backward, every pixel's old value counts in the sums: beta == 1 keeps all classes)
+            const bool drop = (g.beta == 1.0f && !g.bq_partial) || (g.beta == 0.0f && can_fill);
             active = 0;
             for(int c = 0; c < g.classes; c++) {
                 const int r0 = ((c >> g.sshift) + g.pad) & (g.stride - 1), s0 = ((c & (g.stride - 1)) + g.pad) & (g.stride - 1);
@@ -1653,10 +1915,23 @@ template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
             if(tile == 5 && (int64_t)((g.Mc + 255) / 256) * ((g.Ngemm + 127) / 128) * active <= 256)
                 tile = 12;
         }
+        // linked to a batch norm's backward: only the 256-row tiles carry the link
+        if(g.bq_partial && tile != 5 && tile != 12 && tile != 13)
+            tile = g.Ngemm <= 64 ? 13 : 5;
 #define LAUNCH(BM, BN, WGM, WGN, BKT, PROD)                                                            \
     do {                                                                                               \
-        auto kern = conv_gather_gemm_dma<BM, BN, WGM, WGN, ST, BKT, BWD, PROD>;                         \
-        constexpr int lds = ST * (BM + BN) * BKT * 2;                                                  \
+        if constexpr(BWD && BM == 256 && (PROD > 0 || BN == 128)) {                                     \
+            if(g.bq_partial) {                                                                         \
+                LAUNCH_(BM, BN, WGM, WGN, BKT, PROD, true);                                            \
+                break;                                                                                 \
+            }                                                                                          \
+        }                                                                                              \
+        LAUNCH_(BM, BN, WGM, WGN, BKT, PROD, false);                                                   \
+    } while(0)
+#define LAUNCH_(BM, BN, WGM, WGN, BKT, PROD, BQ)                                                       \
+    do {                                                                                               \
+        auto kern = conv_gather_gemm_dma<BM, BN, WGM, WGN, ST, BKT, BWD, PROD, BQ>;                     \
+        constexpr int lds = ST * (BM + BN) * BKT * 2 + (BQ ? 3 * BN * 4 : 0);                          \
         static bool once = false;                                                                      \
         if(lds > 64 * 1024 && !once) {                                                                 \
             const hipError_t e__ = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds); \
@@ -1668,7 +1943,7 @@ template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
         g.blocks_per_class = ((g.Mc + BM - 1) / BM) * g.nblk_n;                                        \
         g.nblocks = g.blocks_per_class * active;                                                       \
         g.nactive = active;                                                                            \
-        g.stats_rows = (g.Mc + BM - 1) / BM;                                                           \
+        g.stats_rows = ((g.Mc + BM - 1) / BM) * active;                                                \
         kern<<<g.nblocks, 64 * (WGM * WGN + PROD), lds, st>>>(g);                                      \
     } while(0)
         switch(tile) {
@@ -1679,10 +1954,11 @@ template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
         default: LAUNCH(256, 64, 4, 1, 32, 0); break;
         }
 #undef LAUNCH
+#undef LAUNCH_
         SAGA_CHECK_LAUNCH();
         return 0;
     }
-    if(g.stats || (!BWD && g.bn_s))
+    if(g.stats || (!BWD && g.bn_s) || g.bq_partial)
         return SAGA_HIP_EUNSUPPORTED;
     // tile choice by output-channel count; M tiles are 128 or 256 rows
     if(g.Ngemm > 64) {
@@ -1753,6 +2029,13 @@ static bool set_bn(GatherArgs &a, const ConvBnFold *bn, const SagaTensorView *y,
 }
 
 } // namespace
+
+// floats a linked backward-data launch may write: per residue class of the stride, one row per 128 pixels
+size_t conv_mfma_bnbwd_floats(const ConvGeom &g)
+{
+    const int64_t Mc = (int64_t)g.N * ((g.H + g.stride - 1) / g.stride) * ((g.W + g.stride - 1) / g.stride);
+    return (size_t)((Mc + 127) / 128) * g.stride * g.stride * g.C * 2;
+}
 
 // floats a forward launch may write into its statistics buffer: the smallest M tile is 128 rows
 size_t conv_mfma_stats_floats(const ConvGeom &g)
@@ -1832,6 +2115,7 @@ int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTe
         a.a_bytes = (unsigned)(px * 8);
         a.b_bytes = (unsigned)(wn * 2);
         a.stats = stats;
+        a.bq_partial = nullptr;
         if(!set_bn(a, bn, y, ly))
             return SAGA_HIP_EUNSUPPORTED;
         const int rc = launch_gather<false>(a, st);
@@ -1875,6 +2159,7 @@ int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTe
         a.b_bytes = bb < 0x7fffff00 ? (unsigned)bb : 0;
     }
     a.stats = stats;
+    a.bq_partial = nullptr;
     if(!set_bn(a, bn, y, ly))
         return SAGA_HIP_EUNSUPPORTED;
     const int rc = launch_gather<false>(a, st);
@@ -1902,14 +2187,29 @@ bool conv_mfma_bwd_data_ok(const SagaTensorView *dy, const SagaTensorView *w, co
 // otherwise it is transposed into the workspace first
 int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx,
                        const ConvGeom &g, float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st,
-                       const void *wt_ready)
+                       const void *wt_ready, const ConvBnBwdLink *link)
 {
-    CLInfo ldy, ldx;
+    CLInfo ldy, ldx, lbx;
     if(!common_ok(dy, w, dx, g, &ldy, &ldx))
         return SAGA_HIP_EUNSUPPORTED;
     const int sshift = ilog2_exact(g.stride);
     if(sshift < 0)
         return SAGA_HIP_EUNSUPPORTED;
+    if(link) {
+        // only the pipelined kernel's vector epilogue carries the link; checked before anything is launched
+        const int64_t ab = ((ldy.rows - 1) * ldy.pitch + ldy.C) * 2, bb = (int64_t)g.K * g.R * g.S * g.C * 2;
+        const bool kernel_ok = dma_stages() >= 2 && ab < 0x7fffff00 && bb < 0x7fffff00 && g.dil == 1 && g.stride <= 4 &&
+                               ((g.R + g.stride - 1) / g.stride) * ((g.S + g.stride - 1) / g.stride) <= 64;
+        const bool vec = ldx.pitch % 8 == 0 && g.C % 8 == 0 && aligned16(dx->ptr);
+        if(!kernel_ok || !vec || !link->x || link->x->dtype != SAGA_HALF || !same_dims(link->x, dx) ||
+           !as_channels_last(link->x, &lbx) || lbx.rows != ldx.rows || lbx.pitch % 8 || !aligned16(link->x->ptr) ||
+           link->x->ptr == dx->ptr)
+            return SAGA_HIP_EUNSUPPORTED;
+        if(!link->mean || !link->partial || (link->relu && (!link->s || !link->b || !link->invstd)))
+            return SAGA_HIP_EINVAL;
+        if(link->partial_floats < conv_mfma_bnbwd_floats(g))
+            return SAGA_HIP_EWORKSPACE;
+    }
     const half_t *wt = (const half_t *)wt_ready;
     if(!wt) {
         const size_t need = (size_t)g.K * g.C * g.R * g.S * sizeof(half_t);
@@ -1943,7 +2243,18 @@ int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const 
     }
     a.stats = nullptr;
     a.bn_s = nullptr;
-    return launch_gather<true>(a, st);
+    a.bq_partial = nullptr;
+    if(link) {
+        a.bq_x = (const half_t *)link->x->ptr;
+        a.bq_ldx = (int)lbx.pitch;
+        a.bq_mean = link->mean; a.bq_s = link->s; a.bq_invstd = link->invstd; a.bq_b = link->b;
+        a.bq_relu = link->relu ? 1 : 0;
+        a.bq_partial = link->partial;
+    }
+    const int rc = launch_gather<true>(a, st);
+    if(link && link->partial_rows)
+        *link->partial_rows = a.stats_rows;
+    return rc;
 }
 
 int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, const SagaTensorView *dw,

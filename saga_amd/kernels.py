@@ -29,6 +29,12 @@ class FilterTransposeJob(C.Structure):
                 ("first_block", C.c_int32)]
 
 
+class BnBwdLink(C.Structure):
+    _fields_ = [("x", C.POINTER(TensorView)), ("s", C.c_void_p), ("b", C.c_void_p), ("save_mean", C.c_void_p),
+                ("save_invstd", C.c_void_p), ("flags", C.c_int32), ("partial_rows", C.c_int32), ("partial", C.c_void_p),
+                ("partial_bytes", C.c_size_t)]
+
+
 class SagaHipError(RuntimeError):
     pass
 
@@ -54,6 +60,9 @@ SIGNATURES = {
     "saga_hip_filter_transpose_blocks": (_I, [_TV]),
     "saga_hip_filter_transpose_batched": (_I, [_VP, _I, _I, _VP]),
     "saga_hip_conv2d_bwd_data_wt": (_I, [_TV, _TV, _VP, _TV, C.POINTER(ConvParams), _F, _F, _VP, _SZ, _VP]),
+    "saga_hip_conv2d_bwd_data_bnbwd_size": (_SZ, [_TV, _TV, _TV, C.POINTER(ConvParams)]),
+    "saga_hip_conv2d_bwd_data_bnbwd": (_I, [_TV, _TV, _VP, _TV, C.POINTER(ConvParams), _F, _F, _VP, _SZ,
+                                            C.POINTER(BnBwdLink), _VP]),
     "saga_hip_bias_add": (_I, [_TV, _TV, _VP]),
     "saga_hip_bias_bwd_workspace_size": (_SZ, [_TV]),
     "saga_hip_bias_bwd": (_I, [_TV, _TV, _F, _VP, _SZ, _VP]),
@@ -67,6 +76,7 @@ SIGNATURES = {
     "saga_hip_bn_bwd": (_I, [_TV, _TV, _TV, _TV, _TV, _VP, _VP, _VP, _VP, _VP, _F, _F, _F, _I, _VP, _SZ, _VP]),
     "saga_hip_bn_bwd_ex": (_I, [_TV, _TV, _TV, _TV, _TV, _VP, _VP, _VP, _VP, _VP, _VP, _F, _F, _F, _I, _VP, _VP, _SZ,
                                 _VP]),
+    "saga_hip_bn_bwd_linked": (_I, [_TV, _TV, _TV, _VP, _VP, _VP, _VP, _VP, _F, _F, _VP, _I, _VP, _SZ, _VP]),
     "saga_hip_act_fwd": (_I, [_I, _F, _TV, _TV, _F, _VP]),
     "saga_hip_act_bwd": (_I, [_I, _F, _TV, _TV, _TV, _TV, _F, _VP]),
     "saga_hip_pool_fwd": (_I, [_I, _TV, _TV, _TV, _I, _I, _I, _VP]),

@@ -192,6 +192,10 @@ struct HipOperation {
     std::string m_kind;
 };
 
+struct HipProgram;
+// hip_ops.cpp: hands the first pass of a batch norm's backward to the convolution that writes its gradient
+void link_bn_backward(HipProgram &p, std::vector<std::shared_ptr<HipOperation>> &ops);
+
 struct HipProgramUnit {
     Nodes m_transformed;
     int m_batch_size = 1;

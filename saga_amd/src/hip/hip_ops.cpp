@@ -227,11 +227,46 @@ struct FilterTransposeBatch : public HipOperation {
     }
 };
 
+// Per-channel sums of a relu-masked gradient, handed from the ConvBwdData that is the last writer of a
+// batch norm's output gradient to that norm's BnBwd, which then skips its own first pass over the tensor.
+struct BnBwdLinkState {
+    std::shared_ptr<HipMemory> partial;
+    int rows = 0;
+    bool valid = false; // set by every ConvBwdData::exec, consumed by the BnBwd::exec that follows
+};
+
 struct ConvBwdData : public HipOperation {
     const T w_, dy_, dx_;
     T wt_; // the filter as C,R,S,K, written by the program's FilterTransposeBatch (null: transposed per call)
     const SagaConvParams cp_;
     float beta_ = 0;
+    // dx is the gradient of a batch norm's (+ relu) output and this is its last writer: the epilogue masks it
+    // and leaves the sums of the norm's backward (x, scale, bias, saved mean and 1/std of that norm)
+    std::shared_ptr<BnBwdLinkState> link_;
+    T bn_x_, bn_s_, bn_b_, bn_sm_, bn_sv_;
+    int bn_flags_ = 0;
+    std::shared_ptr<BnBwdLinkState> linkBnBwd(T x, T s, T b, T sm, T sv, int flags)
+    {
+        if(link_)
+            return nullptr;
+        // The epilogue's extra work (one more tensor to read, the mask and the sums) costs the convolution
+        // more than the norm's first pass saves where the convolution has little arithmetic per output to
+        // hide it behind: measured on MI355X at batch 256, linking loses at 64 channels (1x1 and 3x3) and
+        // at 128 channels under a 1x1 filter, and wins from there up.  SAGA_HIP_BNBWD_LINK_ALL links all.
+        const int channels = (int)dx_->m_dims[1], taps = (int)w_->m_dims[2] * (int)w_->m_dims[3];
+        if(!(channels >= 256 || (channels >= 128 && taps > 1)) && !getenv("SAGA_HIP_BNBWD_LINK_ALL"))
+            return nullptr;
+        const SagaTensorView vx = dx_->shapeView(), vw = w_->shapeView(), vy = dy_->shapeView();
+        const size_t bytes = saga_hip_conv2d_bwd_data_bnbwd_size(&vy, &vw, &vx, &cp_);
+        if(!bytes)
+            return nullptr;
+        link_ = std::make_shared<BnBwdLinkState>();
+        link_->partial = std::make_shared<HipMemory>(bytes);
+        bn_x_ = x; bn_s_ = s; bn_b_ = b; bn_sm_ = sm; bn_sv_ = sv;
+        bn_flags_ = flags;
+        m_kind = "convbwddata.bn";
+        return link_;
+    }
     ConvBwdData(HipProgram &p, HipProgramUnit &pu, T w, T dy, T dx, SagaConvParams cp)
       : HipOperation("convbwddata"), w_(w), dy_(dy), dx_(dx), cp_(cp)
     {
@@ -251,6 +286,28 @@ struct ConvBwdData : public HipOperation {
     void exec(HipProgram &p) override
     {
         const SagaTensorView vdy = dy_->view(), vw = w_->view(), vdx = dx_->view();
+        if(link_) {
+            link_->valid = false;
+            const SagaTensorView vx = bn_x_->view();
+            SagaBnBwdLink l = {&vx,
+                               (const float *)bn_s_->deviceMem(),
+                               (const float *)bn_b_->deviceMem(),
+                               (const float *)bn_sm_->deviceMem(),
+                               (const float *)bn_sv_->deviceMem(),
+                               bn_flags_,
+                               0,
+                               (float *)link_->partial->m_ptr,
+                               link_->partial->m_bytes};
+            const int r = saga_hip_conv2d_bwd_data_bnbwd(&vdy, &vw, wt_ ? wt_->deviceMem() : nullptr, &vdx, &cp_, 1.0f, beta_,
+                                                         p.m_ctx->m_workspace.ptr(), p.m_ctx->m_workspace.size(), &l, S(p));
+            if(r == 0) {
+                link_->rows = l.partial_rows;
+                link_->valid = true;
+                return;
+            }
+            if(r != SAGA_HIP_EUNSUPPORTED)
+                chkSaga(r);
+        }
         chkSaga(saga_hip_conv2d_bwd_data_wt(&vdy, &vw, wt_ ? wt_->deviceMem() : nullptr, &vdx, &cp_, 1.0f, beta_,
                                             p.m_ctx->m_workspace.ptr(), p.m_ctx->m_workspace.size(), S(p)));
     }
@@ -259,12 +316,17 @@ struct ConvBwdData : public HipOperation {
         HipOpArgs r{{"w", w_}, {"dy", dy_}};
         if(wt_)
             r.push_back({"wt", wt_});
+        if(link_)
+            r.insert(r.end(), {{"bn.x", bn_x_}, {"bn.s", bn_s_}, {"bn.b", bn_b_}, {"bn.sm", bn_sm_}, {"bn.sv", bn_sv_}});
         return r;
     }
     HipOpArgs listOutputs() const override { return {{"dx", dx_}}; }
     float *getBeta(const T &t) override { return t == dx_ ? &beta_ : nullptr; }
     double flops() const override { return conv_flops(dx_, w_, dy_, cp_.group); }
-    double bytes() const override { return nbytes(dy_) + nbytes(w_) + nbytes(dx_) * (beta_ != 0 ? 2 : 1); }
+    double bytes() const override
+    {
+        return nbytes(dy_) + nbytes(w_) + nbytes(dx_) * ((beta_ != 0 ? 2 : 1) + (link_ ? 1 : 0));
+    }
 };
 
 struct ConvBwdFilter : public HipOperation {
@@ -908,6 +970,7 @@ struct BnBwd : public HipOperation {
     const T ds_, db_;
     int flags_;
     float dx_beta_ = 0, dz_beta_ = 0, ds_beta_ = 0, db_beta_ = 0;
+    std::shared_ptr<BnBwdLinkState> link_; // the last writer of dy leaves it masked, with its per-channel sums
     BnBwd(std::shared_ptr<BnTrain> fwd, T dy, T dx, T dz, T ds, T db, int flags)
       : HipOperation(flags ? "bnbwd.fused" : "bnbwd"), fwd_(fwd), dy_(dy), dx_(dx), dz_(dz), ds_(ds), db_(db), flags_(flags)
     {
@@ -919,6 +982,15 @@ struct BnBwd : public HipOperation {
         SagaTensorView vdz;
         if(dz_)
             vdz = dz_->view();
+        if(link_ && link_->valid) {
+            link_->valid = false;
+            chkSaga(saga_hip_bn_bwd_linked(&vx, &vdy, &vdx, (const float *)fwd_->s_->deviceMem(),
+                                           (const float *)fwd_->sm_->deviceMem(), (const float *)fwd_->sv_->deviceMem(),
+                                           (float *)ds_->deviceMem(), (float *)db_->deviceMem(), dx_beta_, ds_beta_,
+                                           (const float *)link_->partial->m_ptr, link_->rows, p.m_ctx->m_workspace.ptr(),
+                                           p.m_ctx->m_workspace.size(), S(p)));
+            return;
+        }
         // the bias lets the kernels rebuild the relu mask from x when there is no residual
         chkSaga(saga_hip_bn_bwd_ex(&vx, relu ? &vy : nullptr, &vdy, &vdx, dz_ ? &vdz : nullptr,
                                 (const float *)fwd_->s_->deviceMem(), (const float *)fwd_->b_->deviceMem(),
@@ -956,6 +1028,8 @@ struct BnBwd : public HipOperation {
     double bytes() const override
     {
         const double e = nbytes(dx_);
+        if(link_) // one pass: x and the masked gradient in, dx out
+            return e * (3 + (dx_beta_ != 0 ? 1 : 0));
         const bool reads_y = (flags_ & SAGA_BN_RELU) && (flags_ & SAGA_BN_ADD);
         if(reads_y && dz_ && dz_beta_ == 0) // pass 1: x, y (or its 1-bit mask), dy -> dz ; pass 2: x, dz -> dx
             return e * ((fwd_->mask_ ? 6.0625 : 7) + (dx_beta_ != 0 ? 1 : 0));
@@ -975,6 +1049,54 @@ struct BnBwd : public HipOperation {
         return nullptr;
     }
 };
+
+} // namespace
+
+// Training programs: where the gradient of a batch norm's (+ relu) output is written last by a convolution's
+// backward data and read by nobody but the norm's backward, that convolution masks the gradient and sums it
+// per channel on the way out, and the norm's backward starts from those sums.
+void link_bn_backward(HipProgram &p, HipOps &ops)
+{
+    if(getenv("SAGA_HIP_NO_BNBWD_LINK"))
+        return;
+    for(size_t ib = 0; ib < ops.size(); ib++) {
+        auto *bn = dynamic_cast<BnBwd *>(ops[ib].get());
+        if(!bn || bn->link_ || (bn->flags_ & SAGA_BN_ADD) || bn->dz_)
+            continue;
+        const T &g = bn->dy_, &x = bn->fwd_->x_;
+        if(g->m_data_type != Tensor::DataType::HALF || x->m_data_type != Tensor::DataType::HALF ||
+           x->m_storage == g->m_storage || x->m_dims.i64() != g->m_dims.i64())
+            continue;
+        const auto &ex = p.m_ctx->m_exported;
+        if(std::any_of(ex.begin(), ex.end(), [&](const auto &e) { return e == g->m_storage; }))
+            continue; // the host may look at the unmasked gradient
+        ssize_t last_writer = -1;
+        bool clean = true;
+        for(size_t i = 0; i < ops.size() && clean; i++) {
+            if(i == ib)
+                continue;
+            for(const auto &o : ops[i]->listOutputs())
+                if(o.second->m_storage == g->m_storage) {
+                    if(i > ib || o.second != g)
+                        clean = false;
+                    last_writer = (ssize_t)i;
+                }
+            for(const auto &in : ops[i]->listInputs())
+                if(in.second->m_storage == g->m_storage)
+                    clean = false;
+        }
+        if(!clean || last_writer < 0)
+            continue;
+        auto *conv = dynamic_cast<ConvBwdData *>(ops[last_writer].get());
+        if(!conv || conv->dx_ != g)
+            continue;
+        bn->link_ = conv->linkBnBwd(x, bn->fwd_->s_, bn->fwd_->b_, bn->fwd_->sm_, bn->fwd_->sv_, bn->flags_ & SAGA_BN_RELU);
+        if(bn->link_)
+            bn->m_kind = "bnbwd.linked";
+    }
+}
+
+namespace {
 
 bool single_consumer(const Nodes &nodes, const std::shared_ptr<Tensor> &t);
 

@@ -592,6 +592,8 @@ void HipProgram::finalize()
     m_opt.clear();
 
     eliminateDeadOps();
+    if(m_pt == ProgramType::TRAINING)
+        link_bn_backward(*this, m_ops);
 
     m_ctx->m_workspace.alloc();
     m_ctx->m_programs.push_back(this);

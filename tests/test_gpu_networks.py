@@ -237,6 +237,45 @@ def test_resnet50_training_fp16():
                                "s4_2-bn-2-s"])
 
 
+def test_resnet50_training_links_bn_backward_to_convolutions(monkeypatch):
+    """In a training program the backward data of the convolution that consumes relu(bn(x)) does the first pass of
+    that norm's backward: 32 of ResNet-50's 53 norms qualify (the two inner ones of each of the 16 bottlenecks,
+    stride-2 3x3 convolutions included), and the 22 of them where it pays (not at 64 channels, not at 128 under a
+    1x1 filter) are linked unless all are asked for; with the link switched off the same program gives the same
+    gradients."""
+    names = ["s1-conv-w", "s2_1-conv-1-w", "s3_1-conv-2-w", "s4_2-bn-1-s", "s4_2-bn-2-b", "s5_3-conv-1-w"]
+    grads = {}
+    for link in ("all", True, False):
+        if link == "all":
+            monkeypatch.setenv("SAGA_HIP_BNBWD_LINK_ALL", "1")
+        else:
+            monkeypatch.delenv("SAGA_HIP_BNBWD_LINK_ALL", raising=False)
+        if not link:
+            monkeypatch.setenv("SAGA_HIP_NO_BNBWD_LINK", "1")
+        net = N.resnet50(4, image=64)
+        x, labels = inputs(net, 5)
+        ctx = S.Context()
+        g, t = N.build_graph(net, x)
+        p = ctx.create_program(g, net.batch, training=True, learning_rate=1e-4, initial_loss_scale=1024.0)
+        ctx.resolve(t["labels"]).write(labels)
+        dev_grads = {k: ctx.resolve(t[k].grad()) for k in names}
+        p.set_profiling(True)
+        p.run(1)
+        kinds = {r["kind"]: r["launches"] for r in p.profile()}
+        print(" link", link, {k: v for k, v in kinds.items() if "bn" in k})
+        if link:
+            want = 32 if link == "all" else 22
+            assert kinds.get("convbwddata.bn") == want and kinds.get("bnbwd.linked") == want
+        else:
+            assert "convbwddata.bn" not in kinds and "bnbwd.linked" not in kinds
+        grads[link] = {k: dev_grads[k].read().astype(np.float32) for k in names}
+    for k in names:
+        for link in ("all", True):
+            e = rel_err(grads[link][k], grads[False][k])
+            print(f"  grad {k}: linked ({link}) against unlinked {e:.3e}")
+            assert e <= 1e-2, (k, e)  # fp16 rounding differences grown through up to 50 layers; the parity bar is 2e-2
+
+
 def test_unet_training_fp16():
     """Config 5 reduced (batch 2, 32x32, narrower): transposed convs and concat-as-strided-outputs,
     forward + backward + Adam.  The per-pixel head is exercised through a global pooled classifier."""

@@ -350,6 +350,141 @@ def test_bias_bwd_large(shape, padc, dtype):
     assert np.abs(got - want).max() <= 2e-6 * scale, "bias bwd large"
 
 
+BNBWD_LINK_CASES = [
+    # N, C (norm channels = dx channels), H, W, K (dy channels), R, pad, stride, relu, beta, channel pad of dx / x
+    (2, 64, 14, 14, 64, 3, 1, 1, True, 0.0, 0),     # 3x3 of a bottleneck, 256x64 tile
+    (3, 160, 9, 10, 32, 1, 0, 1, True, 0.0, 0),     # 1x1, 160 channels: two block columns, the second ragged
+    (2, 128, 13, 13, 24, 3, 1, 2, True, 0.0, 8),    # stride 2: four residue classes, padded rows
+    (2, 128, 13, 13, 24, 3, 1, 2, True, 1.0, 0),    # stride 2 accumulating onto an earlier writer
+    (2, 64, 12, 12, 64, 1, 0, 2, False, 0.0, 0),    # 1x1 stride 2: three classes get no tap and are zero-filled
+    (6, 64, 7, 7, 136, 3, 1, 1, False, 1.0, 0),     # no relu, beta 1, 7x7 images
+    (2, 64, 56, 56, 64, 3, 1, 1, True, 0.0, 0),     # many block rows
+    (5, 512, 7, 7, 128, 1, 0, 1, True, 0.0, 0),     # at most one block per CU: the kernel with producer wavefronts
+    (11, 256, 56, 56, 64, 1, 0, 1, True, 0.0, 0),   # more than 256 blocks of 256x128
+]
+
+
+@pytest.mark.parametrize("case", BNBWD_LINK_CASES)
+def test_conv_bwd_data_linked_to_bn_backward(case):
+    """saga_hip_conv2d_bwd_data_bnbwd + saga_hip_bn_bwd_linked against the two separate entry points
+    (saga_hip_conv2d_bwd_data, saga_hip_bn_bwd_ex) and the oracle: the stored gradient is the unlinked one
+    masked by the norm's relu, bit for bit; the partial sums are its per-channel sums; dx, ds, db agree."""
+    N, Cc, H, W, Kk, R, pad, stride, relu, beta, padc = case
+    dtype = torch.float16
+    rng = np.random.default_rng(Cc * 11 + Kk + R)
+    L = K.lib()
+    # the norm's forward on the device: its own statistics and output define the mask
+    x = rnd(rng, N, Cc, H, W, dtype=dtype) * 1.5 + 0.5
+    x = x.astype(np.float16).astype(np.float32)
+    s, b, m, v = _bn_params(rng, Cc)
+    flags = K.BN_RELU if relu else 0
+    xd, yd = dev(x, dtype, "nhwc", padc), dev(np.zeros_like(x), dtype, "nhwc")
+    sd, bd, md, vd = (dev(t) for t in (s, b, m, v))
+    sm, sv = dev(np.zeros(Cc, np.float32)), dev(np.zeros(Cc, np.float32))
+    wsb = K.bn_workspace(xd)
+    K.check(L.saga_hip_bn_train_fwd(C.byref(K.view(xd)), None, C.byref(K.view(yd)), K.ptr(sd), K.ptr(bd), K.ptr(md),
+                                    K.ptr(vd), K.ptr(sm), K.ptr(sv), 1e-5, 0.1, flags, K.ptr(wsb), wsb.numel(), S()))
+    keep = host(yd) > 0 if relu else np.ones_like(x, bool)
+    # the convolution whose backward data produces the gradient of y
+    P, Q = ref.conv_out(H, R, pad, stride), ref.conv_out(W, R, pad, stride)
+    w = rnd(rng, Kk, Cc, R, R, dtype=dtype, scale=(2.0 / (Kk * R * R)) ** 0.5)
+    dy = rnd(rng, N, Kk, P, Q, dtype=dtype)
+    old = rnd(rng, N, Cc, H, W, dtype=dtype)
+    wd, dyd = dev(w, dtype, "nhwc"), dev(dy, dtype, "nhwc")
+    ga, gb = dev(old, dtype, "nhwc", padc), dev(old, dtype, "nhwc", padc)
+    p = K.ConvParams(pad, stride, 1, 1)
+    vdy, vw, va, vb, vx = K.view(dyd), K.view(wd), K.view(ga), K.view(gb), K.view(xd)
+    wsz = L.saga_hip_conv2d_workspace_size(K.CONV_BWD_DATA, C.byref(va), C.byref(vw), C.byref(vdy), C.byref(p))
+    ws = torch.empty(max(wsz, 16), dtype=torch.uint8, device="cuda")
+    # unlinked
+    K.check(L.saga_hip_conv2d_bwd_data(C.byref(vdy), C.byref(vw), C.byref(va), C.byref(p), 1.0, beta, K.ptr(ws),
+                                       ws.numel(), S()))
+    g_ref = ref.round_half(ref.conv2d_bwd_data(dy, w, x.shape, pad, stride) + beta * old)
+    assert_close(host(ga), g_ref, dtype, "unlinked gradient")
+    dxa = dev(np.zeros_like(x), dtype, "nhwc")
+    dsa, dba = dev(np.zeros(Cc, np.float32)), dev(np.zeros(Cc, np.float32))
+    K.check(L.saga_hip_bn_bwd_ex(C.byref(vx), None, C.byref(va), C.byref(K.view(dxa)), None, K.ptr(sd),
+                                 K.ptr(bd), K.ptr(sm), K.ptr(sv), K.ptr(dsa), K.ptr(dba), 0.0, 0.0, 0.0, flags, None,
+                                 K.ptr(wsb), wsb.numel(), S()))
+    # linked
+    nbytes = L.saga_hip_conv2d_bwd_data_bnbwd_size(C.byref(vdy), C.byref(vw), C.byref(vb), C.byref(p))
+    assert nbytes > 0
+    partial = torch.full((nbytes // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    link = K.BnBwdLink(C.pointer(vx), K.ptr(sd), K.ptr(bd), K.ptr(sm), K.ptr(sv), flags, 0, K.ptr(partial), nbytes)
+    K.check(L.saga_hip_conv2d_bwd_data_bnbwd(C.byref(vdy), C.byref(vw), None, C.byref(vb), C.byref(p), 1.0, beta,
+                                             K.ptr(ws), ws.numel(), C.byref(link), S()))
+    rows = link.partial_rows
+    assert 0 < rows * Cc * 2 * 4 <= nbytes
+    g_masked = np.where(keep, host(ga), 0.0)
+    np.testing.assert_array_equal(host(gb), g_masked)
+    got = host(partial)[: rows * Cc * 2].reshape(rows, Cc, 2).astype(np.float64)
+    assert np.isfinite(got).all(), "a partial row was not written"
+    got = got.sum(0)
+    mean = host(sm).astype(np.float64).reshape(1, Cc, 1, 1)
+    gm = g_masked.astype(np.float64)
+    want0, want1 = gm.sum((0, 2, 3)), (gm * (x - mean)).sum((0, 2, 3))
+    np.testing.assert_allclose(got[:, 0], want0, rtol=1e-4, atol=1e-3 * max(1.0, np.abs(want0).max()))
+    np.testing.assert_allclose(got[:, 1], want1, rtol=1e-4, atol=1e-3 * max(1.0, np.abs(want1).max()))
+    dxb = dev(np.ones_like(x), dtype, "nhwc")
+    dsb, dbb = dev(np.ones(Cc, np.float32)), dev(np.ones(Cc, np.float32))
+    K.check(L.saga_hip_bn_bwd_linked(C.byref(vx), C.byref(vb), C.byref(K.view(dxb)), K.ptr(sd), K.ptr(sm), K.ptr(sv),
+                                     K.ptr(dsb), K.ptr(dbb), 0.0, 0.0, K.ptr(partial), rows, K.ptr(wsb), wsb.numel(),
+                                     S()))
+    dx_ref, ds_ref, db_ref = ref.bn_bwd(x, g_masked, s, host(sm), host(sv))
+    for what, got_d, want_d in (("linked", dxb, dx_ref), ("unlinked", dxa, dx_ref)):
+        assert_close(host(got_d), want_d, dtype, f"bn dx ({what})")
+    assert_close(host(dxb), host(dxa), dtype, "bn dx linked against unlinked", 2e-3)
+    assert_close(host(dsb), ds_ref, torch.float32, "bn ds", 5e-3)
+    assert_close(host(dbb), db_ref, torch.float32, "bn db", 5e-3)
+    assert_close(host(dsb), host(dsa), torch.float32, "bn ds linked against unlinked", 1e-4)
+    assert_close(host(dbb), host(dba), torch.float32, "bn db linked against unlinked", 1e-4)
+    # accumulation of the parameter gradients and of dx
+    K.check(L.saga_hip_bn_bwd_linked(C.byref(vx), C.byref(vb), C.byref(K.view(dxb)), K.ptr(sd), K.ptr(sm), K.ptr(sv),
+                                     K.ptr(dsb), K.ptr(dbb), 1.0, 1.0, K.ptr(partial), rows, K.ptr(wsb), wsb.numel(),
+                                     S()))
+    assert_close(host(dxb), 2 * dx_ref, dtype, "bn dx (beta 1)")
+    assert_close(host(dsb), 2 * ds_ref, torch.float32, "bn ds (beta 1)", 5e-3)
+
+
+def test_conv_bwd_data_bn_link_rejections():
+    """Outside the pipelined fp16 channels-last path the linked entry point says so and leaves dx alone."""
+    L = K.lib()
+    rng = np.random.default_rng(5)
+    dtype = torch.float16
+
+    def attempt(Cc, layout, xdtype=torch.float16, dil=1, size=None):
+        x = rnd(rng, 2, Cc, 8, 8, dtype=dtype)
+        w = rnd(rng, 16, Cc, 3, 3, dtype=dtype)
+        Pq = ref.conv_out(8, 3, dil, 1, dil)
+        dyd, wd = dev(rnd(rng, 2, 16, Pq, Pq, dtype=dtype), dtype, layout), w_dev(w, dtype, layout)
+        xd, gd = dev(x, xdtype, layout), dev(np.full_like(x, 3.0), dtype, layout)
+        par = [dev(np.ones(Cc, np.float32)) for _ in range(4)]
+        p = K.ConvParams(dil, 1, dil, 1)
+        vdy, vw, vg, vx = K.view(dyd), K.view(wd), K.view(gd), K.view(xd)
+        nbytes = L.saga_hip_conv2d_bwd_data_bnbwd_size(C.byref(vdy), C.byref(vw), C.byref(vg), C.byref(p))
+        partial = torch.zeros(max(1, nbytes if size is None else size) // 4 + 1, dtype=torch.float32, device="cuda")
+        link = K.BnBwdLink(C.pointer(vx), *(K.ptr(t) for t in par), K.BN_RELU, 0, K.ptr(partial),
+                           nbytes if size is None else size)
+        ws = torch.empty(1 << 20, dtype=torch.uint8, device="cuda")
+        rc = L.saga_hip_conv2d_bwd_data_bnbwd(C.byref(vdy), C.byref(vw), None, C.byref(vg), C.byref(p), 1.0, 0.0,
+                                              K.ptr(ws), ws.numel(), C.byref(link), S())
+        torch.cuda.synchronize()
+        return rc, nbytes, host(gd)
+
+    rc, nbytes, g = attempt(20, "nhwc")            # channel count no multiple of 8
+    assert (rc, nbytes) == (-3, 0) and (g == 3.0).all()
+    rc, nbytes, g = attempt(16, "nchw")            # channels-first
+    assert (rc, nbytes) == (-3, 0) and (g == 3.0).all()
+    rc, nbytes, g = attempt(16, "nhwc", dil=2)     # dilated
+    assert (rc, nbytes) == (-3, 0) and (g == 3.0).all()
+    rc, nbytes, g = attempt(16, "nhwc", xdtype=torch.float32)  # the norm's input in another type
+    assert rc == -3 and (g == 3.0).all()
+    rc, nbytes, g = attempt(16, "nhwc", size=64)   # partial buffer too small
+    assert rc == -4 and nbytes > 64 and (g == 3.0).all()
+    rc, nbytes, g = attempt(16, "nhwc")
+    assert rc == 0 and not (g == 3.0).all()
+
+
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("tA,tB", [(0, 0), (0, 1), (1, 0), (1, 1)])
 def test_gemm(tA, tB, dtype):
