@@ -49,7 +49,7 @@ MEASURED_HBM_BYTES_PER_LAUNCH = {
     "conv": 275571868,
     "batchnorm": 460542165,
 }
-TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE snapshot at commit 92e6e3e (profiles/resnet50_b256_fp16_hbm_counters.txt)"
+TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE snapshot at commit a71b442 (profiles/resnet50_b256_fp16_hbm_counters.txt)"
 
 
 def by_kind(rows):
