@@ -322,20 +322,48 @@ __device__ __forceinline__ void load_row32(const half_t *row, bool ok, int nb, i
     }
 }
 
-// One step of a halving exchange over n live values per lane: the lane with bit m set keeps
-// the upper half, its partner (lane ^ m) the lower half, and each adds what the other held of
-// its half.  n is a template parameter so that every array index is a constant and the
-// arrays stay in registers.
-template <int n, int NV>
-__device__ __forceinline__ void halve_exchange(float (&a)[NV], float (&b)[NV], int lane, int m)
+// One step of a halving exchange over n live values per lane: the lane with bit M set keeps
+// the upper half, its partner the lower half, and each adds what the other held of its half.
+// n is a template parameter so that every array index is a constant and the arrays stay in
+// registers.  The partner only has to differ in bit M and agree in the bits above it (the bits
+// below are exchanged by the later steps), which lets every step run in the vector ALU instead of
+// going through the LDS crossbar (ds_bpermute):
+//   M = 16: v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even rows
+//           of the second, after which a lane's two results are its own and its partner's value of the
+//           half it keeps (the results pass through an opaque statement: hipcc 7.2 otherwise folds the
+//           sum of the two results of one swap into twice the first);
+//   M = 8, 4: the partner is the mirror lane of the row of 16 / of the half row of 8 (DPP row_mirror,
+//           row_half_mirror); M = 2, 1: the lane two / one away inside the quad (DPP quad_perm).
+template <int CTRL> __device__ __forceinline__ float dpp_read(float v)
 {
-    const bool up = lane & m;
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+template <int n, int M, int NV>
+__device__ __forceinline__ void halve_exchange(float (&a)[NV], float (&b)[NV], int lane)
+{
+    static_assert(M == 16 || M == 8 || M == 4 || M == 2 || M == 1, "partner distance");
+    if constexpr(M == 16) {
 #pragma unroll
-    for(int k = 0; k < n / 2; k++) {
-        const float ka = up ? a[k + n / 2] : a[k], sa = up ? a[k] : a[k + n / 2];
-        const float kb = up ? b[k + n / 2] : b[k], sb = up ? b[k] : b[k + n / 2];
-        a[k] = ka + __shfl_xor(sa, m, 64);
-        b[k] = kb + __shfl_xor(sb, m, 64);
+        for(int k = 0; k < n / 2; k++) {
+            const auto ra = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, a[k]),
+                                                             __builtin_bit_cast(unsigned, a[k + n / 2]), false, false);
+            const auto rb = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, b[k]),
+                                                             __builtin_bit_cast(unsigned, b[k + n / 2]), false, false);
+            unsigned a0 = ra[0], a1 = ra[1], b0 = rb[0], b1 = rb[1];
+            asm volatile("" : "+v"(a0), "+v"(a1), "+v"(b0), "+v"(b1));
+            a[k] = __builtin_bit_cast(float, a0) + __builtin_bit_cast(float, a1);
+            b[k] = __builtin_bit_cast(float, b0) + __builtin_bit_cast(float, b1);
+        }
+    } else {
+        constexpr int CTRL = M == 8 ? 0x140 : M == 4 ? 0x141 : M == 2 ? 0x4e : 0xb1;
+        const bool up = lane & M;
+#pragma unroll
+        for(int k = 0; k < n / 2; k++) {
+            const float ka = up ? a[k + n / 2] : a[k], sa = up ? a[k] : a[k + n / 2];
+            const float kb = up ? b[k + n / 2] : b[k], sb = up ? b[k] : b[k + n / 2];
+            a[k] = ka + dpp_read<CTRL>(sa);
+            b[k] = kb + dpp_read<CTRL>(sb);
+        }
     }
 }
 
@@ -484,18 +512,18 @@ __device__ __forceinline__ void gather_epilogue(const GatherArgs &g, float16_t (
                     qv[j * 16 + v] = q;
                 }
             if constexpr(NV == 32) {
-                halve_exchange<32>(sv, qv, lane, 16);
-                halve_exchange<16>(sv, qv, lane, 8);
-                halve_exchange<8>(sv, qv, lane, 4);
-                halve_exchange<4>(sv, qv, lane, 2);
-                halve_exchange<2>(sv, qv, lane, 1);
+                halve_exchange<32, 16>(sv, qv, lane);
+                halve_exchange<16, 8>(sv, qv, lane);
+                halve_exchange<8, 4>(sv, qv, lane);
+                halve_exchange<4, 2>(sv, qv, lane);
+                halve_exchange<2, 1>(sv, qv, lane);
             } else {
-                halve_exchange<16>(sv, qv, lane, 16);
-                halve_exchange<8>(sv, qv, lane, 8);
-                halve_exchange<4>(sv, qv, lane, 4);
-                halve_exchange<2>(sv, qv, lane, 2);
-                sv[0] += __shfl_xor(sv[0], 1, 64);
-                qv[0] += __shfl_xor(qv[0], 1, 64);
+                halve_exchange<16, 16>(sv, qv, lane);
+                halve_exchange<8, 8>(sv, qv, lane);
+                halve_exchange<4, 4>(sv, qv, lane);
+                halve_exchange<2, 2>(sv, qv, lane);
+                sv[0] += dpp_read<0xb1>(sv[0]);
+                qv[0] += dpp_read<0xb1>(qv[0]);
             }
             const int idx = NV == 32 ? (lane & 31) : (lane & 31) >> 1;
             const int chl = 32 * (idx >> 4) + 8 * ((idx & 15) >> 2) + 4 * hi + (idx & 3); // channel inside the wave tile
@@ -705,11 +733,11 @@ __device__ __forceinline__ void gather_epilogue_bnbwd(const GatherArgs &g, float
         if(i == TM - 1) {
             // lanes of a half-wave hold different pixels of the same 16 channels: after the remaining halving
             // exchanges each pair of lanes holds one channel's total over the wave tile's rows
-            halve_exchange<8>(sv, qv, lane, 8);
-            halve_exchange<4>(sv, qv, lane, 4);
-            halve_exchange<2>(sv, qv, lane, 2);
-            sres[j] = sv[0] + __shfl_xor(sv[0], 1, 64);
-            qres[j] = qv[0] + __shfl_xor(qv[0], 1, 64);
+            halve_exchange<8, 8>(sv, qv, lane);
+            halve_exchange<4, 4>(sv, qv, lane);
+            halve_exchange<2, 2>(sv, qv, lane);
+            sres[j] = sv[0] + dpp_read<0xb1>(sv[0]);
+            qres[j] = qv[0] + dpp_read<0xb1>(qv[0]);
         }
         __builtin_amdgcn_sched_barrier(0); // one sub-tile at a time: interleaving them costs registers
     }
