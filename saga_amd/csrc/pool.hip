@@ -490,6 +490,70 @@ __global__ void __launch_bounds__(256)
     PV<T, VN>::store(out, acc);
 }
 
+// The same for 3x3 windows at stride 2, four input positions per thread.  In padded coordinates (hh = h + pad)
+// window p covers rows 2p .. 2p+2, so the input rows 2a-1 and 2a are reached by the windows a-1 and a only, and
+// the 2x2 patch (2a-1 .. 2a) x (2b-1 .. 2b) by the four windows (a-1 .. a) x (b-1 .. b): four gradient vectors
+// and four code vectors are loaded for four results (the kernel above loads four of each per result).  Which
+// window position a patch element is for each window is fixed:
+//   (2a-1, 2b-1): position 4 of window (a-1, b-1)
+//   (2a-1, 2b)  : 5 of (a-1, b-1), 3 of (a-1, b)
+//   (2a,   2b-1): 7 of (a-1, b-1), 1 of (a, b-1)
+//   (2a,   2b)  : 8 of (a-1, b-1), 6 of (a-1, b), 2 of (a, b-1), 0 of (a, b)
+// blockIdx.z = sample, blockIdx.y = a, threadIdx.x = channel vector, threadIdx.y (+ blockIdx.x) = b
+template <typename T, int VN>
+__global__ void __launch_bounds__(256)
+    maxpool_bwd_codes_3x3s2_k(const uint8_t *__restrict__ codes, DView dy, DView dx, int pad, float beta)
+{
+    const int C = dx.d[1], H = dx.d[2], W = dx.d[3], P = dy.d[2], Q = dy.d[3];
+    const int n = blockIdx.z, a = blockIdx.y;
+    const int b = blockIdx.x * blockDim.y + threadIdx.y;
+    const int c = threadIdx.x * VN;
+    if(c >= C || 2 * b - 1 - pad >= W)
+        return;
+    float g[4][VN];
+    typename CodeVec<VN>::type cd[4];
+    bool okw[4];
+#pragma unroll
+    for(int e = 0; e < 4; e++) {
+        const int p = a - 1 + (e >> 1), q = b - 1 + (e & 1);
+        okw[e] = p >= 0 && p < P && q >= 0 && q < Q;
+        const int pc = p < 0 ? 0 : p >= P ? P - 1 : p, qc = q < 0 ? 0 : q >= Q ? Q - 1 : q;
+        PV<T, VN>::load((const T *)dy.ptr + off4(dy, n, c, pc, qc), g[e]);
+        cd[e] = *(const typename CodeVec<VN>::type *)(codes + ((((size_t)n * P + pc) * Q + qc) * C + c));
+    }
+    auto code = [&](int e, int j) -> unsigned {
+        if constexpr(VN == 8)
+            return (cd[e][j >> 2] >> (8 * (j & 3))) & 255u;
+        else
+            return (cd[e] >> (8 * j)) & 255u;
+    };
+    // term(e, k, j): what window e gives the position it calls k
+    auto term = [&](int e, unsigned k, int j) { return (okw[e] && code(e, j) == k) ? g[e][j] : 0.0f; };
+    float out[4][VN];
+#pragma unroll
+    for(int j = 0; j < VN; j++) {
+        out[0][j] = term(0, 4, j);
+        out[1][j] = term(0, 5, j) + term(1, 3, j);
+        out[2][j] = term(0, 7, j) + term(2, 1, j);
+        out[3][j] = term(0, 8, j) + term(1, 6, j) + term(2, 2, j) + term(3, 0, j);
+    }
+#pragma unroll
+    for(int e = 0; e < 4; e++) {
+        const int h = 2 * a - 1 + (e >> 1) - pad, w = 2 * b - 1 + (e & 1) - pad;
+        if(h < 0 || h >= H || w < 0 || w >= W)
+            continue;
+        T *o = (T *)dx.ptr + off4(dx, n, c, h, w);
+        if(beta != 0.0f) {
+            float old[VN];
+            PV<T, VN>::load(o, old);
+#pragma unroll
+            for(int j = 0; j < VN; j++)
+                out[e][j] += beta * old[j];
+        }
+        PV<T, VN>::store(o, out[e]);
+    }
+}
+
 static int vec_for(int dtype, std::initializer_list<const SagaTensorView *> vs)
 {
     const int vn = dtype == SAGA_HALF ? 8 : 4;
@@ -677,9 +741,20 @@ int saga_hip_maxpool_bwd_codes(const uint8_t *codes, const SagaTensorView *dy, c
         return SAGA_HIP_EUNSUPPORTED;
     const int vn = dx->dtype == SAGA_HALF ? 8 : 4;
     dim3 grid, block;
-    codes_launch_shape(dx->dims[1] / vn, dx->dims[3], dx->dims[2], dx->dims[0], grid, block);
     hipStream_t st = as_stream(stream);
     const DView dvdy = dview(dy), dvdx = dview(dx);
+    if(size == 3 && stride == 2) {
+        // patches (2a-1 .. 2a) x (2b-1 .. 2b) in padded coordinates: a = 0 .. (H - 1 + pad + 1) / 2
+        const int na = (dx->dims[2] + pad) / 2 + 1, nb = (dx->dims[3] + pad) / 2 + 1;
+        codes_launch_shape(dx->dims[1] / vn, nb, na, dx->dims[0], grid, block);
+        if(dx->dtype == SAGA_HALF)
+            maxpool_bwd_codes_3x3s2_k<half_t, 8><<<grid, block, 0, st>>>(codes, dvdy, dvdx, pad, beta);
+        else
+            maxpool_bwd_codes_3x3s2_k<float, 4><<<grid, block, 0, st>>>(codes, dvdy, dvdx, pad, beta);
+        SAGA_CHECK_LAUNCH();
+        return 0;
+    }
+    codes_launch_shape(dx->dims[1] / vn, dx->dims[3], dx->dims[2], dx->dims[0], grid, block);
 #define GO2(T, VN, K, S) maxpool_bwd_codes_k<T, VN, K, S><<<grid, block, 0, st>>>(codes, dvdy, dvdx, pad, beta)
 #define GO(T, VN)                                                                                              \
     do {                                                                                                       \

@@ -682,7 +682,7 @@ def test_pooling(k, pad, stride, H, layout, padc, dtype):
 
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("padc", [0, 8])
-@pytest.mark.parametrize("k,pad,stride,H", [(2, 0, 2, 8), (3, 1, 2, 9), (3, 1, 2, 12), (3, 1, 1, 6), (3, 0, 3, 10), (2, 1, 1, 5)])
+@pytest.mark.parametrize("k,pad,stride,H", [(2, 0, 2, 8), (3, 1, 2, 9), (3, 1, 2, 12), (3, 0, 2, 11), (3, 0, 2, 8), (3, 1, 1, 6), (3, 0, 3, 10), (2, 1, 1, 5)])
 def test_maxpool_with_position_codes(k, pad, stride, H, padc, dtype):
     """The training pair saga_hip_maxpool_fwd_codes / _bwd_codes on channels-last tensors (dense and
     with a wider channel pitch): y and the recorded first-maximum positions bit-exact against the
