@@ -195,6 +195,8 @@ struct HipOperation {
 struct HipProgram;
 // hip_ops.cpp: hands the first pass of a batch norm's backward to the convolution that writes its gradient
 void link_bn_backward(HipProgram &p, std::vector<std::shared_ptr<HipOperation>> &ops);
+// hip_ops.cpp: a strided 1x1 backward data that writes a fan-in gradient first is moved behind the last writer
+void reorder_sparse_first_writers(std::vector<std::shared_ptr<HipOperation>> &ops);
 
 struct HipProgramUnit {
     Nodes m_transformed;

@@ -1052,6 +1052,63 @@ struct BnBwd : public HipOperation {
 
 } // namespace
 
+// Gradients that fan in are summed by letting every writer after the first accumulate.  A 1x1 backward data at
+// stride 2 (the projection of a downsampling residual block) reaches one output pixel in four: as the FIRST
+// writer it has to fill the other three quarters with zeros, and the dense writer after it then reads all of
+// that back to add to it; as the LAST writer it adds to its own quarter and touches nothing else.  Where such
+// an operation writes first and other operations write the same tensor later, it is moved behind the last of
+// them - nothing in between reads the tensor (it is incomplete until then) or writes what the moved operation
+// reads.  Runs before the accumulation factors are assigned.
+void reorder_sparse_first_writers(HipOps &ops)
+{
+    if(getenv("SAGA_HIP_NO_WRITER_REORDER"))
+        return;
+    for(size_t i = 0; i < ops.size(); i++) {
+        auto *conv = dynamic_cast<ConvBwdData *>(ops[i].get());
+        if(!conv || conv->cp_.stride < 2 || ((int)conv->w_->m_dims[2] >= conv->cp_.stride && (int)conv->w_->m_dims[3] >= conv->cp_.stride))
+            continue;
+        const T &t = conv->dx_;
+        bool first = true;
+        for(size_t k = 0; k < i && first; k++)
+            for(const auto &o : ops[k]->listOutputs())
+                if(o.second->m_storage == t->m_storage)
+                    first = false;
+        if(!first)
+            continue;
+        ssize_t last = -1;
+        bool ok = true;
+        for(size_t k = i + 1; k < ops.size() && ok; k++) {
+            bool writes = false;
+            for(const auto &o : ops[k]->listOutputs())
+                if(o.second->m_storage == t->m_storage) {
+                    // every later writer must be able to go first or to accumulate, on this very tensor
+                    if(o.second != t || !ops[k]->getBeta(o.second))
+                        ok = false;
+                    writes = true;
+                }
+            if(writes)
+                last = (ssize_t)k;
+        }
+        if(!ok || last < 0)
+            continue;
+        for(size_t k = i + 1; k <= (size_t)last && ok; k++) {
+            for(const auto &in : ops[k]->listInputs())
+                if(in.second->m_storage == t->m_storage)
+                    ok = false; // somebody reads the sum before it is complete: leave the order alone
+            for(const auto &o : ops[k]->listOutputs())
+                for(const auto &in : conv->listInputs())
+                    if(o.second->m_storage == in.second->m_storage)
+                        ok = false;
+        }
+        if(!ok)
+            continue;
+        auto moved = ops[i];
+        ops.erase(ops.begin() + i);
+        ops.insert(ops.begin() + last, moved); // `last` shifted down by one: this is right behind it
+        i--;                                     // what slid into position i is looked at next
+    }
+}
+
 // Training programs: where the gradient of a batch norm's (+ relu) output is written last by a convolution's
 // backward data and read by nobody but the norm's backward, that convolution masks the gradient and sums it
 // per channel on the way out, and the norm's backward starts from those sums.

@@ -574,6 +574,8 @@ void HipProgram::finalize()
     // are added inside the convolution / GEMM epilogue (reference: src/cuda/cuda_program.cpp:429-453).
     // An accumulating writer reads its output, so the dead-op pass below keeps the first writer
     // whenever it keeps a later one.
+    if(m_pt == ProgramType::TRAINING)
+        reorder_sparse_first_writers(m_ops);
     std::set<HipTensor *> written;
     for(auto &op : m_ops) {
         for(auto &o : op->listOutputs()) {

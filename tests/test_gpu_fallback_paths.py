@@ -4,7 +4,7 @@ The kernel library reads its switches once per process, so every case runs a sel
 test files in a child process with the switch set: the register-staged fp16 convolution kernels, the
 direct (one output per lane) convolutions, the table-driven fp32 convolutions, batch-norm backward with
 the relu mask read from y, and the engine without relu bit masks / position codes / arena / batched
-filter transposes / batch-norm backward link."""
+filter transposes / batch-norm backward link / reordering of fan-in writers."""
 import os
 import subprocess
 import sys
@@ -27,6 +27,7 @@ CASES = [
     ("SAGA_HIP_NO_ARENA", "1", ["tests/test_gpu_networks.py", "-k", "training"]),
     ("SAGA_HIP_NO_BATCHED_TRANSPOSE", "1", ["tests/test_gpu_networks.py", "-k", "training and not links"]),
     ("SAGA_HIP_NO_BNBWD_LINK", "1", ["tests/test_gpu_networks.py", "-k", "training and not links"]),
+    ("SAGA_HIP_NO_WRITER_REORDER", "1", ["tests/test_gpu_networks.py", "-k", "training"]),
 ]
 
 
