@@ -1697,7 +1697,7 @@ struct FilterPlan {
 };
 
 // big_ok: the caller will run the pipelined kernel, the only one that has the large tiles
-static FilterPlan plan_filter(const ConvGeom &g, bool big_ok = true)
+static FilterPlan plan_filter(const ConvGeom &g, bool big_ok = true, bool thin = false)
 {
     FilterPlan p;
     const int RSC = g.R * g.S * g.C;
@@ -1721,6 +1721,9 @@ static FilterPlan plan_filter(const ConvGeom &g, bool big_ok = true)
         target = 512;
     } else if(big_ok && g.K <= 64 && RSC >= 512 && g.R * g.S > 1 && forced != 128) {
         p.bn = 256; // 64x256 on four wavefronts with two stages, four blocks per CU (measured 17 % faster)
+        target = 1024;
+    } else if(thin && g.K <= 64 && RSC > 128 && RSC <= 256 && forced != 128) {
+        p.bn = 256; // the stem: all 7 x 32 virtual channels in one tile, so dy (the large operand) is read once
         target = 1024;
     }
     p.tiles_k = (g.K + p.bm - 1) / p.bm;
@@ -2098,7 +2101,7 @@ size_t conv_mfma_workspace(int kind, const SagaTensorView *x, const SagaTensorVi
             ConvGeom gv = g;
             gv.C = 32;
             gv.S = 1;
-            const FilterPlan pv = plan_filter(gv);
+            const FilterPlan pv = plan_filter(gv, true, true);
             need = std::max(need, tg.x4_bytes + (size_t)pv.splits * g.K * g.R * 32 * sizeof(float));
         }
         return need + 256;
@@ -2300,7 +2303,7 @@ int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, cons
         ConvGeom gv = g;
         gv.C = 32;
         gv.S = 1;
-        const FilterPlan p = plan_filter(gv);
+        const FilterPlan p = plan_filter(gv, true, true);
         const size_t need = tg.x4_bytes + (size_t)p.splits * g.K * g.R * 32 * sizeof(float);
         const int64_t yb = ((ldy.rows - 1) * ldy.pitch + ldy.C) * 2;
         if(!ws || ws_bytes < need || !aligned16(ws))
@@ -2327,6 +2330,8 @@ int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, cons
         constexpr int ST = 3, FNW = 8;
         if(p.bm == 128)
             conv_bwd_filter_dma<128, 128, ST, FNW><<<blocks, 64 * FNW, ST * BK * 512, st>>>(a, (unsigned)(px * 8), (unsigned)yb);
+        else if(p.bn == 256)
+            conv_bwd_filter_dma<64, 256, 2, 4><<<blocks, 256, 2 * BK * 640, st>>>(a, (unsigned)(px * 8), (unsigned)yb);
         else
             conv_bwd_filter_dma<64, 128, ST, 4><<<blocks, 256, ST * BK * 384, st>>>(a, (unsigned)(px * 8), (unsigned)yb);
         SAGA_CHECK_LAUNCH();
