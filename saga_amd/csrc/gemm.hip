@@ -138,7 +138,11 @@ __global__ void __launch_bounds__(256)
 // halves.  kcontig: element (row, k) is at base[row*ld + k], else at base[k*ld + row].
 // Every lane moves 8 elements that are contiguous in memory, with one 16-byte load when the
 // run is in range and aligned.
-constexpr int GLDK = 40;
+// An iteration of the main loop takes GBK = 128 reduction steps (four 32-wide pieces per operand, eight 16-byte
+// loads per lane in flight): with 32 the loop of a tall reduction (fc 2048 -> 1000 at batch 256: 64 blocks of 64
+// iterations) paid one trip to memory per iteration and took 69 us; LDS rows are GLDK halves.
+constexpr int GBK = 128;
+constexpr int GLDK = GBK + 8;
 
 __device__ __forceinline__ void gemm_stage(half_t (*dst)[GLDK], const half_t *__restrict__ base, int ld, bool kcontig,
                                            int row0, int rows, int k0, int K, bool vec_ok, int tid)
@@ -188,18 +192,68 @@ __global__ void __launch_bounds__(256)
     for(int v = 0; v < 16; v++)
         acc[v] = 0.0f;
     const int frow = lane & 31, fk = (lane >> 5) * 8;
-    const int KT = (K + 31) / 32;
-    gemm_stage(As[0], A, lda, !tA, m0, M, 0, K, a_vec, tid);
-    gemm_stage(Bs[0], B, ldb, tB, n0, N, 0, K, b_vec, tid);
+    const int KT = (K + GBK - 1) / GBK;
+    // Vector path (both operands 16-byte loadable): all eight loads of an iteration are issued before the first
+    // LDS write waits for one - branch-free, out-of-range runs read the operand's first bytes and are zeroed -
+    // so an iteration pays one trip to memory, not eight.
+    const bool fast = a_vec && b_vec;
+    auto fetch = [&](const half_t *__restrict__ base, int ld, bool kcontig, int row0, int rows, int k0, bool &ok) {
+        int gr, gk;
+        if(kcontig) {
+            gr = row0 + (tid >> 2); gk = k0 + (tid & 3) * 8;
+            ok = gr < rows && gk + 8 <= K;
+            return *(const half8_t *)(base + (ok ? (int64_t)gr * ld + gk : 0));
+        }
+        gk = k0 + (tid >> 3); gr = row0 + (tid & 7) * 8;
+        ok = gk < K && gr + 8 <= rows;
+        return *(const half8_t *)(base + (ok ? (int64_t)gk * ld + gr : 0));
+    };
+    auto put = [&](half_t(*dst)[GLDK], bool kcontig, half8_t v, bool ok) {
+        if(!ok)
+            v = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        if(kcontig) {
+            *(half8_t *)&dst[tid >> 2][(tid & 3) * 8] = v;
+        } else {
+#pragma unroll
+            for(int j = 0; j < 8; j++)
+                dst[(tid & 7) * 8 + j][tid >> 3] = v[j];
+        }
+    };
+    // a run that is only partly in range (K or the row count no multiple of 8) is rare: those tiles take the
+    // element-wise path of gemm_stage
+    auto partial = [&](int row0, int rows, int k0, bool kcontig) {
+        return kcontig ? (K % 8 != 0 && k0 + GBK > K) : (rows % 8 != 0 && row0 + 64 > rows);
+    };
+    auto stage = [&](int buf, int k0) {
+        if(fast && !partial(m0, M, k0, !tA) && !partial(n0, N, k0, tB)) {
+            half8_t va[GBK / 32], vb[GBK / 32];
+            bool oa[GBK / 32], ob[GBK / 32];
+#pragma unroll
+            for(int j = 0; j < GBK / 32; j++) {
+                va[j] = fetch(A, lda, !tA, m0, M, k0 + 32 * j, oa[j]);
+                vb[j] = fetch(B, ldb, tB, n0, N, k0 + 32 * j, ob[j]);
+            }
+#pragma unroll
+            for(int j = 0; j < GBK / 32; j++) {
+                put((half_t(*)[GLDK]) & As[buf][0][32 * j], !tA, va[j], oa[j]);
+                put((half_t(*)[GLDK]) & Bs[buf][0][32 * j], tB, vb[j], ob[j]);
+            }
+            return;
+        }
+#pragma unroll
+        for(int j = 0; j < GBK / 32; j++) {
+            gemm_stage((half_t(*)[GLDK]) & As[buf][0][32 * j], A, lda, !tA, m0, M, k0 + 32 * j, K, a_vec, tid);
+            gemm_stage((half_t(*)[GLDK]) & Bs[buf][0][32 * j], B, ldb, tB, n0, N, k0 + 32 * j, K, b_vec, tid);
+        }
+    };
+    stage(0, 0);
     for(int kt = 0; kt < KT; kt++) {
         __syncthreads();
         const int cur = kt & 1;
-        if(kt + 1 < KT) {
-            gemm_stage(As[cur ^ 1], A, lda, !tA, m0, M, (kt + 1) * 32, K, a_vec, tid);
-            gemm_stage(Bs[cur ^ 1], B, ldb, tB, n0, N, (kt + 1) * 32, K, b_vec, tid);
-        }
+        if(kt + 1 < KT)
+            stage(cur ^ 1, (kt + 1) * GBK);
 #pragma unroll
-        for(int kk = 0; kk < 2; kk++) {
+        for(int kk = 0; kk < GBK / 16; kk++) {
             const half8_t fa = *(const half8_t *)&As[cur][wm + frow][kk * 16 + fk];
             const half8_t fb = *(const half8_t *)&Bs[cur][wn + frow][kk * 16 + fk];
             acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fb, acc, 0, 0, 0);
