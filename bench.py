@@ -46,10 +46,10 @@ FAMILIES = {
 # lines, the per-kernel table and the commit the counters were taken at are in
 # profiles/resnet50_b256_fp16_hbm_counters.txt; they go stale when kernels change, hence the label.
 MEASURED_HBM_BYTES_PER_LAUNCH = {
-    "conv": 282601494,
-    "batchnorm": 439134997,
+    "conv": 275687193,
+    "batchnorm": 439128728,
 }
-TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE snapshot at commit a71b442 (profiles/resnet50_b256_fp16_hbm_counters.txt)"
+TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE snapshot at commit 4799a37 (profiles/resnet50_b256_fp16_hbm_counters.txt)"
 
 
 def by_kind(rows):
