@@ -179,3 +179,47 @@ def test_anomaly_detection_reports_a_planted_nan(where, monkeypatch, capfd):
     assert "*** Anomaly in tensor" in out and "(input)" in out
     if where == "weight":
         assert "s3_1-conv-2" in str(err.value) or "s3_1-conv-2" in out
+
+
+def test_sparse_first_writer_is_moved_behind_the_dense_one(monkeypatch, tmp_path):
+    """The gradient of a downsampling block's input has two writers: the projection's backward data (1x1 at
+    stride 2, one pixel in four) and the block's first convolution (dense).  In graph order the projection writes
+    first; the engine moves it behind the dense writer (three blocks in ResNet-50), which changes nothing but the
+    order of the two and the side that accumulates - same writers per tensor, same gradients."""
+    import re
+    writers, grads = {}, {}
+    names = ["s1-conv-w", "s3_1-conv-p-w", "s4_1-conv-1-w", "s5_1-bn-p-s"]
+    for reorder in (True, False):
+        if not reorder:
+            monkeypatch.setenv("SAGA_HIP_NO_WRITER_REORDER", "1")
+        net = N.resnet50(4, image=64)
+        rng = np.random.default_rng(11)
+        x = rng.standard_normal((4, 3, 64, 64)).astype(np.float32)
+        ctx = S.Context()
+        g, t = N.build_graph(net, x)
+        p = ctx.create_program(g, net.batch, training=True, learning_rate=1e-4, initial_loss_scale=1024.0)
+        ctx.resolve(t["labels"]).write(rng.integers(0, 1000, 4).astype(np.int32))
+        dev = {k: ctx.resolve(t[k].grad()) for k in names}
+        path = tmp_path / f"ops_{reorder}.txt"
+        p.dump(str(path), False)
+        w = {}
+        for line in open(path):
+            m = re.match(r"#\s*\d+: (\+?)dx:(T\d+) = convbwddata(?:\.bn)?\(w:(T\d+)", line)
+            if m:
+                w.setdefault(m.group(2), []).append((m.group(3), m.group(1) == "+"))
+        writers[reorder] = w
+        p.run(1)
+        grads[reorder] = {k: dev[k].read().astype(np.float32) for k in names}
+    on, off = writers[True], writers[False]
+    assert on.keys() == off.keys()
+    moved = [k for k in on if on[k] != off[k]]
+    assert len(moved) == 3, moved
+    for k in on:
+        assert sorted(v[0] for v in on[k]) == sorted(v[0] for v in off[k])          # the same writers
+    for k in moved:
+        assert [v[0] for v in on[k]] == [v[0] for v in off[k]][::-1]
+        assert [v[1] for v in on[k]] == [False, True] == [v[1] for v in off[k]]      # the first overwrites, the second adds
+    for k in names:
+        e = rel_err(grads[True][k], grads[False][k])
+        print(f"  grad {k}: reordered against graph order {e:.3e}")
+        assert e <= 1e-2, (k, e)
