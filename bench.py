@@ -7,7 +7,8 @@ Saga Graph/Context/Program boundary on the hip engine.
 
 Prints ONE JSON line.  `value` is training images/sec over exactly K timed steps with the
 input batch already resident in HBM; `infer_images_per_sec` is the inference program on the
-same weights.  `roofline` describes the kernel family that takes the most GPU time in the
+same weights (`roofline_infer`: its dominant kernel family, timed the same way).  `roofline` describes the
+kernel family that takes the most GPU time in the
 training step (the convolutions; HIP-event timing of every operation on the engine's stream, taken in a
 second pass of K steps so that the events do not sit inside the timed region), `roofline_hbm` the
 HBM-bound family with the most time (batch norm); `families` and `kernels` list every family and
@@ -34,7 +35,7 @@ CONV_KINDS = ("convfwd", "convbwddata", "convbwddata.bn", "convbwdfilter")
 # Operation kinds that share kernels and a roofline bound form a family; `roofline` describes the family with
 # the most GPU time in the training step.
 FAMILIES = {
-    "conv": ("convfwd", "convbwddata", "convbwddata.bn", "convbwdfilter"),
+    "conv": ("convfwd", "convfwd.bn", "convbwddata", "convbwddata.bn", "convbwdfilter"),
     "batchnorm": ("bntrain", "bntrain.fused", "bnbwd", "bnbwd.fused", "bnbwd.linked"),
     "pool": ("poolfwd", "poolbwd"),
 }
@@ -118,7 +119,7 @@ def profile_rows(rows):
     return out
 
 
-def family_rows(rows, steps):
+def family_rows(rows, steps, with_traffic=True):
     """Operation kinds grouped into families (FAMILIES; every other kind is its own family), most GPU time first.
     achieved = algorithmic flops (matrix families) or bytes (the others) of all launches / their summed time,
     both from this run; `algorithmic` and `traffic` are per launch, averaged over the same launches."""
@@ -144,7 +145,8 @@ def family_rows(rows, steps):
             alg = a["bytes"] / a["launches"]
         out.append({"kernel": a["kernel"], "kinds": sorted(a["kinds"]), "bound": "mfma" if matrix else "hbm",
                     "achieved": round(ach, 1), "peak": peak, "unit": unit, "frac": round(ach / peak, 4),
-                    "traffic": MEASURED_HBM_BYTES_PER_LAUNCH.get(a["kernel"]), "traffic_source": TRAFFIC_SOURCE,
+                    "traffic": MEASURED_HBM_BYTES_PER_LAUNCH.get(a["kernel"]) if with_traffic else None,
+                    "traffic_source": TRAFFIC_SOURCE if with_traffic else None,
                     "algorithmic": round(alg), "algorithmic_unit": "flop/launch" if matrix else "byte/launch",
                     "algorithmic_bytes": round(a["bytes"] / a["launches"]),
                     "avg_launch_us": round(a["ms"] * 1e3 / a["launches"], 2), "launches": a["launches"],
@@ -385,6 +387,17 @@ def main():
                     # against each layer's own bound (HBM for the wide 1x1 layers, MFMA for the others)
                     "frac_of_roofline": round(sum(r["roof_ms"] for r in cr) / sum(r["ms"] for r in cr), 4)}
 
+    # the inference program the same way: its convolutions carry the folded batch norm, relu and residual add
+    # ("convfwd.bn"), so one family holds nearly all of its time.  The HBM counters were taken on training
+    # launches only, so `traffic` is null here.
+    roof_infer, families_infer = None, []
+    if infer and not args.no_profile:
+        infer.set_profiling(True)
+        infer.run(args.steps)
+        families_infer = family_rows(by_kind(infer.profile()), args.steps, with_traffic=False)
+        infer.set_profiling(False)
+        roof_infer = families_infer[0] if families_infer else None
+
     flops_step = 3 * net.flops_fwd * args.batch  # fwd + bwd-data + bwd-filter (the stem has no bwd-data)
     ips = args.batch * args.steps / t_train
     out = {
@@ -411,6 +424,8 @@ def main():
         "mean_loss": round(mean_loss, 4),
         "roofline": roof,
         "roofline_hbm": roof_hbm,
+        "roofline_infer": roof_infer,
+        "families_infer": families_infer,
         "hbm_copy_rate": copy_rate,
         "conv": conv,
         "families": families,

@@ -197,8 +197,12 @@ int saga_hip_bias_bwd(const SagaTensorView *dy, const SagaTensorView *db, float 
  * SAGA_HIP_BIAS_BWD_NOALLOC_MAX_BYTES of device memory that every GPU the library runs on holds until the
  * process ends.  Returns SAGA_HIP_ETOOLARGE, with nothing written, when saga_hip_bias_bwd_workspace_size(dy)
  * exceeds that (channels-last tensors of more than 2048 channels once they have 2^20 elements).  The
- * device the stream belongs to must be current.  All calls on one GPU share the array: calls that overlap
- * on one GPU (two streams, two threads) race; calls in stream order do not. */
+ * device the stream belongs to must be current (SAGA_HIP_EINVAL when the stream reports another device).
+ * saga_hip_init(device) resolves the array's address; without it the first call on a device does, which loads
+ * the code object - runtime work that must not happen under stream capture, so a first call made while the
+ * stream is capturing returns SAGA_HIP_EINVAL: call saga_hip_init(device) before capturing.  All calls on one
+ * GPU share the array: calls that overlap on one GPU (two streams, two threads) race; calls in stream order do
+ * not. */
 #define SAGA_HIP_BIAS_BWD_NOALLOC_MAX_BYTES (4u << 20)
 int saga_hip_bias_bwd_noalloc(const SagaTensorView *dy, const SagaTensorView *db, float beta, saga_stream_t stream);
 

@@ -95,9 +95,15 @@ class OracleNet:
             elif ty == "fc":
                 x_ = get(i["x"])
                 x2 = x_.reshape(x_.shape[0], -1)  # flatten in logical (C,H,W) order
-                y = ref.fc_fwd(x2, get(i["w"]), False)
+                y = ref.fc_fwd(x2, get(i["w"]), bool(at.get("transW", False)))
                 if "b" in i:
                     y = self._r(y) + get(i["b"]).reshape(1, -1)
+            elif ty == "reshape":
+                # elements keep their logical (N,C,H,W) order (src/cuda/cuda_dnn.cpp:2504-2540 aliases the storage)
+                y = get(i["x"]).reshape([int(v) for v in at["shape"]])
+            elif ty == "loss":
+                # forward copies x (CudaLossFwd, src/cuda/cuda_dnn.cpp:1358-1393)
+                y = get(i["x"])
             else:
                 raise NotImplementedError(ty)
             a[out] = self._r(y)
@@ -107,17 +113,22 @@ class OracleNet:
         return ref.catclassifier_fwd(self.forward(x, False))
 
     # ------------------------------------------------------------------ backward
-    def backward(self, labels):
+    def backward(self, labels=None):
         """After forward(training=True).  Returns {param name: gradient}, per-sample loss, predictions;
-        activation gradients stay in self.dacts."""
+        activation gradients stay in self.dacts.  A network that ends in an L2 loss node takes no labels: its
+        backward pass starts at that node, the second return value is the node's mmss rows and the third None."""
         a = self.acts
-        logits = a[self.net.output]
-        n = logits.shape[0]
-        pred = ref.catclassifier_fwd(logits)
-        scale = (1.0 / n) * (float(self.loss_scale) if self.half else 1.0)
-        dlogits, loss = ref.catclassifier_bwd(logits, pred, labels, np.float32(scale))
-        d = self.dacts = {self.net.output: self._r(dlogits)}
         grads = {}
+        if getattr(self.net, "loss", None) is None:
+            logits = a[self.net.output]
+            n = logits.shape[0]
+            pred = ref.catclassifier_fwd(logits)
+            scale = (1.0 / n) * (float(self.loss_scale) if self.half else 1.0)
+            dlogits, loss = ref.catclassifier_bwd(logits, pred, labels, np.float32(scale))
+            d = self.dacts = {self.net.output: self._r(dlogits)}
+        else:
+            d, loss, pred = {}, None, None
+            self.dacts = d
         get = lambda name: a[name] if name in a else self.p[name]
 
         def acc(name, g):
@@ -128,6 +139,14 @@ class OracleNet:
 
         for node in reversed(self.net.nodes):
             ty, i, at, out = node["type"], node["in"], node["attrs"], node["out"]
+            if ty == "loss":
+                # dx = (x - target) * strength / N * the program's loss scale, in EVERY precision
+                # (CudaLossBwd, src/cuda/cuda_dnn.cpp:1395-1443; an fp32 program never divides it out again)
+                x_ = get(i["x"])
+                scale = np.float32(np.float32(at.get("strength", 1.0)) / np.float32(x_.shape[0])) * self.loss_scale
+                dx, loss = ref.loss_bwd(x_, get(i["target"]), scale)
+                acc(i["x"], dx)
+                continue
             if out not in d:
                 continue
             dy = d[out]
@@ -172,10 +191,14 @@ class OracleNet:
             elif ty == "fc":
                 x_ = get(i["x"])
                 x2 = x_.reshape(x_.shape[0], -1)
-                grads[i["w"]] = self._r(ref.fc_bwd_w(x2, dy, False))
+                tw = bool(at.get("transW", False))
+                grads[i["w"]] = self._r(ref.fc_bwd_w(x2, dy, tw))
                 if "b" in i:
                     grads[i["b"]] = self._r(dy.sum(0))
-                acc(i["x"], ref.fc_bwd_x(dy, get(i["w"]), False).reshape(x_.shape))
+                if i["x"] != self.net.input:
+                    acc(i["x"], ref.fc_bwd_x(dy, get(i["w"]), tw).reshape(x_.shape))
+            elif ty == "reshape":
+                acc(i["x"], dy.reshape(get(i["x"]).shape))
             else:
                 raise NotImplementedError(ty)
         return grads, loss, pred
@@ -204,7 +227,7 @@ class OracleNet:
             self.loss_scale = ref.loss_scale_update(self.loss_scale, flags)
         return flags
 
-    def train_step(self, x, labels):
+    def train_step(self, x, labels=None):
         self.forward(x, training=True)
         grads, loss, pred = self.backward(labels)
         flags = self.adam(grads)

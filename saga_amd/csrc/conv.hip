@@ -182,8 +182,7 @@ size_t saga_hip_conv2d_bwd_data_bnbwd_size(const SagaTensorView *dy, const SagaT
                                            const SagaConvParams *p)
 {
     ConvGeom g;
-    if(geometry(dx, w, dy, p, &g) || force_direct() || !conv_mfma_bwd_data_ok(dy, w, dx, g) || g.C % 8 || g.dil != 1 ||
-       g.stride > 4)
+    if(geometry(dx, w, dy, p, &g) || force_direct() || !conv_mfma_bnbwd_link_ok(dy, w, dx, g))
         return 0;
     return conv_mfma_bnbwd_floats(g) * sizeof(float);
 }

@@ -51,6 +51,7 @@ int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const 
                        const ConvGeom &g, float alpha, float beta, void *ws, size_t ws_bytes, hipStream_t st,
                        const void *wt_ready = nullptr, const ConvBnBwdLink *link = nullptr);
 bool conv_mfma_bwd_data_ok(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx, const ConvGeom &g);
+bool conv_mfma_bnbwd_link_ok(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx, const ConvGeom &g);
 int conv_mfma_transpose_blocks(int K, int C, int RS);
 int conv_mfma_transpose_batched(const SagaFilterTransposeJob *jobs, int njobs, int total_blocks, hipStream_t st);
 int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, const SagaTensorView *dw,

@@ -2214,6 +2214,21 @@ bool conv_mfma_bwd_data_ok(const SagaTensorView *dy, const SagaTensorView *w, co
     return common_ok(dy, w, dx, g, &ldy, &ldx) && ilog2_exact(g.stride) >= 0;
 }
 
+// Whether a backward-data launch of this geometry can carry a batch-norm backward link: the conditions on the
+// convolution's own tensors (those on the norm's input are checked at the launch).  The size query and the
+// launcher share it, so that a caller is never told to allocate partials for a launch that would be refused.
+bool conv_mfma_bnbwd_link_ok(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx, const ConvGeom &g)
+{
+    CLInfo ldy, ldx;
+    if(!common_ok(dy, w, dx, g, &ldy, &ldx) || ilog2_exact(g.stride) < 0)
+        return false;
+    const int64_t ab = ((ldy.rows - 1) * ldy.pitch + ldy.C) * 2, bb = (int64_t)g.K * g.R * g.S * g.C * 2;
+    const bool kernel_ok = dma_stages() >= 2 && ab < 0x7fffff00 && bb < 0x7fffff00 && g.dil == 1 && g.stride <= 4 &&
+                           ((g.R + g.stride - 1) / g.stride) * ((g.S + g.stride - 1) / g.stride) <= 64;
+    const bool vec = ldx.pitch % 8 == 0 && g.C % 8 == 0 && aligned16(dx->ptr);
+    return kernel_ok && vec;
+}
+
 // wt_ready: the filter already transposed to C,R,S,K (by transpose_filter or the batched kernel below);
 // otherwise it is transposed into the workspace first
 int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const SagaTensorView *dx,
@@ -2228,13 +2243,9 @@ int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const 
         return SAGA_HIP_EUNSUPPORTED;
     if(link) {
         // only the pipelined kernel's vector epilogue carries the link; checked before anything is launched
-        const int64_t ab = ((ldy.rows - 1) * ldy.pitch + ldy.C) * 2, bb = (int64_t)g.K * g.R * g.S * g.C * 2;
-        const bool kernel_ok = dma_stages() >= 2 && ab < 0x7fffff00 && bb < 0x7fffff00 && g.dil == 1 && g.stride <= 4 &&
-                               ((g.R + g.stride - 1) / g.stride) * ((g.S + g.stride - 1) / g.stride) <= 64;
-        const bool vec = ldx.pitch % 8 == 0 && g.C % 8 == 0 && aligned16(dx->ptr);
-        if(!kernel_ok || !vec || !link->x || link->x->dtype != SAGA_HALF || !same_dims(link->x, dx) ||
+        if(!conv_mfma_bnbwd_link_ok(dy, w, dx, g) || !link->x || link->x->dtype != SAGA_HALF || !same_dims(link->x, dx) ||
            !as_channels_last(link->x, &lbx) || lbx.rows != ldx.rows || lbx.pitch % 8 || !aligned16(link->x->ptr) ||
-           link->x->ptr == dx->ptr)
+           lbx.rows * lbx.pitch >= (int64_t)1 << 31 || link->x->ptr == dx->ptr)
             return SAGA_HIP_EUNSUPPORTED;
         if(!link->mean || !link->partial || (link->relu && (!link->s || !link->b || !link->invstd)))
             return SAGA_HIP_EINVAL;

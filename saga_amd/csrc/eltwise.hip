@@ -730,6 +730,21 @@ int saga_hip_bias_bwd_noalloc(const SagaTensorView *dy, const SagaTensorView *db
         const hipError_t e = hipGetDevice(&device);
         if(e != hipSuccess)
             return (int)e;
+        if(device < 0 || device >= MAX_SCRATCH_DEVICES)
+            return SAGA_HIP_EINVAL;
+        // the scratch array belongs to the current device: a stream of another device would hand its kernels
+        // an address of the wrong GPU
+        hipDevice_t stream_device = device;
+        if(stream && hipStreamGetDevice(as_stream(stream), &stream_device) == hipSuccess && (int)stream_device != device)
+            return SAGA_HIP_EINVAL;
+        if(!bias_scratch_ptr[device].load(std::memory_order_acquire)) {
+            // resolving the symbol loads the code object and materialises the array: not under stream capture,
+            // where saga_hip_init(device) has to have done it beforehand
+            hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+            if(hipStreamIsCapturing(as_stream(stream), &capturing) == hipSuccess &&
+               capturing != hipStreamCaptureStatusNone)
+                return SAGA_HIP_EINVAL;
+        }
         const int rc = resolve_bias_scratch(device, &ws);
         if(rc)
             return rc;

@@ -19,6 +19,8 @@ class Net:
         self.trainable = []  # parameter names updated by the optimizer, in creation order
         self._n = 0
         self.input = "input"
+        self.rows = batch    # samples in the input tensor (the conv harness runs 2 rows at program batch size 1)
+        self.loss = None     # output of an L2 loss node, when the network ends in one instead of a classifier
         self.output = None   # logits
         self.flops_fwd = 0   # multiply-add counted as 2
 
@@ -118,13 +120,16 @@ class Builder:
         self.shape[y] = (c,) + tuple(self.shape[xs[0]][1:])
         return y
 
-    def fc(self, x, name, outputs, bias=True):
+    def fc(self, x, name, outputs, bias=True, transW=False):
         net = self.net
         fin = int(np.prod(self.shape[x]))
-        net.params[name + "-w"] = self.he((fin, outputs), fin)  # transW = false: [in, out]
+        # transW = false: [in, out]; true: [out, in] (reference: src/node.cpp:266-275)
+        net.params[name + "-w"] = self.he((outputs, fin) if transW else (fin, outputs), fin)
         net.trainable.append(name + "-w")
         ins = {"x": x, "w": name + "-w"}
         attrs = {"outputs": outputs}
+        if transW:
+            attrs["transW"] = True
         if bias:
             net.params[name + "-b"] = np.zeros((outputs,), np.float32)
             net.trainable.append(name + "-b")
@@ -133,6 +138,23 @@ class Builder:
         y = net.add("fc", ins, attrs, name)
         self.shape[y] = (outputs,)
         net.flops_fwd += 2 * fin * outputs
+        return y
+
+    def reshape(self, x, shape):
+        """shape: the new (C, H, W) of a sample; elements keep their logical order."""
+        assert int(np.prod(shape)) == int(np.prod(self.shape[x]))
+        y = self.net.add("reshape", {"x": x}, {"shape": S.Dims([self.net.rows, *shape])})
+        self.shape[y] = tuple(shape)
+        return y
+
+    def loss(self, x, target, strength=1.0):
+        """The L2 loss node against a target held like a parameter (not trained); its y copies x, its second
+        output (per-sample min / max / mean / mean square of x - target) is named y + "-mmss"."""
+        net = self.net
+        net.params["target"] = np.asarray(target, np.float32)
+        y = net.add("loss", {"x": x, "target": "target"}, {"strength": float(strength)})
+        self.shape[y] = self.shape[x]
+        net.loss = y
         return y
 
     # reference: Graph::addResNet, src/graph.cpp:384-425
@@ -232,6 +254,24 @@ def unet(batch=16, seed=5, dtype=S.HALF, image=256, classes=8, widths=(64, 128, 
     return net
 
 
+def conv_harness(dtype=S.FLOAT, seed=6):
+    """The training graph of the reference's `conv` command (test/test_conv.cpp:96-140): two 1x5x5 diagonal
+    patterns -> 3x3 stride-2 conv to 5 channels + bias -> relu -> fc to 20 with transposed weights + bias -> relu
+    -> reshape to 5x2x2 -> 3x3 stride-2 transposed conv to 1 channel + bias -> L2 loss against the input.
+    The program's batch size is 1 although the tensors hold two samples, as in the harness, so the initial
+    loss scale is 1.  Returns (net, x)."""
+    net = Net("conv-harness", 1, (1, 5, 5), 0, dtype)
+    net.rows = 2
+    b = Builder(net, seed)
+    x = np.stack([np.eye(5, dtype=np.float32), np.eye(5, dtype=np.float32)[:, ::-1]])[:, None]
+    h = b.relu(b.conv(net.input, "node1", 5, 3, 2, 0, bias=True))
+    h = b.relu(b.fc(h, "fc1", 20, transW=True))
+    h = b.reshape(h, (5, 2, 2))
+    net.output = b.conv(h, "node2", 1, 3, 2, 0, bias=True, transpose=True)
+    b.loss(net.output, x)
+    return net, x
+
+
 def np_dtype(code):
     return np.float16 if code == S.HALF else np.float32
 
@@ -251,7 +291,9 @@ def build_graph(net, x, labels=None, with_classifier=True, param_dtype=None):
     for n in net.nodes:
         node = g.add_node(n["type"], {k: t[v] for k, v in n["in"].items()}, n["attrs"], n["name"])
         t[n["out"]] = node.y()
-    if with_classifier:
+        if n["type"] == "loss":
+            t[n["out"] + "-mmss"] = node.output("mmss")
+    if with_classifier and net.loss is None:
         node = g.add_node("catclassifier", {"x": t[net.output]})
         t["pred"] = node.y()
         t["loss"] = node.output("loss")

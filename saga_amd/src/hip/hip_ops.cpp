@@ -233,6 +233,9 @@ struct BnBwdLinkState {
     std::shared_ptr<HipMemory> partial;
     int rows = 0;
     bool valid = false; // set by every ConvBwdData::exec, consumed by the BnBwd::exec that follows
+    // the kernel library refused the linked launch (the norm's input is a view it cannot read in the epilogue):
+    // both operations stay on their separate paths from then on and report the traffic of those
+    bool refused = false;
 };
 
 struct ConvBwdData : public HipOperation {
@@ -286,7 +289,7 @@ struct ConvBwdData : public HipOperation {
     void exec(HipProgram &p) override
     {
         const SagaTensorView vdy = dy_->view(), vw = w_->view(), vdx = dx_->view();
-        if(link_) {
+        if(link_ && !link_->refused) {
             link_->valid = false;
             const SagaTensorView vx = bn_x_->view();
             SagaBnBwdLink l = {&vx,
@@ -307,6 +310,7 @@ struct ConvBwdData : public HipOperation {
             }
             if(r != SAGA_HIP_EUNSUPPORTED)
                 chkSaga(r);
+            link_->refused = true;
         }
         chkSaga(saga_hip_conv2d_bwd_data_wt(&vdy, &vw, wt_ ? wt_->deviceMem() : nullptr, &vdx, &cp_, 1.0f, beta_,
                                             p.m_ctx->m_workspace.ptr(), p.m_ctx->m_workspace.size(), S(p)));
@@ -325,7 +329,7 @@ struct ConvBwdData : public HipOperation {
     double flops() const override { return conv_flops(dx_, w_, dy_, cp_.group); }
     double bytes() const override
     {
-        return nbytes(dy_) + nbytes(w_) + nbytes(dx_) * ((beta_ != 0 ? 2 : 1) + (link_ ? 1 : 0));
+        return nbytes(dy_) + nbytes(w_) + nbytes(dx_) * ((beta_ != 0 ? 2 : 1) + (link_ && !link_->refused ? 1 : 0));
     }
 };
 
@@ -1028,7 +1032,7 @@ struct BnBwd : public HipOperation {
     double bytes() const override
     {
         const double e = nbytes(dx_);
-        if(link_) // one pass: x and the masked gradient in, dx out
+        if(link_ && !link_->refused) // one pass: x and the masked gradient in, dx out
             return e * (3 + (dx_beta_ != 0 ? 1 : 0));
         const bool reads_y = (flags_ & SAGA_BN_RELU) && (flags_ & SAGA_BN_ADD);
         if(reads_y && dz_ && dz_beta_ == 0) // pass 1: x, y (or its 1-bit mask), dy -> dz ; pass 2: x, dz -> dx

@@ -279,6 +279,49 @@ def test_resnet50_training_links_bn_backward_to_convolutions(monkeypatch):
             assert e <= 1e-2, (k, e)  # fp16 rounding differences grown through up to 50 layers; the parity bar is 2e-2
 
 
+def test_bn_backward_link_through_a_strided_projection(monkeypatch):
+    """A batch norm + relu whose output feeds a 3x3 stride-2 convolution and the 1x1 stride-2 projection of the
+    same downsampling block.  The engine moves the projection's backward data (one pixel in four) behind the
+    dense writer, so the LAST writer of the norm's output gradient - the one that carries the link - is a 1x1
+    stride-2 launch accumulating onto the 3x3's result: three of its four residue classes have no tap and only
+    mask and sum the old gradient.  Gradients with the link against the program without it and the oracle."""
+    names = ["stem-w", "stem-bn-s", "stem-bn-b", "blk-conv-1-w", "blk-conv-p-w"]
+
+    def build():
+        net = N.Net("strided-link", 4, (8, 24, 24), 10, S.HALF)
+        b = N.Builder(net, 21)
+        x = b.relu(b.bn(b.conv(net.input, "stem", 256, 3, 1, 1), "stem-bn"))
+        x = b.basic_block(x, 64, True, "blk")
+        net.output = b.fc(b.pool("avgpool", x, global_=True), "fc", 10)
+        return net
+
+    grads, kinds = {}, {}
+    for link in (True, False):
+        if not link:
+            monkeypatch.setenv("SAGA_HIP_NO_BNBWD_LINK", "1")
+        net = build()
+        x, labels = inputs(net, 21)
+        ctx = S.Context()
+        g, t = N.build_graph(net, x)
+        p = ctx.create_program(g, net.batch, training=True, learning_rate=1e-4, initial_loss_scale=64.0)
+        ctx.resolve(t["labels"]).write(labels)
+        dev_grads = {k: ctx.resolve(t[k].grad()) for k in names}
+        p.set_profiling(True)
+        p.run(1)
+        kinds[link] = {r["kind"]: r["launches"] for r in p.profile()}
+        grads[link] = {k: dev_grads[k].read().astype(np.float32) for k in names}
+    print(" kinds with the link:", {k: v for k, v in kinds[True].items() if "bn" in k or "conv" in k})
+    assert kinds[True].get("convbwddata.bn", 0) >= 1 and "convbwddata.bn" not in kinds[False]
+    o = OracleNet(build(), lr=1e-4, loss_scale=64.0)
+    o.forward(x, True)
+    og, _, _ = o.backward(labels)
+    for k in names:
+        e = rel_err(grads[True][k], grads[False][k])
+        eo = rel_err(grads[True][k], og[k].reshape(grads[True][k].shape))
+        print(f"  grad {k}: linked against unlinked {e:.3e}, against the oracle {eo:.3e}")
+        assert e <= 1e-2 and eo <= 2e-2, (k, e, eo)
+
+
 def test_unet_training_fp16():
     """Config 5 reduced (batch 2, 32x32, narrower): transposed convs and concat-as-strided-outputs,
     forward + backward + Adam.  The per-pixel head is exercised through a global pooled classifier."""

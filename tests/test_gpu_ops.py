@@ -361,6 +361,9 @@ BNBWD_LINK_CASES = [
     (2, 64, 56, 56, 64, 3, 1, 1, True, 0.0, 0),     # many block rows
     (5, 512, 7, 7, 128, 1, 0, 1, True, 0.0, 0),     # at most one block per CU: the kernel with producer wavefronts
     (11, 256, 56, 56, 64, 1, 0, 1, True, 0.0, 0),   # more than 256 blocks of 256x128
+    (2, 256, 12, 12, 64, 1, 0, 2, True, 1.0, 0),    # 1x1 stride 2 accumulating: three classes run blocks with no
+                                                    # reduction step at all, which mask and sum the old gradient
+    (2, 128, 13, 13, 24, 3, 1, 4, True, 1.0, 8),    # stride 4: sixteen residue classes, seven without a tap
 ]
 
 

@@ -78,26 +78,59 @@ def test_reference_fc_harness(half):
     assert ("adam-mixed" if half else "adam-f32") in r.stdout and "RESULT:" in r.stdout and "nan" not in r.stdout
 
 
+def stream_until(cmd, want_rows, prefix, cap_seconds, env=None):
+    """Starts cmd, reads its standard output until `want_rows` lines starting with `prefix` have arrived or
+    cap_seconds have passed, then interrupts it (the harness loops until SIGINT).  Returns all complete lines."""
+    import select
+    import signal
+    import time
+    proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, env=env)
+    deadline = time.monotonic() + cap_seconds
+    buf, rows = b"", 0
+    try:
+        while rows < want_rows and time.monotonic() < deadline and proc.poll() is None:
+            ready, _, _ = select.select([proc.stdout], [], [], 0.5)
+            if not ready:
+                continue
+            chunk = os.read(proc.stdout.fileno(), 1 << 16)
+            if not chunk:
+                break
+            buf += chunk
+            rows = sum(1 for l in buf.split(b"\n")[:-1] if l.startswith(prefix))
+    finally:
+        if proc.poll() is None:
+            proc.send_signal(signal.SIGINT)
+            try:
+                proc.wait(timeout=20)
+            except subprocess.TimeoutExpired:
+                proc.kill()
+                proc.wait()
+    err = proc.stderr.read().decode(errors="replace")
+    print(err[-2000:])
+    return buf.decode(errors="replace").split("\n")[:-1]  # what follows the last newline is a cut line
+
+
 @pytest.mark.parametrize("half", [False, True])
 def test_reference_conv_training_loop(half):
     """`saga conv` (test/test_conv.cpp): strided conv + bias -> relu -> fc -> relu -> reshape -> transposed conv
-    + bias -> L2 loss, trained in an endless loop that prints every 1000 steps; the test lets it run a few
-    seconds.  The target is the input pattern; the mean squared error it prints (last column of MMSS) must fall
-    well below the 0.2 of an untrained net and stay finite."""
+    + bias -> L2 loss, trained in an endless loop that prints every 1000 steps.  Its weights are drawn from a
+    generator seeded with the clock (src/tensor.cpp:1081-1085) and some draws settle in a local minimum, so the
+    criterion is one that holds for every draw and every machine speed: the test reads ten print blocks (however
+    long they take, up to a generous cap), every value must be finite, and the mean squared error (last column
+    of MMSS, one row per sample) at the last block must be at most half of what the first block - printed
+    after the first step - shows.  tests/test_gpu_conv_harness_graph.py runs the same graph from seeded
+    weights against the oracle step by step."""
     if not os.path.exists(BIN):
         pytest.skip("oracle/_ref/saga_refhost not built (make -C oracle -f Makefile.ref)")
-    r = subprocess.run(["timeout", "-s", "INT", "6", BIN, "conv", *(["-h"] if half else [])], capture_output=True,
-                       text=True, timeout=60)
-    lines = r.stdout.splitlines()
-    if not r.stdout.endswith("\n"):
-        lines = lines[:-1]  # the signal cut the last line in the middle
+    lines = stream_until([BIN, "conv", *(["-h"] if half else [])], 20, b"MMSS: [", 150)
     rows = [l.split() for l in lines if l.startswith("MMSS: [")]
-    assert len(rows) >= 4, r.stdout[-2000:]
-    rows = rows[:len(rows) // 2 * 2]  # the last block may have been cut by the signal
+    rows = rows[:len(rows) // 2 * 2]  # whole blocks of two samples
+    assert len(rows) >= 6, "\n".join(lines[-40:])
     ms = [float(row[-1]) for row in rows]
-    print("mean squared error per print:", ms[:2], "...", ms[-2:])
-    assert all(np.isfinite(v) for v in ms)
-    assert max(ms[-2:]) <= 0.08 and sum(ms[-2:]) <= sum(ms[:2])
+    vals = [float(v) for row in rows for v in row[-4:]]
+    print("mean squared error per print:", ms)
+    assert all(np.isfinite(v) for v in vals)
+    assert sum(ms[-2:]) <= 0.5 * sum(ms[:2])
 
 
 def write_idx_dataset(path, n_train=6400, n_test=1280, seed=0):
@@ -122,6 +155,29 @@ def write_idx_dataset(path, n_train=6400, n_test=1280, seed=0):
             f.write(np.array([2051, n, 28, 28], ">u4").tobytes() + img.tobytes())
         with open(os.path.join(path, f"{prefix}-labels-idx1-ubyte"), "wb") as f:
             f.write(np.array([2049, n], ">u4").tobytes() + lab.tobytes())
+
+
+def write_cifar_dataset(path, seed=0):
+    """A stand-in for the CIFAR-10 binary files the reference's `cifar` command maps (test/cifar.cpp:51-62,
+    104-110: data_batch_1..5.bin and test_batch.bin, 10000 records each of one label byte followed by a
+    3 x 32 x 32 planar image): ten fixed 3 x 8 x 8 colour patterns blown up to 32 x 32, shifted by up to two
+    pixels, with noise."""
+    rng = np.random.default_rng(seed)
+    templates = (rng.random((10, 3, 8, 8)) > 0.5).astype(np.float32).repeat(4, axis=2).repeat(4, axis=3)
+    for name in [f"data_batch_{i}.bin" for i in range(1, 6)] + ["test_batch.bin"]:
+        n = 10000
+        labels = rng.integers(0, 10, n).astype(np.uint8)
+        dy, dx = rng.integers(-2, 3, n), rng.integers(-2, 3, n)
+        img = np.empty((n, 3, 32, 32), np.float32)
+        for sy in range(-2, 3):
+            for sx in range(-2, 3):
+                sel = (dy == sy) & (dx == sx)
+                img[sel] = np.roll(templates[labels[sel]], (sy, sx), axis=(2, 3))
+        img = np.clip(img * 180.0 + 30.0 + rng.normal(0, 25, img.shape), 0, 255).astype(np.uint8)
+        rec = np.empty((n, 3073), np.uint8)
+        rec[:, 0] = labels
+        rec[:, 1:] = img.reshape(n, -1)
+        rec.tofile(os.path.join(path, name))
 
 
 def accuracies(stdout):
@@ -172,3 +228,30 @@ def test_reference_classifier_harness(tmp_path, args, floor, graphs):
     print(r2.stderr[-2000:])
     print("accuracy after reload:", acc2[-5:])
     assert r2.returncode == 0 and acc2 and acc2[0] >= floor
+
+
+@pytest.fixture(scope="module")
+def cifar_dir(tmp_path_factory):
+    if not os.path.exists(BIN):
+        pytest.skip("oracle/_ref/saga_refhost not built (make -C oracle -f Makefile.ref)")
+    d = tmp_path_factory.mktemp("cifar")
+    write_cifar_dataset(str(d))
+    return str(d)
+
+
+@pytest.mark.parametrize("args,floor", [
+    (["-m", "resnet-18", "-h", "-c", "-b", "128", "-r", "1e-3"], 95.0),
+    (["-m", "squeezenet+bn", "-b", "128", "-r", "1e-3"], 90.0),
+], ids=["resnet18-fp16-nhwc", "squeezenet-bn-fp32"])
+def test_reference_cifar_harness(cifar_dir, args, floor):
+    """The reference's `cifar` command (test/cifar.cpp) on synthesised CIFAR-format files: 3 x 32 x 32 uint8
+    batches interleaved to channels-last by its loader, 50000 training and 10000 test records, the basic-block
+    ResNet of Graph::addResNet and the fire modules of SqueezeNet (concat of a 1x1 and a 3x3 branch, unpadded
+    3x3 stride-2 max pooling) trained through the same double-buffered loop as `mnist`."""
+    r = subprocess.run([BIN, "cifar", cifar_dir, *args], capture_output=True, text=True, timeout=300)
+    acc = accuracies(r.stdout)
+    print(r.stdout[-1500:].replace("\033", "<esc>"))
+    print(r.stderr[-2000:])
+    print("accuracy per refresh:", acc[-25:])
+    assert r.returncode == 0
+    assert acc and max(acc) >= floor

@@ -97,9 +97,14 @@ class TorchNet:
             elif ty == "concat":
                 y = torch.cat([get(i[f"x{j}"]) for j in range(len(i))], dim=at.get("axis", 1))
             elif ty == "fc":
-                y = get(i["x"]).flatten(1) @ get(i["w"])
+                w = get(i["w"])
+                y = get(i["x"]).flatten(1) @ (w.T if at.get("transW") else w)
                 if "b" in i:
                     y = y + get(i["b"]).reshape(1, -1)
+            elif ty == "reshape":
+                y = get(i["x"]).reshape([int(v) for v in at["shape"]])
+            elif ty == "loss":
+                y = get(i["x"])
             else:
                 raise NotImplementedError(ty)
             a[out] = y
@@ -115,6 +120,18 @@ class TorchNet:
         (per_sample.mean() * scale).backward()
         return ({k: self.p[k].grad.numpy().copy() for k in self.net.trainable}, logits.detach().numpy(),
                 per_sample.detach().numpy())
+
+
+    def l2_grads(self, x, scale=1.0):
+        """d(scale * strength / (2 N) * sum (y - target)^2)/d(parameter) for a network ending in an L2 loss node,
+        whose own gradient is then (y - target) * strength / N * scale; returns (gradients, y)."""
+        for k in self.net.trainable:
+            self.p[k].grad = None
+        y = self.forward(x, True)
+        node = [n for n in self.net.nodes if n["type"] == "loss"][0]
+        r = y - self.p[node["in"]["target"]]
+        (r.pow(2).sum() * (0.5 * node["attrs"].get("strength", 1.0) / y.shape[0] * scale)).backward()
+        return {k: self.p[k].grad.numpy().copy() for k in self.net.trainable}, y.detach().numpy()
 
 
 def worst(got, want):
@@ -322,3 +339,62 @@ def test_per_pixel_softmax_head_against_torch():
     want = torch.softmax(F.conv2d(torch.tensor(x.astype(np.float64)), w, torch.tensor(net.params["c-bt"].astype(np.float64)).reshape(-1)), 1)
     assert worst(got, want.numpy()) <= 1e-6
     np.testing.assert_allclose(got.sum(1), 1.0, atol=1e-6)
+
+
+def off_zero(net, rng):
+    for k in net.trainable:
+        if k.endswith(("-b", "-bt")):
+            net.params[k] = (rng.standard_normal(net.params[k].shape) * 0.2).astype(np.float32)
+
+
+@pytest.mark.parametrize("loss_scale", [1.0, 8.0])
+def test_conv_harness_graph_loss_reshape_transw_against_torch_double(loss_scale):
+    """The graph of the reference's `conv` command (test/test_conv.cpp:96-140): the three node kinds the
+    other networks do not use - fc with transposed weights, reshape, the L2 loss node as the start of the
+    backward pass - against autograd of strength / (2 N) * sum (y - target)^2 times the loss scale, which
+    the node applies in fp32 programs too (src/cuda/cuda_dnn.cpp:1433-1443)."""
+    net, x = N.conv_harness(S.FLOAT)
+    off_zero(net, np.random.default_rng(3))
+    [n for n in net.nodes if n["type"] == "loss"][0]["attrs"]["strength"] = 1.5
+    o = OracleNet(net, loss_scale=loss_scale)
+    assert OracleNet(net).loss_scale == 1.0  # program batch size 1 with two rows in the tensors
+    o.forward(x, training=True)
+    grads, mmss, pred = o.backward()
+    assert pred is None and set(grads) == set(net.trainable)
+    t = TorchNet(net)
+    tg, ty = t.l2_grads(x, loss_scale)
+    errs = {"y": worst(o.acts[net.output], ty), "loss y": worst(o.acts[net.loss], ty)}
+    for n in net.nodes:
+        errs["act " + n["out"]] = worst(o.acts[n["out"]], t.acts[n["out"]].detach().numpy())
+    for k in net.trainable:
+        errs["d " + k] = worst(grads[k], tg[k])
+    r = (ty - x.astype(np.float64)).reshape(2, -1)
+    want_mmss = np.stack([np.minimum(r.min(1), 0), np.maximum(r.max(1), 0), r.mean(1), (r * r).mean(1)], 1)
+    errs["mmss"] = worst(mmss, want_mmss)
+    print({k: f"{v:.1e}" for k, v in errs.items()})
+    bad = {k: v for k, v in errs.items() if v > 2e-6}
+    assert not bad, bad
+    # the transposed fc weight really is [out, in]
+    assert net.params["fc1-w"].shape == (20, 20) and net.params["node1-w"].shape == (5, 1, 3, 3)
+    assert net.params["node2-w"].shape == (5, 1, 3, 3)
+
+
+def test_conv_harness_graph_trains_like_autograd_plus_numpy_adam():
+    """Twenty fp32 steps of the conv harness graph: oracle weights against torch double gradients fed to the
+    numpy Adam, and the mean squared error falls."""
+    net, x = N.conv_harness(S.FLOAT)
+    lr = 1e-2
+    o = OracleNet(net, lr=lr)
+    w = {k: np.array(net.params[k], np.float32).reshape(-1) for k in net.trainable}
+    m = {k: np.zeros_like(w[k]) for k in net.trainable}
+    v = {k: np.zeros_like(w[k]) for k in net.trainable}
+    mse = []
+    for step in range(1, 21):
+        params = {k: (w[k].reshape(net.params[k].shape) if k in w else net.params[k]) for k in net.params}
+        tg, _ = TorchNet(net, params).l2_grads(x)
+        mmss, _, grads, flags = o.train_step(x)
+        mse.append(float(mmss[:, 3].mean()))
+        for k in net.trainable:
+            numpy_adam(w[k], tg[k].astype(np.float32).reshape(-1), m[k], v[k], step, lr, 0.0)
+            assert worst(o.p[k], w[k]) <= 1e-5, (step, k)
+    assert mse[-1] < 0.8 * mse[0], mse
