@@ -73,24 +73,52 @@ template <> struct Vec<float> {
     static constexpr int n = 4;
 };
 
-// Flat, dense, same layout for every operand: 16-byte vectors, grid-stride.
+// Flat, dense, same layout for every operand: 16-byte vectors.  A block owns a contiguous run of tiles of
+// 4 x 256 vectors (16 KB per operand) and requests the four vectors of a lane before it stores the first
+// result; the grid has up to 65535 blocks, dispatched in order, so that at any time the chip works on one
+// compact window of the tensors.  Measured on MI355X with a 1 GiB copy: 5.4 - 6.0 TB/s this way, 4.1 - 4.5 TB/s
+// with a grid-stride loop whose four vectors lie a whole grid apart, 5.2 TB/s for the runtime's own copy.
 template <typename T, int NIN, bool READ_OLD, typename F>
 __global__ void __launch_bounds__(256) ew_flat(T *__restrict__ out, const T *__restrict__ a, const T *__restrict__ b,
                                                int64_t nvec, int64_t total, F f)
 {
     typedef typename Vec<T>::type V;
     constexpr int VN = Vec<T>::n;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += stride) {
-        V va = ((const V *)a)[i];
-        V vb = NIN > 1 ? ((const V *)b)[i] : va;
-        V vo = READ_OLD ? ((const V *)out)[i] : va;
+    constexpr int U = 4;
+    auto apply = [&](const V &va, const V &vb, const V &vo) {
         V r;
 #pragma unroll
         for(int j = 0; j < VN; j++)
             r[j] = (T)f((float)va[j], (float)vb[j], (float)vo[j]);
-        ((V *)out)[i] = r;
+        return r;
+    };
+    const int64_t tiles = (nvec + 256 * U - 1) / (256 * U);
+    const int64_t per = (tiles + gridDim.x - 1) / gridDim.x;
+    const int64_t t0 = (int64_t)blockIdx.x * per;
+    const int64_t t1 = t0 + per < tiles ? t0 + per : tiles;
+    for(int64_t t = t0; t < t1; t++) {
+        const int64_t i = t * (256 * U) + threadIdx.x;
+        if(i + (U - 1) * 256 < nvec) {
+            V va[U], vb[U], vo[U];
+#pragma unroll
+            for(int u = 0; u < U; u++) {
+                va[u] = ((const V *)a)[i + u * 256];
+                vb[u] = NIN > 1 ? ((const V *)b)[i + u * 256] : va[u];
+                vo[u] = READ_OLD ? ((const V *)out)[i + u * 256] : va[u];
+            }
+#pragma unroll
+            for(int u = 0; u < U; u++)
+                ((V *)out)[i + u * 256] = apply(va[u], vb[u], vo[u]);
+        } else {
+            for(int64_t k = i; k < nvec; k += 256) {
+                const V va = ((const V *)a)[k];
+                const V vb = NIN > 1 ? ((const V *)b)[k] : va;
+                const V vo = READ_OLD ? ((const V *)out)[k] : va;
+                ((V *)out)[k] = apply(va, vb, vo);
+            }
+        }
     }
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     // tail
     const int64_t base = nvec * VN;
     for(int64_t i = base + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
@@ -193,7 +221,7 @@ int launch_ew_t(const SagaTensorView *out, const SagaTensorView *a, const SagaTe
     const bool al = aligned16(out->ptr) && aligned16(a->ptr) && (NIN < 2 || aligned16(b->ptr));
     if(dense(out) && same_strides(out, a) && (NIN < 2 || same_strides(out, b)) && al) {
         const int64_t nvec = total / VN;
-        ew_flat<T, NIN, READ_OLD, F><<<grid_for(nvec ? nvec : 1, 256, 256 * 16), 256, 0, st>>>(
+        ew_flat<T, NIN, READ_OLD, F><<<grid_for(nvec ? (nvec + 3) / 4 : 1, 256, 65535), 256, 0, st>>>(
             (T *)out->ptr, (const T *)a->ptr, (const T *)(NIN > 1 ? b->ptr : a->ptr), nvec, total, f);
         SAGA_CHECK_LAUNCH();
         return 0;
