@@ -146,8 +146,10 @@ int saga_hip_adam_f32(size_t n, float *w, const float *g, float *m, float *v, fl
         return 0;
     if(!aligned16(w) || !aligned16(g) || !aligned16(m) || !aligned16(v))
         return SAGA_HIP_EUNSUPPORTED;
-    adam_f32_k<<<grid_for((int64_t)(n / 4 + 1), 256, 256 * 8), 256, 0, as_stream(stream)>>>(n, w, g, m, v, b1t, b2t, lr,
-                                                                                          lambda, aux);
+    // one 16-byte vector per lane and as many blocks as that takes: dispatched in order, the blocks sweep the
+    // arena front to back, which this GPU's memory system serves faster than a grid-stride walk
+    adam_f32_k<<<grid_for((int64_t)(n / 4 + 1), 256, 1 << 24), 256, 0, as_stream(stream)>>>(n, w, g, m, v, b1t, b2t, lr,
+                                                                                         lambda, aux);
     SAGA_CHECK_LAUNCH();
     return 0;
 }
@@ -161,7 +163,7 @@ int saga_hip_adam_mixed(size_t n, float alpha, void *w_half, const void *g_half,
         return 0;
     if(((uintptr_t)w_half & 7) || ((uintptr_t)g_half & 7) || !aligned16(m) || !aligned16(v) || !aligned16(c))
         return SAGA_HIP_EUNSUPPORTED;
-    adam_mixed_k<<<grid_for((int64_t)(n / 4 + 1), 256, 256 * 8), 256, 0, as_stream(stream)>>>(
+    adam_mixed_k<<<grid_for((int64_t)(n / 4 + 1), 256, 1 << 24), 256, 0, as_stream(stream)>>>(
         n, alpha, (half_t *)w_half, (const half_t *)g_half, m, v, c, b1t, b2t, lr, lambda, aux);
     SAGA_CHECK_LAUNCH();
     return 0;

@@ -550,11 +550,23 @@ __device__ __forceinline__ void gather_epilogue(const GatherArgs &g, float16_t (
 #pragma unroll
                 for(int v = 0; v < 16; v++) {
                     float a = 0.0f, q = 0.0f;
+                    if constexpr(TM == 2) {
+                        // the two rows of a channel rounded to fp16 as they are stored, in one packed register;
+                        // sum and sum of squares are one two-element dot product each (fp32 result)
+                        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+                        h2 pr;
+                        pr[0] = (!MASK || okr[0]) ? (_Float16)(g.alpha * acc[0][j][v]) : (_Float16)0;
+                        pr[1] = (!MASK || okr[1]) ? (_Float16)(g.alpha * acc[1][j][v]) : (_Float16)0;
+                        const h2 ones = {(_Float16)1, (_Float16)1};
+                        a = __builtin_amdgcn_fdot2(pr, ones, 0.0f, false);
+                        q = __builtin_amdgcn_fdot2(pr, pr, 0.0f, false);
+                    } else {
 #pragma unroll
-                    for(int i = 0; i < TM; i++) {
-                        const float r = (!MASK || okr[i]) ? (float)(half_t)(g.alpha * acc[i][j][v]) : 0.0f;
-                        a += r;
-                        q += r * r;
+                        for(int i = 0; i < TM; i++) {
+                            const float r = (!MASK || okr[i]) ? (float)(half_t)(g.alpha * acc[i][j][v]) : 0.0f;
+                            a += r;
+                            q += r * r;
+                        }
                     }
                     sv[j * 16 + v] = a;
                     qv[j * 16 + v] = q;
@@ -870,8 +882,15 @@ __global__ void __launch_bounds__(64 * (WGM * WGN + PROD), (BQ && WGM * WGN + PR
     // rowoff + a term that is the same for every lane (kept in scalar registers), and which
     // taps fall inside the image is one bit each of a 64-bit mask computed once per row.
     const int sy = BWD ? -1 : g.dil;
+    // a 1x1 filter of stride 1 without padding reads input pixel m for output pixel m: no decoding, one tap
+    const bool plain = g.R == 1 && g.S == 1 && g.pad == 0 && g.stride == 1 && g.IH == g.OH && g.IW == g.OW;
     auto row_setup = [&](int m, int kvv, int &ro, unsigned long long &mask) {
         bool ok = m < Mloc;
+        if(plain) {
+            ro = ((ok ? m : 0) * g.lda + kvv) * 2;
+            mask = ok ? 1ull : 0ull;
+            return;
+        }
         const int mm = ok ? m : 0;
         const int ox = mm % PW;
         const int t = mm / PW;

@@ -1461,7 +1461,8 @@ void spatialtransform_setup(HipProgram &p, HipProgramUnit &pu, const Node &n)
     auto theta = p.lower(pu, th);
     if(theta->m_data_type != Tensor::DataType::FLOAT || theta->m_dims.elements() != (size_t)(int)x->m_dims[0] * 6 ||
        !theta->rowMajor())
-        throw std::runtime_error("spatialtransform: theta must be an fp32 [N,2,3] tensor");
+        throw std::runtime_error("spatialtransform: theta must be an fp32 [N,2,3] tensor in row-major order (got " +
+                                 theta->info() + " for x " + x->info() + ")");
     if(x->m_data_type != y->m_data_type ||
        (x->m_data_type != Tensor::DataType::FLOAT && x->m_data_type != Tensor::DataType::HALF))
         throw std::runtime_error("spatialtransform: x and y must both be fp32 or both fp16");

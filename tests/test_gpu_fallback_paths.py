@@ -19,7 +19,7 @@ CONV = "test_conv_fwd_bwd or test_conv_golden or test_transposed_conv or test_co
 CASES = [
     ("SAGA_HIP_CONV_STAGES", "0", ["tests/test_gpu_ops.py", "-k", CONV]),
     # (without the pipelined kernels there is no batch-norm backward link to count)
-    ("SAGA_HIP_CONV_STAGES", "0", ["tests/test_gpu_networks.py", "-k", "not links"]),
+    ("SAGA_HIP_CONV_STAGES", "0", ["tests/test_gpu_networks.py", "-k", "not link"]),
     ("SAGA_HIP_FORCE_DIRECT", "1", ["tests/test_gpu_ops.py", "-k", CONV]),
     ("SAGA_HIP_F32_NO_UNIFORM", "1", ["tests/test_gpu_ops.py", "-k", CONV]),
     ("SAGA_HIP_BN_MASK_FROM_Y", "1", ["tests/test_gpu_networks.py"]),
