@@ -2011,13 +2011,6 @@ template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
             // at most 64 output channels: 256x64 on four wavefronts, which then hold five load
             // instructions per eight MFMAs each - four more wavefronts take the loads over (5-8 % faster)
             tile = g.Ngemm <= 64 ? 13 : 5;
-            // ... and 128x64 on four wavefronts (four blocks per CU instead of two) where the reduction is short or
-            // re-reads its input from L2 tap after tap: the 3x3 layers with 64 output channels, the stem's virtual
-            // 7-tap convolution and 64 -> 64 1x1 (measured 9-15 % faster forward, 2-9 % with the statistics
-            // epilogue, 3 % backward; the 1x1 layers with 256 input channels stream 4x the input and keep the
-            // producer wavefronts)
-            if(tile == 13 && (g.R * g.S > 1 || g.Cred <= 64))
-                tile = 14;
             // at most one block per CU: nothing else on the CU hides the time a wavefront spends
             // issuing its loads, so four extra wavefronts per block do the issuing (measured
             // 5-15 % faster on the 7x7-pixel layers of ResNet-50, slower once CUs hold two blocks)
@@ -2060,7 +2053,6 @@ template <bool BWD> static int launch_gather(GatherArgs &g, hipStream_t st)
         case 5: LAUNCH(256, 128, 4, 2, 32, 0); break;
         case 12: LAUNCH(256, 128, 4, 2, 32, 4); break;
         case 13: LAUNCH(256, 64, 4, 1, 32, 4); break;
-        case 14: LAUNCH(128, 64, 4, 1, 32, 0); break;
         default: LAUNCH(256, 64, 4, 1, 32, 0); break;
         }
 #undef LAUNCH
