@@ -423,7 +423,8 @@ __global__ void __launch_bounds__(256) maxpool_fwd_codes_k(DView x, DView y, uin
     } else {
         packed = code[0] | code[1] << 8 | code[2] << 16 | code[3] << 24;
     }
-    *(typename CodeVec<VN>::type *)(codes + ((((size_t)n * P + p) * Q + q) * C + c)) = packed;
+    if(codes)
+        *(typename CodeVec<VN>::type *)(codes + ((((size_t)n * P + p) * Q + q) * C + c)) = packed;
 }
 
 // floor(a / S) for a that may be negative, S a compile-time constant
@@ -573,6 +574,10 @@ static int pool_dim(int in, int k, int pad, int stride) { return 1 + (in + 2 * p
 
 } // namespace
 
+static bool codes_ok(const SagaTensorView *a, const SagaTensorView *b, int size, int pad, int stride);
+static void launch_maxpool_codes(const SagaTensorView *x, const SagaTensorView *y, uint8_t *codes, int size, int pad,
+                                 int stride, hipStream_t st);
+
 extern "C" {
 
 int saga_hip_pool_fwd(int mode, const SagaTensorView *x, const SagaTensorView *y, const SagaTensorView *idx,
@@ -591,6 +596,14 @@ int saga_hip_pool_fwd(int mode, const SagaTensorView *x, const SagaTensorView *y
     const int64_t total = view_elements(y) / vn;
     const int g = grid_for(total, 256, 256 * 32);
     hipStream_t st = as_stream(stream);
+    // max pooling without indices over 2x2 / 3x3 windows of a channels-last tensor: the kernel of the training
+    // variant, which has all loads of a window in flight at once (no division in the work mapping), without its
+    // position codes (the 112x112 stem output of ResNet-50 b256: 150 -> 110 us)
+    if(mode == SAGA_POOL_MAX && !idx && codes_ok(x, y, size, pad, stride)) {
+        launch_maxpool_codes(x, y, nullptr, size, pad, stride, st);
+        SAGA_CHECK_LAUNCH();
+        return 0;
+    }
     DView dvx = dview(x), dvy = dview(y), dvi = idx ? dview(idx) : dview(y);
 #define GO(T, VN)                                                                                        \
     do {                                                                                                 \
@@ -703,10 +716,19 @@ int saga_hip_maxpool_fwd_codes(const SagaTensorView *x, const SagaTensorView *y,
         return SAGA_HIP_ESHAPE;
     if(!codes_ok(x, y, size, pad, stride) || ((uintptr_t)codes & 7))
         return SAGA_HIP_EUNSUPPORTED;
+    launch_maxpool_codes(x, y, codes, size, pad, stride, as_stream(stream));
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
+} // extern "C"
+
+static void launch_maxpool_codes(const SagaTensorView *x, const SagaTensorView *y, uint8_t *codes, int size, int pad,
+                                 int stride, hipStream_t st)
+{
     const int vn = x->dtype == SAGA_HALF ? 8 : 4;
     dim3 grid, block;
     codes_launch_shape(y->dims[1] / vn, y->dims[3], y->dims[2], y->dims[0], grid, block);
-    hipStream_t st = as_stream(stream);
     const DView dvx = dview(x), dvy = dview(y);
 #define GO2(T, VN, K, S) maxpool_fwd_codes_k<T, VN, K, S><<<grid, block, 0, st>>>(dvx, dvy, codes, pad)
 #define GO(T, VN)                                                                                              \
@@ -725,9 +747,9 @@ int saga_hip_maxpool_fwd_codes(const SagaTensorView *x, const SagaTensorView *y,
         GO(float, 4);
 #undef GO
 #undef GO2
-    SAGA_CHECK_LAUNCH();
-    return 0;
 }
+
+extern "C" {
 
 int saga_hip_maxpool_bwd_codes(const uint8_t *codes, const SagaTensorView *dy, const SagaTensorView *dx, int size, int pad,
                                int stride, float beta, saga_stream_t stream)
