@@ -70,6 +70,7 @@ struct GatherArgs {
     int bq_relu;
     float *bq_partial;  // null: no link
     int no_stage;      // the epilogue stores straight from registers (experiment switch SAGA_HIP_NO_STAGED_STORES)
+    unsigned out_bytes; // extent of out, for the epilogue variant that stores through a range-checked buffer (BUFST)
     float *stats;      // forward only, optional: per block row and output channel, sum and sum of
                        // squares of the stored outputs, [ceil(M / BM)][Ngemm][2]
     int stats_rows;    // out: block rows the launch wrote
@@ -382,13 +383,99 @@ __device__ __forceinline__ void halve_exchange(float (&a)[NV], float (&b)[NV], i
 // reuse once every wavefront has left the main loop (the barriers inside see to that).
 // whether gather_epilogue stores through LDS (the producer wavefronts of a block count its barriers)
 // (not the 64-channel tiles: their rows are 128 bytes to begin with and the detour measured 3 - 7 % slower)
+// Per-channel sum and sum of squares of a wavefront's outputs (as stored, i.e. rounded to fp16), for a batch
+// normalisation that follows.  Columns past Ngemm hold zeros in the accumulators and add nothing; so do rows that
+// are not ok unless MASK says they may hold anything, in which case they are left out here.  Lanes of one
+// half-wave hold different pixels of the same channels: a halving exchange (each step swaps half of the values
+// with the lane 16, 8, .. 1 away) leaves every lane - every even lane for 32-channel tiles - with the totals of
+// one channel, stats_channel() of the wave tile.
+template <int TM, int TN, bool MASK>
+__device__ __forceinline__ void stats_lane_totals(float alpha, float16_t (&acc)[TM][TN], const bool (&okr)[TM], int lane,
+                                                  float &s_out, float &q_out)
+{
+    constexpr int NV = TN * 16;
+    static_assert(NV == 16 || NV == 32, "stats layout");
+    float sv[NV], qv[NV];
+#pragma unroll
+    for(int j = 0; j < TN; j++)
+#pragma unroll
+        for(int v = 0; v < 16; v++) {
+            float a = 0.0f, q = 0.0f;
+            if constexpr(TM == 2) {
+                // the two rows of a channel rounded to fp16 as they are stored, in one packed register;
+                // sum and sum of squares are one two-element dot product each (fp32 result)
+                typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+                h2 pr;
+                pr[0] = (!MASK || okr[0]) ? (_Float16)(alpha * acc[0][j][v]) : (_Float16)0;
+                pr[1] = (!MASK || okr[1]) ? (_Float16)(alpha * acc[1][j][v]) : (_Float16)0;
+                const h2 ones = {(_Float16)1, (_Float16)1};
+                a = __builtin_amdgcn_fdot2(pr, ones, 0.0f, false);
+                q = __builtin_amdgcn_fdot2(pr, pr, 0.0f, false);
+            } else {
+#pragma unroll
+                for(int i = 0; i < TM; i++) {
+                    const float r = (!MASK || okr[i]) ? (float)(half_t)(alpha * acc[i][j][v]) : 0.0f;
+                    a += r;
+                    q += r * r;
+                }
+            }
+            sv[j * 16 + v] = a;
+            qv[j * 16 + v] = q;
+        }
+    if constexpr(NV == 32) {
+        halve_exchange<32, 16>(sv, qv, lane);
+        halve_exchange<16, 8>(sv, qv, lane);
+        halve_exchange<8, 4>(sv, qv, lane);
+        halve_exchange<4, 2>(sv, qv, lane);
+        halve_exchange<2, 1>(sv, qv, lane);
+    } else {
+        halve_exchange<16, 16>(sv, qv, lane);
+        halve_exchange<8, 8>(sv, qv, lane);
+        halve_exchange<4, 4>(sv, qv, lane);
+        halve_exchange<2, 2>(sv, qv, lane);
+        sv[0] += dpp_read<0xb1>(sv[0]);
+        qv[0] += dpp_read<0xb1>(qv[0]);
+    }
+    s_out = sv[0];
+    q_out = qv[0];
+}
+
+// The wavefronts stacked along M are added through LDS (red: WGM * BN pairs) in a fixed order and the block's
+// [channel][2] row goes to g.stats[stats_row].  The caller has made sure that nobody still reads what red overlays.
+template <int TN, int WGM, int WGN, int BN>
+__device__ __forceinline__ void stats_block_write(const GatherArgs &g, char *red_mem, int tid, int lane, int wave, int wn,
+                                                  int n0, int stats_row, float s0, float q0)
+{
+    constexpr int NV = TN * 16;
+    const int hi = lane >> 5;
+    const int idx = NV == 32 ? (lane & 31) : (lane & 31) >> 1;
+    const int chl = 32 * (idx >> 4) + 8 * ((idx & 15) >> 2) + 4 * hi + (idx & 3); // channel inside the wave tile
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    float2_t *red = (float2_t *)red_mem;
+    if(NV == 32 || (lane & 1) == 0) {
+        float2_t v2 = {s0, q0};
+        red[(wave / WGN) * BN + wn + chl] = v2;
+    }
+    __syncthreads();
+    if(tid < BN && n0 + tid < g.Ngemm) {
+        float2_t t = red[tid];
+#pragma unroll
+        for(int wy = 1; wy < WGM; wy++)
+            t += red[wy * BN + tid];
+        *(float2_t *)(g.stats + ((int64_t)stats_row * g.Ngemm + n0 + tid) * 2) = t;
+    }
+}
+
 template <int TM, int TN, int BN, bool BWD> __device__ __forceinline__ bool stores_staged(const GatherArgs &g)
 {
     const bool vec_ok = (g.ldo & 7) == 0 && (g.Ngemm & 7) == 0 && ((uintptr_t)g.out & 15) == 0;
     return TM == 2 && TN == 2 && BN >= 128 && vec_ok && !(BWD && g.classes > 1) && !g.no_stage;
 }
 
-template <int TM, int TN, int WGM, int WGN, int BN, bool BWD, bool MASK, typename RowPix>
+// BUFST: the direct 16-byte stores go through a range-checked buffer with an out-of-range offset for the lanes that
+// have nothing to store, so that every wavefront issues the same number of store instructions whatever its rows
+// (a caller that counts outstanding memory operations needs that).
+template <int TM, int TN, int WGM, int WGN, int BN, bool BWD, bool MASK, bool BUFST = false, typename RowPix>
 __device__ __forceinline__ void gather_epilogue(const GatherArgs &g, float16_t (&acc)[TM][TN], char *smem, int tid, int lane,
                                                 int wave, int wm, int wn, int n0, int stats_row, RowPix rowpix)
 {
@@ -478,7 +565,11 @@ __device__ __forceinline__ void gather_epilogue(const GatherArgs &g, float16_t (
                     const int n = nb + 16 * q + 8 * hi;
                     typedef unsigned u4 __attribute__((ext_vector_type(4)));
                     const u4 o = {s0_[0], s1_[0], s0_[1], s1_[1]};
-                    if(staged) {
+                    if constexpr(BUFST) {
+                        const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc((void *)g.out, 0, g.out_bytes, 0x00020000);
+                        const unsigned off = (ok && n < g.Ngemm) ? (unsigned)((pix * g.ldo + n) * 2) : 0x7fffff00u;
+                        __builtin_amdgcn_raw_buffer_store_b128(o, ro, off, 0, 0);
+                    } else if(staged) {
                         const int row = i * 32 + (lane & 31), chunk = 4 * j + 2 * q + hi;
                         *(u4 *)(stg + row * (TN * 64) + ((chunk ^ (row & 7)) << 4)) = o;
                     } else if(ok && n < g.Ngemm) {
@@ -533,75 +624,15 @@ __device__ __forceinline__ void gather_epilogue(const GatherArgs &g, float16_t (
             }
         }
     }
-    // Optional: per-channel sum and sum of squares of this block's outputs (as stored, i.e.
-    // rounded to fp16), for a batch normalisation that follows.  Columns past Ngemm hold zeros in
-    // the accumulators and add nothing; so do rows that are not ok unless MASK says they may hold
-    // anything, in which case they are left out here.  Lanes of one half-wave hold
-    // different pixels of the same channels: a halving exchange (each step swaps half of the
-    // values with the lane 16, 8, .. 1 away) leaves every lane with the total of one channel;
-    // the wavefronts stacked along M are then added through LDS in a fixed order.
+    // Optional: per-channel sum and sum of squares of this block's outputs, for a batch normalisation that follows
+    // (stats_lane_totals, stats_block_write).
     if constexpr(!BWD) {
         if(g.stats) {
-            constexpr int NV = TN * 16;
-            static_assert(NV == 16 || NV == 32, "stats layout");
-            float sv[NV], qv[NV];
-#pragma unroll
-            for(int j = 0; j < TN; j++)
-#pragma unroll
-                for(int v = 0; v < 16; v++) {
-                    float a = 0.0f, q = 0.0f;
-                    if constexpr(TM == 2) {
-                        // the two rows of a channel rounded to fp16 as they are stored, in one packed register;
-                        // sum and sum of squares are one two-element dot product each (fp32 result)
-                        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-                        h2 pr;
-                        pr[0] = (!MASK || okr[0]) ? (_Float16)(g.alpha * acc[0][j][v]) : (_Float16)0;
-                        pr[1] = (!MASK || okr[1]) ? (_Float16)(g.alpha * acc[1][j][v]) : (_Float16)0;
-                        const h2 ones = {(_Float16)1, (_Float16)1};
-                        a = __builtin_amdgcn_fdot2(pr, ones, 0.0f, false);
-                        q = __builtin_amdgcn_fdot2(pr, pr, 0.0f, false);
-                    } else {
-#pragma unroll
-                        for(int i = 0; i < TM; i++) {
-                            const float r = (!MASK || okr[i]) ? (float)(half_t)(g.alpha * acc[i][j][v]) : 0.0f;
-                            a += r;
-                            q += r * r;
-                        }
-                    }
-                    sv[j * 16 + v] = a;
-                    qv[j * 16 + v] = q;
-                }
-            if constexpr(NV == 32) {
-                halve_exchange<32, 16>(sv, qv, lane);
-                halve_exchange<16, 8>(sv, qv, lane);
-                halve_exchange<8, 4>(sv, qv, lane);
-                halve_exchange<4, 2>(sv, qv, lane);
-                halve_exchange<2, 1>(sv, qv, lane);
-            } else {
-                halve_exchange<16, 16>(sv, qv, lane);
-                halve_exchange<8, 8>(sv, qv, lane);
-                halve_exchange<4, 4>(sv, qv, lane);
-                halve_exchange<2, 2>(sv, qv, lane);
-                sv[0] += dpp_read<0xb1>(sv[0]);
-                qv[0] += dpp_read<0xb1>(qv[0]);
-            }
-            const int idx = NV == 32 ? (lane & 31) : (lane & 31) >> 1;
-            const int chl = 32 * (idx >> 4) + 8 * ((idx & 15) >> 2) + 4 * hi + (idx & 3); // channel inside the wave tile
-            typedef float float2_t __attribute__((ext_vector_type(2)));
-            float2_t *red = (float2_t *)(smem + WGM * WGN * TM * 32 * TN * 64);
+            float s0, q0;
+            stats_lane_totals<TM, TN, MASK>(g.alpha, acc, okr, lane, s0, q0);
             __syncthreads(); // every wavefront is done reading the last slice (and the folded norm's table)
-            if(NV == 32 || (lane & 1) == 0) {
-                float2_t v2 = {sv[0], qv[0]};
-                red[(wave / WGN) * BN + wn + chl] = v2;
-            }
-            __syncthreads();
-            if(tid < BN && n0 + tid < g.Ngemm) {
-                float2_t t = red[tid];
-#pragma unroll
-                for(int wy = 1; wy < WGM; wy++)
-                    t += red[wy * BN + tid];
-                *(float2_t *)(g.stats + ((int64_t)stats_row * g.Ngemm + n0 + tid) * 2) = t;
-            }
+            stats_block_write<TN, WGM, WGN, BN>(g, smem + WGM * WGN * TM * 32 * TN * 64, tid, lane, wave, wn, n0, stats_row,
+                                                s0, q0);
         }
     }
 }
@@ -1849,19 +1880,27 @@ __global__ void __launch_bounds__(256)
              int Wp, int64_t total)
 {
     typedef _Float16 h4 __attribute__((ext_vector_type(4)));
-    for(int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
-        const int wp = (int)(i % Wp);
-        const int64_t t = i / Wp;
-        const int hp = (int)(t % Hp);
-        const int64_t n = t / Hp;
+    // (total < 2^31, checked by thin_ok: 32-bit index arithmetic - the 64-bit divisions were most of this kernel)
+    const unsigned tot = (unsigned)total, step = gridDim.x * blockDim.x;
+    for(unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < tot; i += step) {
+        const unsigned t = i / (unsigned)Wp;
+        const int wp = (int)(i - t * (unsigned)Wp);
+        const unsigned n = t / (unsigned)Hp;
+        const int hp = (int)(t - n * (unsigned)Hp);
         const int h = hp - pad, w = wp - pad;
         h4 v = {0, 0, 0, 0};
         if(h >= 0 && h < H && w >= 0 && w < W) {
-            const half_t *src = x + ((n * H + h) * W + w) * sp;
-            for(int c = 0; c < C; c++)
-                v[c] = src[c];
+            const half_t *src = x + (((int64_t)n * H + h) * W + w) * sp;
+            if(C == 3) {
+                v[0] = src[0];
+                v[1] = src[1];
+                v[2] = src[2];
+            } else {
+                for(int c = 0; c < C; c++)
+                    v[c] = src[c];
+            }
         }
-        *(h4 *)(x4 + i * 4) = v;
+        *(h4 *)(x4 + (size_t)i * 4) = v;
     }
 }
 
@@ -1914,6 +1953,18 @@ __global__ void __launch_bounds__(256)
     }
 }
 
+static int num_cus()
+{
+    static int v = 0;
+    if(v <= 0) {
+        int d = 0;
+        if(hipGetDevice(&d) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, d) != hipSuccess ||
+           v <= 0)
+            v = 256;
+    }
+    return v;
+}
+
 struct ThinGeom {
     int Hp, Wp;
     size_t x4_bytes, wv_bytes;
@@ -1931,6 +1982,203 @@ static bool thin_ok(const ConvGeom &g, ThinGeom *t)
     t->x4_bytes = ((size_t)px * 8 + 255) & ~(size_t)255;
     t->wv_bytes = ((size_t)g.K * g.R * 32 * sizeof(half_t) + 255) & ~(size_t)255;
     return true;
+}
+
+// ---------------------------------------------------------------- thin inputs, whole image rows in LDS
+//
+// The "virtual" convolution of a thin input (above: x4[N][Hp][Wp][4], windows of 8 pixels = 32 halves per filter
+// row) run through the gather kernel loads every output pixel's 64-byte window separately, and neighbouring
+// windows overlap by 48 of their 64 bytes: the LDS fill is four times the input, a block lives for R short
+// slices, and with two blocks per CU the loop is bound by the latency of those fills (RGB stem of ResNet-50:
+// 264 us for 92 GFLOP and 520 MB).  Here a block owns TR whole output rows of one image (TR * Q <= 256 pixels),
+// copies the (TR - 1) * stride + R padded input rows they read ONCE into LDS as they are, and an MFMA operand -
+// 8 halves of pixel window (oy, ox), filter row r - is the 16 bytes at
+//     (orow * stride + r) * row_bytes + ox * stride * 8 + 16 * (k / 8)
+// of that copy: overlapping windows are overlapping reads.  The filter (64 output channels x R x 32 halves) stays
+// in registers for the whole launch; blocks are persistent and walk the tiles grid-strided with two LDS buffers,
+// the rows of the tile after next being requested while the current one is multiplied.  Order inside one
+// iteration: multiply tile t - wait for everything outstanding (the rows of t + 1 and the stores of t - 1, both
+// issued a whole multiplication ago; loads and stores retire through one in-order counter) - barrier - store
+// tile t - request the rows of t + 2 into the buffer that t was read from.
+constexpr int THIN_ROWS_DEPTH = 4; // tiles whose rows are in LDS or on their way
+struct ThinRowsArgs {
+    int TR;          // output rows per tile
+    int tpi;         // tiles per image
+    int ntiles;
+    int npix;        // TR * Q
+    int Hp;          // rows of the padded input per image
+    int row_bytes;   // bytes per padded input row
+    int chunks_row;  // 16-byte chunks per input row
+    int chunks_tile; // chunks_row * input rows per tile
+    int buf_bytes;   // one LDS buffer: a tile's rows, rounded up to the 1 KB a load instruction fills
+    int epi_off;     // where the epilogue's LDS scratch starts, minus what gather_epilogue adds itself
+};
+
+// MODE: 0 plain (alpha, beta), 1 folded inference batch norm, 2 batch-norm statistics - one instantiation each, so
+// that the register allocation of one epilogue does not pay for the others.
+template <int R, int MODE> __global__ void __launch_bounds__(256, 2) conv_thin_rows(GatherArgs g, ThinRowsArgs t)
+{
+    if constexpr(MODE != 1)
+        g.bn_s = nullptr;
+    // (statistics: every lane keeps the running totals of one channel over the tiles its block walks, and the block
+    // leaves ONE partial row at the end - no barrier or LDS round trip per tile, and a finalize step that adds a few
+    // hundred rows instead of one per tile)
+    float *const stats = MODE == 2 ? g.stats : nullptr;
+    g.stats = nullptr;
+    float run_s = 0.0f, run_q = 0.0f;
+    if constexpr(MODE != 0)
+        g.beta = 0.0f;
+    constexpr int TM = 2, TN = 2, NLD_MAX = 8, D = THIN_ROWS_DEPTH;
+    constexpr unsigned OOB = 0x7fffff00u;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int hi = lane >> 5;
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void *)g.a, 0, g.a_bytes, 0x00020000);
+
+    // the filter: fragment (r, kk, j) = halves 16*kk + 8*hi .. +8 of filter row r of output channel 32*j + lane%32
+    half8_t fb[R][2][TN];
+#pragma unroll
+    for(int j = 0; j < TN; j++) {
+        const int o = j * 32 + (lane & 31);
+        const bool ok = o < g.Ngemm;
+        const half_t *src = g.b + ((int64_t)(ok ? o : 0) * R) * 32 + hi * 8;
+#pragma unroll
+        for(int r = 0; r < R; r++)
+#pragma unroll
+            for(int kk = 0; kk < 2; kk++) {
+                const half8_t v = *(const half8_t *)(src + r * 32 + kk * 16);
+                const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+                fb[r][kk][j] = ok ? v : zero;
+            }
+    }
+    // Chunk (q * 4 + wave) * 64 + lane of a tile's rows is this lane's share of load q; its place in the padded
+    // input relative to the tile's first row is the same for every tile.  (Recomputed for every request rather
+    // than kept: registers are what limits this kernel, and a value spilled here would be reloaded behind the
+    // epilogue's stores.)  A wavefront issues my_nld loads per tile - those with at least one chunk of the tile.
+    const int c0 = wave * 64 + lane;
+    const int row0 = c0 / t.chunks_row, col0 = c0 - row0 * t.chunks_row;
+    const int my_nld = t.chunks_tile > wave * 64 ? (t.chunks_tile - wave * 64 + 255) / 256 : 0;
+    auto request = [&](int tile, int b) {
+        const int n = tile / t.tpi;
+        const int oy0 = (tile - n * t.tpi) * t.TR;
+        const int base = (n * t.Hp + oy0 * g.stride) * t.row_bytes; // (the whole padded input is below 2 GB)
+        char *dst = smem + b * t.buf_bytes + wave * 1024;
+        // chunk c0 + 256 q: 256 chunks further on is rows256 rows and cols256 columns further on, with a carry
+        const int rows256 = 256 / t.chunks_row, cols256 = 256 - rows256 * t.chunks_row;
+        int row = row0, col = col0;
+#pragma unroll
+        for(int q = 0; q < NLD_MAX; q++)
+            if(q < my_nld) {
+                const unsigned off = c0 + 256 * q < t.chunks_tile ? (unsigned)(row * t.row_bytes + col * 16) : OOB;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(dst + q * 4096), 16, off, base, 0, 0);
+                row += rows256;
+                col += cols256;
+                if(col >= t.chunks_row) {
+                    col -= t.chunks_row;
+                    row++;
+                }
+            }
+    };
+    // this lane's two pixels (row blocks i of the wavefront's 64) inside a tile, as byte offsets into the LDS copy
+    int abase[TM];
+#pragma unroll
+    for(int i = 0; i < TM; i++) {
+        const int p = wave * 64 + i * 32 + (lane & 31);
+        const int pp = p < t.npix ? p : 0;
+        const int orow = pp / g.OW;
+        abase[i] = orow * g.stride * t.row_bytes + (pp - orow * g.OW) * g.stride * 8 + hi * 16;
+    }
+    char *epi = smem + t.epi_off;
+    const int G = gridDim.x;
+
+    // each die's blocks take neighbouring tiles, which share input rows: the die's L2 then fetches those rows once
+    int tile = xcd_remap(blockIdx.x, G);
+    const int first_tile = tile; // also the block's row in the statistics
+#pragma unroll
+    for(int d = 0; d < D; d++)
+        if(tile + d * G < t.ntiles)
+            request(tile + d * G, d);
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    int b = 0; // buffer of the current tile
+    for(; tile < t.ntiles; tile += G) {
+        const char *buf = smem + b * t.buf_bytes;
+        float16_t acc[TM][TN];
+#pragma unroll
+        for(int i = 0; i < TM; i++)
+#pragma unroll
+            for(int j = 0; j < TN; j++)
+#pragma unroll
+                for(int v = 0; v < 16; v++)
+                    acc[i][j][v] = 0.0f;
+#pragma unroll
+        for(int r = 0; r < R; r++) {
+            half8_t fa[2][TM];
+#pragma unroll
+            for(int kk = 0; kk < 2; kk++)
+#pragma unroll
+                for(int i = 0; i < TM; i++)
+                    fa[kk][i] = *(const half8_t *)(buf + abase[i] + r * t.row_bytes + kk * 32);
+#pragma unroll
+            for(int kk = 0; kk < 2; kk++)
+#pragma unroll
+                for(int i = 0; i < TM; i++)
+#pragma unroll
+                    for(int j = 0; j < TN; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[r][kk][j], fa[kk][i], acc[i][j], 0, 0, 0);
+        }
+        // The rows of the NEXT tile must have arrived before the barrier that lets everybody read them.  This
+        // wavefront's memory operations retire in order, and behind those rows it has issued, per tile, NST stores
+        // (the epilogue's, always all of them: BUFST) and its my_nld loads, for D - 2 tiles: those may stay in flight,
+        // so neither the stores nor the later rows are waited for until they are two multiplications old.  Near the
+        // end of the walk fewer operations are behind the rows, and the wait is for everything.
+        constexpr int NST = TM * TN * 2;
+        if(tile + (D - 1) * G < t.ntiles) {
+            switch(my_nld) {
+            case 0: asm volatile("s_waitcnt vmcnt(%0)" ::"n"((0 + NST) * (D - 2)) : "memory"); break;
+            case 1: asm volatile("s_waitcnt vmcnt(%0)" ::"n"((1 + NST) * (D - 2)) : "memory"); break;
+            case 2: asm volatile("s_waitcnt vmcnt(%0)" ::"n"((2 + NST) * (D - 2)) : "memory"); break;
+            case 3: asm volatile("s_waitcnt vmcnt(%0)" ::"n"((3 + NST) * (D - 2)) : "memory"); break;
+            case 4: asm volatile("s_waitcnt vmcnt(%0)" ::"n"((4 + NST) * (D - 2)) : "memory"); break;
+            case 5: asm volatile("s_waitcnt vmcnt(%0)" ::"n"((5 + NST) * (D - 2)) : "memory"); break;
+            case 6: asm volatile("s_waitcnt vmcnt(%0)" ::"n"((6 + NST) * (D - 2)) : "memory"); break;
+            case 7: asm volatile("s_waitcnt vmcnt(%0)" ::"n"((7 + NST) * (D - 2)) : "memory"); break;
+            default: asm volatile("s_waitcnt vmcnt(%0)" ::"n"((8 + NST) * (D - 2)) : "memory"); break;
+            }
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        asm volatile("s_barrier" ::: "memory");
+        const int n = tile / t.tpi;
+        const int oy0 = (tile - n * t.tpi) * t.TR;
+        const int64_t pix0 = ((int64_t)n * g.OH + oy0) * g.OW;
+        auto rowpix = [&](int mrow, bool &ok, int64_t &pix) {
+            ok = mrow < t.npix && oy0 + mrow / g.OW < g.OH;
+            pix = pix0 + (ok ? mrow : 0);
+        };
+        gather_epilogue<TM, TN, 4, 1, 64, false, true, true>(g, acc, epi, tid, lane, wave, wave * 64, 0, 0, tile, rowpix);
+        if constexpr(MODE == 2) {
+            bool okr[TM];
+#pragma unroll
+            for(int i = 0; i < TM; i++) {
+                int64_t pix;
+                rowpix(wave * 64 + i * 32 + (lane & 31), okr[i], pix);
+            }
+            float s0, q0;
+            stats_lane_totals<TM, TN, true>(g.alpha, acc, okr, lane, s0, q0);
+            run_s += s0;
+            run_q += q0;
+        }
+        // every wavefront is past the barrier, so nobody reads this tile's buffer any more
+        if(tile + D * G < t.ntiles)
+            request(tile + D * G, b);
+        b = b + 1 == D ? 0 : b + 1;
+    }
+    if constexpr(MODE == 2) {
+        g.stats = stats;
+        __syncthreads();
+        stats_block_write<TN, 4, 1, 64>(g, epi + 32768, tid, lane, wave, 0, 0, first_tile, run_s, run_q);
+    }
 }
 
 // out[row][0..C) = 0 for rows of pitch `pitch` elements (C and pitch multiples of 8, 16-byte aligned)
@@ -2198,7 +2446,7 @@ int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTe
             return SAGA_HIP_EWORKSPACE;
         half_t *x4 = (half_t *)ws, *wv = (half_t *)((char *)ws + tg.x4_bytes);
         const int64_t px = (int64_t)g.N * tg.Hp * tg.Wp, wn = (int64_t)g.K * g.R * 32;
-        pad_thin<<<grid_for(px, 256, 256 * 16), 256, 0, st>>>((const half_t *)x->ptr, lx.pitch, g.C, g.H, g.W, g.pad, x4,
+        pad_thin<<<grid_for(px, 256, 1 << 20), 256, 0, st>>>((const half_t *)x->ptr, lx.pitch, g.C, g.H, g.W, g.pad, x4,
                                                               tg.Hp, tg.Wp, px);
         repack_thin_filter<<<grid_for(wn, 256, 256 * 16), 256, 0, st>>>((const half_t *)w->ptr, wv, g.C, g.S, wn);
         GatherArgs a;
@@ -2220,6 +2468,59 @@ int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTe
         a.bq_partial = nullptr;
         if(!set_bn(a, bn, y, ly))
             return SAGA_HIP_EUNSUPPORTED;
+        // whole rows in LDS (conv_thin_rows): 7-row filters into at most 64 channels, output rows of at most 256 pixels
+        static const bool rows_off = getenv("SAGA_HIP_THIN_ROWS") && atoi(getenv("SAGA_HIP_THIN_ROWS")) == 0;
+        if(!rows_off && g.R == 7 && g.K <= 64 && g.Q <= 256) {
+            ThinRowsArgs t;
+            t.TR = 256 / g.Q;
+            if(t.TR > g.P)
+                t.TR = g.P;
+            t.tpi = (g.P + t.TR - 1) / t.TR;
+            t.ntiles = g.N * t.tpi;
+            t.npix = t.TR * g.Q;
+            t.Hp = tg.Hp;
+            t.row_bytes = tg.Wp * 8;
+            t.chunks_row = t.row_bytes / 16;
+            t.chunks_tile = t.chunks_row * ((t.TR - 1) * g.stride + g.R);
+            t.buf_bytes = (t.chunks_tile * 16 + 1023) & ~1023;
+            const int epi_at = std::max(THIN_ROWS_DEPTH * t.buf_bytes, 32768); // gather_epilogue's scratch sits 32 KB behind its base
+            t.epi_off = epi_at - 32768;
+            const int lds = epi_at + 4096;
+            const bool vec_ok = (ly.pitch & 7) == 0 && (g.K & 7) == 0 && aligned16(y->ptr) &&
+                                ((ly.rows - 1) * ly.pitch + g.K) * 2 < 0x7fffff00ll;
+            const bool fits = vec_ok && t.chunks_tile <= 8 * 256 && lds <= 76 * 1024 && t.row_bytes % 16 == 0 &&
+                              (!stats || (size_t)std::min(t.ntiles, 2 * num_cus()) * g.K * 2 <= stats_floats) &&
+                              // the last window of a row ends inside the row's copy
+                              ((g.Q - 1) * g.stride + 8) * 8 <= t.row_bytes;
+            if(fits) {
+                static bool once = false;
+                if(!once) {
+                    for(const void *k : {(const void *)conv_thin_rows<7, 0>, (const void *)conv_thin_rows<7, 1>,
+                                         (const void *)conv_thin_rows<7, 2>}) {
+                        const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 76 * 1024);
+                        if(e != hipSuccess)
+                            return (int)e;
+                    }
+                    once = true;
+                }
+                a.classes = 1;
+                a.no_stage = 1;
+                a.out_bytes = (unsigned)(((ly.rows - 1) * ly.pitch + g.K) * 2); // rows * pitch < 2^31 on this path
+                a.nblk_n = 1;
+                const int blocks = std::min(t.ntiles, 2 * num_cus());
+                a.stats_rows = blocks;
+                if(a.bn_s)
+                    conv_thin_rows<7, 1><<<blocks, 256, lds, st>>>(a, t);
+                else if(a.stats)
+                    conv_thin_rows<7, 2><<<blocks, 256, lds, st>>>(a, t);
+                else
+                    conv_thin_rows<7, 0><<<blocks, 256, lds, st>>>(a, t);
+                SAGA_CHECK_LAUNCH();
+                if(stats_rows)
+                    *stats_rows = a.stats_rows;
+                return 0;
+            }
+        }
         const int rc = launch_gather<false>(a, st);
         if(stats_rows)
             *stats_rows = a.stats_rows;
@@ -2394,7 +2695,7 @@ int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, cons
             return SAGA_HIP_EUNSUPPORTED;
         half_t *x4 = (half_t *)ws;
         const int64_t px = (int64_t)g.N * tg.Hp * tg.Wp;
-        pad_thin<<<grid_for(px, 256, 256 * 16), 256, 0, st>>>((const half_t *)x->ptr, lx.pitch, g.C, g.H, g.W, g.pad, x4,
+        pad_thin<<<grid_for(px, 256, 1 << 20), 256, 0, st>>>((const half_t *)x->ptr, lx.pitch, g.C, g.H, g.W, g.pad, x4,
                                                               tg.Hp, tg.Wp, px);
         FilterArgs a;
         a.x = x4;

@@ -47,6 +47,9 @@ CONV_CASES = [
     (1, 3, 21, 21, 72, 8, 3, 4, 1),
     (2, 32, 12, 11, 72, 5, 2, 2, 1),
     (5, 96, 10, 10, 40, 3, 1, 1, 1),
+    # thin inputs under a 7-row filter: whole output rows per block, several tiles per image, a partial last tile
+    (2, 3, 56, 56, 64, 7, 3, 2, 1),
+    (1, 4, 33, 29, 24, 7, 3, 2, 1),
     # dilated (a tenth entry: dilation)
     (2, 16, 13, 12, 24, 3, 2, 1, 1, 2),
     (2, 32, 15, 15, 16, 3, 3, 2, 1, 3),
@@ -113,6 +116,8 @@ def test_conv_nonsquare_filter(R, S, layout, dtype):
 
 @pytest.mark.parametrize("case", [(2, 64, 14, 64, 3, 1, 1, 3), (3, 32, 9, 160, 1, 0, 1, 1), (2, 128, 13, 24, 3, 1, 2, 0),
                                   (2, 3, 30, 64, 7, 3, 2, 3), (2, 16, 8, 20, 3, 1, 1, 3),
+                                  # the stem kernel: partial last tile; more tiles than blocks and a ragged channel tile
+                                  (2, 3, 56, 64, 7, 3, 2, 3), (130, 3, 64, 40, 7, 3, 2, 1),
                                   # 3x3 layers of the last stages: many channels, tiles with dead rows, 7x7 images
                                   (3, 128, 14, 256, 3, 1, 1, 3), (6, 64, 7, 136, 3, 1, 1, 1), (2, 64, 28, 64, 3, 1, 1, 2)])
 def test_conv_with_folded_bn_inference(case):
@@ -152,6 +157,8 @@ BNSTATS_CASES = [
     (3, 32, 9, 160, 1, 0, 1, True),
     (2, 128, 13, 24, 3, 1, 2, True),
     (2, 3, 30, 64, 7, 3, 2, False),
+    (2, 3, 56, 64, 7, 3, 2, False),
+    (130, 3, 64, 64, 7, 3, 2, True),
     # 3x3 layers of the last stages: row counts that are no multiple of the tile, 7x7 images, 56x56 at 64 channels
     (3, 128, 14, 256, 3, 1, 1, True),
     (6, 64, 7, 136, 3, 1, 1, False),
