@@ -37,7 +37,7 @@ CONV_KINDS = ("convfwd", "convbwddata", "convbwddata.bn", "convbwdfilter")
 FAMILIES = {
     "conv": ("convfwd", "convfwd.bn", "convbwddata", "convbwddata.bn", "convbwdfilter"),
     "batchnorm": ("bntrain", "bntrain.fused", "bnbwd", "bnbwd.fused", "bnbwd.linked"),
-    "pool": ("poolfwd", "poolbwd"),
+    "pool": ("poolfwd", "poolfwd.bn", "poolbwd"),
 }
 
 # HBM bytes per launch of a family, averaged over ALL launches of that family in one training step (the same

@@ -232,7 +232,10 @@ int saga_hip_bn_train_fwd(const SagaTensorView *x, const SagaTensorView *z, cons
  * over x that computes them.  workspace: 2*C floats.  Channels-last tensors only.
  * relu_mask (may be NULL; fp16 with C % 8 == 0 and SAGA_BN_RELU only): rows*C/8 bytes, bit j of byte
  * [row][c/8] set where y[row][c - c%8 + j] > 0 - the role of cuDNN's reserve space for the fused
- * add + relu operation (src/cuda/cuda_dnn.cpp:2095-2136); saga_hip_bn_bwd_ex reads it in place of y. */
+ * add + relu operation (src/cuda/cuda_dnn.cpp:2095-2136); saga_hip_bn_bwd_ex reads it in place of y.
+ * y NULL (then z and relu_mask NULL too): only the statistics are finalised - save_mean, save_invstd, the
+ * running statistics - and the workspace receives scale[c] = s*invstd and shift[c] = b - mean*scale (2*C
+ * floats), for a consumer that normalises on the fly (saga_hip_maxpool_fwd_codes_bn). */
 int saga_hip_bn_train_fwd_partials(const SagaTensorView *x, const SagaTensorView *z, const SagaTensorView *y,
                                    const float *s, const float *b, float *run_m, float *run_v, float *save_mean,
                                    float *save_invstd, float eps, float expavg, int flags, const float *partial,
@@ -287,6 +290,14 @@ int saga_hip_pool_bwd(int mode, const SagaTensorView *x, const SagaTensorView *y
  * size 2 or 3; SAGA_HIP_EUNSUPPORTED otherwise (use saga_hip_pool_fwd / saga_hip_pool_bwd). */
 int saga_hip_maxpool_fwd_codes(const SagaTensorView *x, const SagaTensorView *y, uint8_t *codes, int size, int pad,
                                int stride, saga_stream_t stream);
+/* The same on the OUTPUT of a batch norm (+ relu) that is never written: x is the norm's input and every window
+ * position holds act(x*scale[c] + shift[c]) rounded to the tensor's type, exactly what
+ * saga_hip_bn_train_fwd_partials would have stored (scale_shift: the 2*C floats that call leaves when its y is
+ * NULL).  The reference runs cudnnBatchNormalizationForwardTrainingEx and cudnnPoolingForward one after the
+ * other (src/cuda/cuda_dnn.cpp:2095-2136, :820-836); fused, the normalised tensor - the largest activation of a
+ * ResNet stem - is neither written nor read.  flags: SAGA_BN_RELU or 0. */
+int saga_hip_maxpool_fwd_codes_bn(const SagaTensorView *x, const SagaTensorView *y, uint8_t *codes, int size, int pad,
+                                  int stride, const float *scale_shift, int flags, saga_stream_t stream);
 int saga_hip_maxpool_bwd_codes(const uint8_t *codes, const SagaTensorView *dy, const SagaTensorView *dx, int size,
                                int pad, int stride, float beta, saga_stream_t stream);
 

@@ -903,8 +903,28 @@ int saga_hip_bn_train_fwd_partials(const SagaTensorView *x, const SagaTensorView
                                    int partial_rows, uint8_t *relu_mask, void *workspace, size_t ws_bytes,
                                    saga_stream_t stream)
 {
-    if(!valid_view(x) || !valid_view(y) || !s || !b || !partial || partial_rows < 1)
+    if(!valid_view(x) || (y && !valid_view(y)) || !s || !b || !partial || partial_rows < 1)
         return SAGA_HIP_EINVAL;
+    if(!y) {
+        // statistics only: mean, 1/std and the running statistics as usual, and scale[c], shift[c] (2*C floats)
+        // into the workspace, for a consumer that applies them itself (saga_hip_maxpool_fwd_codes_bn)
+        if(z || relu_mask || (x->dtype != SAGA_HALF && x->dtype != SAGA_FLOAT))
+            return SAGA_HIP_EINVAL;
+        const int C = x->dims[1];
+        if(!workspace || ws_bytes < 2 * (size_t)C * sizeof(float))
+            return SAGA_HIP_EWORKSPACE;
+        const double rows = (double)x->dims[0] * x->dims[2] * x->dims[3];
+        if(x->dtype == SAGA_HALF)
+            bn_stats_finalize<half_t><<<C, 256, 0, as_stream(stream)>>>(partial, partial_rows, (const half_t *)nullptr, 1, s, b,
+                                                                        run_m, run_v, save_mean, save_invstd,
+                                                                        (float *)workspace, rows, C, eps, expavg);
+        else
+            bn_stats_finalize<float><<<C, 256, 0, as_stream(stream)>>>(partial, partial_rows, (const float *)nullptr, 1, s, b,
+                                                                       run_m, run_v, save_mean, save_invstd,
+                                                                       (float *)workspace, rows, C, eps, expavg);
+        SAGA_CHECK_LAUNCH();
+        return 0;
+    }
     const bool add = flags & SAGA_BN_ADD;
     if(add && !valid_view(z))
         return SAGA_HIP_EINVAL;

@@ -376,8 +376,12 @@ template <> struct CodeVec<4> {
 // values cost more than its memory traffic): blockIdx.z = sample, blockIdx.y = output row,
 // threadIdx.x = channel vector, threadIdx.y (+ blockIdx.x) = output column.  K and the stride
 // are template parameters so that the window arithmetic folds to shifts and constants.
+// ss (may be null): 2*C floats scale[c], shift[c] of a batch norm whose output the pooling reads - the windows then
+// hold relu(x * scale + shift) (relu when `relu` is set), rounded to T as the norm would have stored it, computed
+// here from the norm's INPUT x, and the normalised tensor never exists.
 template <typename T, int VN, int K, int S>
-__global__ void __launch_bounds__(256) maxpool_fwd_codes_k(DView x, DView y, uint8_t *__restrict__ codes, int pad)
+__global__ void __launch_bounds__(256) maxpool_fwd_codes_k(DView x, DView y, uint8_t *__restrict__ codes, int pad,
+                                                           const float *__restrict__ ss = nullptr, int relu = 0)
 {
     const int C = y.d[1], P = y.d[2], Q = y.d[3], H = x.d[2], W = x.d[3];
     const int n = blockIdx.z, p = blockIdx.y;
@@ -397,6 +401,23 @@ __global__ void __launch_bounds__(256) maxpool_fwd_codes_k(DView x, DView y, uin
             const int hc = h < 0 ? 0 : (h >= H ? H - 1 : h), wc = w < 0 ? 0 : (w >= W ? W - 1 : w);
             PV<T, VN>::load((const T *)x.ptr + off4(x, n, c, hc, wc), v[r * K + s]);
         }
+    if(ss) {
+        float sc[VN], sh[VN];
+#pragma unroll
+        for(int j = 0; j < VN; j++) {
+            sc[j] = ss[c + j];
+            sh[j] = ss[C + c + j];
+        }
+#pragma unroll
+        for(int k = 0; k < K * K; k++)
+#pragma unroll
+            for(int j = 0; j < VN; j++) {
+                float t = __builtin_fmaf(v[k][j], sc[j], sh[j]); // bn_apply_cl's expression
+                if(relu)
+                    t = (t != t) ? t : fmaxf(t, 0.0f);
+                v[k][j] = (float)(T)t;
+            }
+    }
     float acc[VN];
     unsigned code[VN];
 #pragma unroll
@@ -576,7 +597,7 @@ static int pool_dim(int in, int k, int pad, int stride) { return 1 + (in + 2 * p
 
 static bool codes_ok(const SagaTensorView *a, const SagaTensorView *b, int size, int pad, int stride);
 static void launch_maxpool_codes(const SagaTensorView *x, const SagaTensorView *y, uint8_t *codes, int size, int pad,
-                                 int stride, hipStream_t st);
+                                 int stride, hipStream_t st, const float *ss = nullptr, int relu = 0);
 
 extern "C" {
 
@@ -721,16 +742,33 @@ int saga_hip_maxpool_fwd_codes(const SagaTensorView *x, const SagaTensorView *y,
     return 0;
 }
 
+int saga_hip_maxpool_fwd_codes_bn(const SagaTensorView *x, const SagaTensorView *y, uint8_t *codes, int size, int pad,
+                                  int stride, const float *scale_shift, int flags, saga_stream_t stream)
+{
+    if(!valid_view(x) || !valid_view(y) || !codes || !scale_shift)
+        return SAGA_HIP_EINVAL;
+    if(flags & ~SAGA_BN_RELU)
+        return SAGA_HIP_EUNSUPPORTED; // a residual would be a third tensor per window position
+    if(x->dims[0] != y->dims[0] || x->dims[1] != y->dims[1] || y->dims[2] != pool_dim(x->dims[2], size, pad, stride) ||
+       y->dims[3] != pool_dim(x->dims[3], size, pad, stride))
+        return SAGA_HIP_ESHAPE;
+    if(!codes_ok(x, y, size, pad, stride) || ((uintptr_t)codes & 7))
+        return SAGA_HIP_EUNSUPPORTED;
+    launch_maxpool_codes(x, y, codes, size, pad, stride, as_stream(stream), scale_shift, flags & SAGA_BN_RELU ? 1 : 0);
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
 } // extern "C"
 
 static void launch_maxpool_codes(const SagaTensorView *x, const SagaTensorView *y, uint8_t *codes, int size, int pad,
-                                 int stride, hipStream_t st)
+                                 int stride, hipStream_t st, const float *ss, int relu)
 {
     const int vn = x->dtype == SAGA_HALF ? 8 : 4;
     dim3 grid, block;
     codes_launch_shape(y->dims[1] / vn, y->dims[3], y->dims[2], y->dims[0], grid, block);
     const DView dvx = dview(x), dvy = dview(y);
-#define GO2(T, VN, K, S) maxpool_fwd_codes_k<T, VN, K, S><<<grid, block, 0, st>>>(dvx, dvy, codes, pad)
+#define GO2(T, VN, K, S) maxpool_fwd_codes_k<T, VN, K, S><<<grid, block, 0, st>>>(dvx, dvy, codes, pad, ss, relu)
 #define GO(T, VN)                                                                                              \
     do {                                                                                                       \
         switch(size * 4 + stride) {                                                                            \

@@ -197,6 +197,7 @@ struct HipProgram;
 void link_bn_backward(HipProgram &p, std::vector<std::shared_ptr<HipOperation>> &ops);
 // hip_ops.cpp: a strided 1x1 backward data that writes a fan-in gradient first is moved behind the last writer
 void reorder_sparse_first_writers(std::vector<std::shared_ptr<HipOperation>> &ops);
+void fuse_bn_pooling(HipProgram &p, std::vector<std::shared_ptr<HipOperation>> &ops);
 
 struct HipProgramUnit {
     Nodes m_transformed;

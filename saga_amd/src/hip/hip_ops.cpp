@@ -518,139 +518,6 @@ REGISTER_HIP_OP("tanh", tanh_setup);
 REGISTER_HIP_OP("swish", swish_setup);
 REGISTER_HIP_OP("leakyrelu", leakyrelu_setup);
 
-// ---------------------------------------------------------------- pooling
-// reference: src/cuda/cuda_dnn.cpp:810-926
-
-struct PoolFwd : public HipOperation {
-    const T x_, y_;
-    const int mode_, size_, pad_, stride_;
-    PoolFwd(T x, T y, int mode, int size, int pad, int stride)
-      : HipOperation("poolfwd"), x_(x), y_(y), mode_(mode), size_(size), pad_(pad), stride_(stride)
-    {
-    }
-    void exec(HipProgram &p) override
-    {
-        const SagaTensorView vx = x_->view(), vy = y_->view();
-        chkSaga(saga_hip_pool_fwd(mode_, &vx, &vy, nullptr, size_, pad_, stride_, S(p)));
-    }
-    HipOpArgs listInputs() const override { return {{"x", x_}}; }
-    HipOpArgs listOutputs() const override { return {{"y", y_}}; }
-    std::string info() const override { return mode_ == SAGA_POOL_MAX ? "max" : "avg"; }
-    double bytes() const override { return nbytes(x_) + nbytes(y_); }
-};
-
-struct PoolBwd : public HipOperation {
-    const T x_, y_, dx_, dy_;
-    const int mode_, size_, pad_, stride_;
-    float beta_ = 0;
-    PoolBwd(T x, T y, T dx, T dy, int mode, int size, int pad, int stride)
-      : HipOperation("poolbwd"), x_(x), y_(y), dx_(dx), dy_(dy), mode_(mode), size_(size), pad_(pad), stride_(stride)
-    {
-    }
-    void exec(HipProgram &p) override
-    {
-        const SagaTensorView vx = x_->view(), vy = y_->view(), vdy = dy_->view(), vdx = dx_->view();
-        chkSaga(saga_hip_pool_bwd(mode_, &vx, &vy, &vdy, &vdx, size_, pad_, stride_, beta_, S(p)));
-    }
-    HipOpArgs listInputs() const override { return {{"x", x_}, {"y", y_}, {"dy", dy_}}; }
-    HipOpArgs listOutputs() const override { return {{"dx", dx_}}; }
-    float *getBeta(const T &t) override { return t == dx_ ? &beta_ : nullptr; }
-    double bytes() const override
-    {
-        return nbytes(dx_) + nbytes(dy_) + (mode_ == SAGA_POOL_MAX ? nbytes(x_) + nbytes(y_) : 0);
-    }
-};
-
-// Max pooling in a training program, channels-last: the forward pass records the position of every
-// maximum in a byte tensor of y's shape and the backward pass reads that instead of x and y.
-struct MaxPoolFwdCodes : public HipOperation {
-    const T x_, y_, codes_;
-    const int size_, pad_, stride_;
-    MaxPoolFwdCodes(T x, T y, T codes, int size, int pad, int stride)
-      : HipOperation("poolfwd"), x_(x), y_(y), codes_(codes), size_(size), pad_(pad), stride_(stride)
-    {
-    }
-    void exec(HipProgram &p) override
-    {
-        const SagaTensorView vx = x_->view(), vy = y_->view();
-        chkSaga(saga_hip_maxpool_fwd_codes(&vx, &vy, (uint8_t *)codes_->deviceMem(), size_, pad_, stride_, S(p)));
-    }
-    HipOpArgs listInputs() const override { return {{"x", x_}}; }
-    HipOpArgs listOutputs() const override { return {{"y", y_}, {"codes", codes_}}; }
-    std::string info() const override { return "max+codes"; }
-    double bytes() const override { return nbytes(x_) + nbytes(y_) + nbytes(codes_); }
-};
-
-struct MaxPoolBwdCodes : public HipOperation {
-    const T codes_, dy_, dx_;
-    const int size_, pad_, stride_;
-    float beta_ = 0;
-    MaxPoolBwdCodes(T codes, T dy, T dx, int size, int pad, int stride)
-      : HipOperation("poolbwd"), codes_(codes), dy_(dy), dx_(dx), size_(size), pad_(pad), stride_(stride)
-    {
-    }
-    void exec(HipProgram &p) override
-    {
-        const SagaTensorView vdy = dy_->view(), vdx = dx_->view();
-        chkSaga(saga_hip_maxpool_bwd_codes((const uint8_t *)codes_->deviceMem(), &vdy, &vdx, size_, pad_, stride_, beta_,
-                                           S(p)));
-    }
-    HipOpArgs listInputs() const override { return {{"codes", codes_}, {"dy", dy_}}; }
-    HipOpArgs listOutputs() const override { return {{"dx", dx_}}; }
-    float *getBeta(const T &t) override { return t == dx_ ? &beta_ : nullptr; }
-    double bytes() const override { return nbytes(dx_) * (beta_ != 0 ? 2 : 1) + nbytes(dy_) + nbytes(codes_); }
-};
-
-// what saga_hip_maxpool_*_codes accept (anything else takes the x / y based kernels)
-static bool maxpool_codes_fit(const HipTensor &x, const HipTensor &y, const HipTensor *dx, const HipTensor *dy, int size,
-                              int pad, int stride)
-{
-    if(getenv("SAGA_HIP_NO_POOL_CODES"))
-        return false;
-    if(size < 2 || size > 3 || stride < 1 || stride > size || pad >= size)
-        return false;
-    const int vn = x.m_data_type == Tensor::DataType::HALF ? 8 : x.m_data_type == Tensor::DataType::FLOAT ? 4 : 0;
-    if(!vn || x.m_dims.size() != 4 || (int)x.m_dims[1] % vn)
-        return false;
-    for(const HipTensor *t : {&x, &y, dx, dy}) {
-        if(!t || !t->cpacked() || t->m_data_type != x.m_data_type || t->m_dims.elements() >= ((size_t)1 << 31))
-            return false;
-        for(int i : {0, 2, 3})
-            if((int)t->m_dims[i] > 1 && t->m_strides[i] % vn)
-                return false;
-    }
-    return true;
-}
-
-void pooling_setup(HipProgram &p, HipProgramUnit &pu, const Node &n, int mode)
-{
-    auto x = p.lower(pu, n.m_inputs["x"]);
-    auto y = p.lowerLike(pu, n.m_outputs["y"], *x);
-    const int size = n.m_attributes.get("global", false) ? (int)x->m_dims[2] : n.m_attributes.get("size", 1);
-    const int pad = n.m_attributes.get("pad", 0);
-    const int stride = n.m_attributes.get("stride", 1);
-    if(p.m_pt == ProgramType::INFERENCE) {
-        pu.fwd(std::make_shared<PoolFwd>(x, y, mode, size, pad, stride));
-        return;
-    }
-    auto dx = p.lowerGrad(pu, n.m_inputs["x"]);
-    auto dy = p.lowerGrad(pu, n.m_outputs["y"]);
-    if(mode == SAGA_POOL_MAX && dx && dy && maxpool_codes_fit(*x, *y, dx.get(), dy.get(), size, pad, stride)) {
-        // dense N,H,W,C bytes whatever pitch y has
-        auto codes = std::make_shared<HipTensor>(Tensor::DataType::U8, y->m_dims, HipLayout::NHWC, p.m_ctx.get(),
-                                                 n.m_outputs["y"]->namePostfix("maxpos"));
-        pu.fwd(std::make_shared<MaxPoolFwdCodes>(x, y, codes, size, pad, stride));
-        pu.bwd(std::make_shared<MaxPoolBwdCodes>(codes, dy, dx, size, pad, stride));
-        return;
-    }
-    pu.fwd(std::make_shared<PoolFwd>(x, y, mode, size, pad, stride));
-    pu.bwd(std::make_shared<PoolBwd>(x, y, dx, dy, mode, size, pad, stride));
-}
-void maxpool_setup(HipProgram &p, HipProgramUnit &pu, const Node &n) { pooling_setup(p, pu, n, SAGA_POOL_MAX); }
-void avgpool_setup(HipProgram &p, HipProgramUnit &pu, const Node &n) { pooling_setup(p, pu, n, SAGA_POOL_AVG); }
-REGISTER_HIP_OP("maxpool", maxpool_setup);
-REGISTER_HIP_OP("avgpool", avgpool_setup);
-
 // ---------------------------------------------------------------- fully connected
 // reference: src/cuda/cuda_dnn.cpp:968-1130 (column-major cuBLAS calls restated row-major)
 
@@ -901,6 +768,11 @@ struct BnTrain : public HipOperation {
     // mask_valid_ says whether the forward pass of this step wrote it
     T mask_;
     bool mask_valid_ = false;
+    // a max pooling is the only reader of y and normalises on the fly (BnMaxPoolFwdCodes): this operation then only
+    // finalises the statistics and leaves scale and shift in ss_; y stays allocated and unwritten.  applied_ says
+    // whether this step's forward pass wrote y after all (the convolution did not deliver its sums).
+    T ss_;
+    bool applied_ = true;
     BnTrain(HipProgram &p, T x, T z, T s, T b, T m, T v, T y, T sm, T sv, float eps, int flags)
       : HipOperation(flags ? "bntrain.fused" : "bntrain")
       , x_(x), z_(z), s_(s), b_(b), m_(m), v_(v), y_(y), sm_(sm), sv_(sv), eps_(eps), flags_(flags)
@@ -918,6 +790,22 @@ struct BnTrain : public HipOperation {
         if(z_)
             vz = z_->view();
         mask_valid_ = false;
+        applied_ = true;
+        if(ss_ && stats_ && stats_->valid) {
+            const int r = saga_hip_bn_train_fwd_partials(
+                &vx, nullptr, nullptr, (const float *)s_->deviceMem(), (const float *)b_->deviceMem(),
+                (float *)m_->deviceMem(), (float *)v_->deviceMem(), (float *)sm_->deviceMem(), (float *)sv_->deviceMem(),
+                eps_, expavg_, flags_, (const float *)stats_->partial->m_ptr, stats_->rows, nullptr, ss_->deviceMem(),
+                ss_->m_dims.elements() * sizeof(float), S(p));
+            if(r == 0) {
+                stats_->valid = false;
+                expavg_ = p.m_pc.bn_expavg;
+                applied_ = false;
+                return;
+            }
+            if(r != SAGA_HIP_EUNSUPPORTED)
+                chkSaga(r);
+        }
         if(stats_ && stats_->valid) {
             stats_->valid = false;
             const int r = saga_hip_bn_train_fwd_partials(
@@ -953,10 +841,17 @@ struct BnTrain : public HipOperation {
         HipOpArgs r{{"y", y_}, {"m", m_}, {"v", v_}, {"sm", sm_}, {"sv", sv_}};
         if(mask_)
             r.push_back({"mask", mask_});
+        if(ss_)
+            r.push_back({"ss", ss_});
         return r;
     }
     // statistics pass reads x (unless the producer supplied the sums), normalise pass reads x (+z), writes y
-    double bytes() const override { return ((z_ ? 4 : 3) - (stats_ ? 1 : 0) + (mask_ ? 0.0625 : 0)) * nbytes(x_); }
+    double bytes() const override
+    {
+        if(ss_ && stats_) // the partial sums in, a few vectors of C floats out
+            return 16.0 * (double)x_->m_dims[1];
+        return ((z_ ? 4 : 3) - (stats_ ? 1 : 0) + (mask_ ? 0.0625 : 0)) * nbytes(x_);
+    }
     float *getBeta(const T &t) override
     {
         if(t == m_)
@@ -996,7 +891,8 @@ struct BnBwd : public HipOperation {
             return;
         }
         // the bias lets the kernels rebuild the relu mask from x when there is no residual
-        chkSaga(saga_hip_bn_bwd_ex(&vx, relu ? &vy : nullptr, &vdy, &vdx, dz_ ? &vdz : nullptr,
+        // (a forward pass that left the normalising to a pooling wrote no y: the mask is then rebuilt from x)
+        chkSaga(saga_hip_bn_bwd_ex(&vx, relu && fwd_->applied_ ? &vy : nullptr, &vdy, &vdx, dz_ ? &vdz : nullptr,
                                 (const float *)fwd_->s_->deviceMem(), (const float *)fwd_->b_->deviceMem(),
                                 (const float *)fwd_->sm_->deviceMem(),
                                 (const float *)fwd_->sv_->deviceMem(), (float *)ds_->deviceMem(),
@@ -1305,6 +1201,169 @@ Nodes batchnorm_relu_transform(HipProgram &p, HipProgramUnit &, const Nodes &nod
     return r;
 }
 REGISTER_HIP_TRANSFORM(500, ProgramType::INFERENCE | ProgramType::TRAINING, batchnorm_relu_transform);
+
+// ---------------------------------------------------------------- pooling
+// reference: src/cuda/cuda_dnn.cpp:810-926
+
+struct PoolFwd : public HipOperation {
+    const T x_, y_;
+    const int mode_, size_, pad_, stride_;
+    PoolFwd(T x, T y, int mode, int size, int pad, int stride)
+      : HipOperation("poolfwd"), x_(x), y_(y), mode_(mode), size_(size), pad_(pad), stride_(stride)
+    {
+    }
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vx = x_->view(), vy = y_->view();
+        chkSaga(saga_hip_pool_fwd(mode_, &vx, &vy, nullptr, size_, pad_, stride_, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"x", x_}}; }
+    HipOpArgs listOutputs() const override { return {{"y", y_}}; }
+    std::string info() const override { return mode_ == SAGA_POOL_MAX ? "max" : "avg"; }
+    double bytes() const override { return nbytes(x_) + nbytes(y_); }
+};
+
+struct PoolBwd : public HipOperation {
+    const T x_, y_, dx_, dy_;
+    const int mode_, size_, pad_, stride_;
+    float beta_ = 0;
+    PoolBwd(T x, T y, T dx, T dy, int mode, int size, int pad, int stride)
+      : HipOperation("poolbwd"), x_(x), y_(y), dx_(dx), dy_(dy), mode_(mode), size_(size), pad_(pad), stride_(stride)
+    {
+    }
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vx = x_->view(), vy = y_->view(), vdy = dy_->view(), vdx = dx_->view();
+        chkSaga(saga_hip_pool_bwd(mode_, &vx, &vy, &vdy, &vdx, size_, pad_, stride_, beta_, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"x", x_}, {"y", y_}, {"dy", dy_}}; }
+    HipOpArgs listOutputs() const override { return {{"dx", dx_}}; }
+    float *getBeta(const T &t) override { return t == dx_ ? &beta_ : nullptr; }
+    double bytes() const override
+    {
+        return nbytes(dx_) + nbytes(dy_) + (mode_ == SAGA_POOL_MAX ? nbytes(x_) + nbytes(y_) : 0);
+    }
+};
+
+// Max pooling in a training program, channels-last: the forward pass records the position of every
+// maximum in a byte tensor of y's shape and the backward pass reads that instead of x and y.
+struct MaxPoolFwdCodes : public HipOperation {
+    const T x_, y_, codes_;
+    const int size_, pad_, stride_;
+    MaxPoolFwdCodes(T x, T y, T codes, int size, int pad, int stride)
+      : HipOperation("poolfwd"), x_(x), y_(y), codes_(codes), size_(size), pad_(pad), stride_(stride)
+    {
+    }
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vx = x_->view(), vy = y_->view();
+        chkSaga(saga_hip_maxpool_fwd_codes(&vx, &vy, (uint8_t *)codes_->deviceMem(), size_, pad_, stride_, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"x", x_}}; }
+    HipOpArgs listOutputs() const override { return {{"y", y_}, {"codes", codes_}}; }
+    std::string info() const override { return "max+codes"; }
+    double bytes() const override { return nbytes(x_) + nbytes(y_) + nbytes(codes_); }
+};
+
+struct MaxPoolBwdCodes : public HipOperation {
+    const T codes_, dy_, dx_;
+    const int size_, pad_, stride_;
+    float beta_ = 0;
+    MaxPoolBwdCodes(T codes, T dy, T dx, int size, int pad, int stride)
+      : HipOperation("poolbwd"), codes_(codes), dy_(dy), dx_(dx), size_(size), pad_(pad), stride_(stride)
+    {
+    }
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vdy = dy_->view(), vdx = dx_->view();
+        chkSaga(saga_hip_maxpool_bwd_codes((const uint8_t *)codes_->deviceMem(), &vdy, &vdx, size_, pad_, stride_, beta_,
+                                           S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"codes", codes_}, {"dy", dy_}}; }
+    HipOpArgs listOutputs() const override { return {{"dx", dx_}}; }
+    float *getBeta(const T &t) override { return t == dx_ ? &beta_ : nullptr; }
+    double bytes() const override { return nbytes(dx_) * (beta_ != 0 ? 2 : 1) + nbytes(dy_) + nbytes(codes_); }
+};
+
+// Max pooling right behind a batch norm (+ relu) that nobody else reads: the windows are normalised on the fly
+// from the norm's input and the normalised tensor - for a ResNet stem the largest activation of the network - is
+// neither written nor read.  bn_: the norm's forward operation, which then only finalises its statistics; if in
+// some step it had to normalise itself after all (applied_), this is the plain pooling of its output.
+struct BnMaxPoolFwdCodes : public HipOperation {
+    const std::shared_ptr<BnTrain> bn_;
+    const T y_, codes_;
+    const int size_, pad_, stride_;
+    BnMaxPoolFwdCodes(std::shared_ptr<BnTrain> bn, T y, T codes, int size, int pad, int stride)
+      : HipOperation("poolfwd.bn"), bn_(bn), y_(y), codes_(codes), size_(size), pad_(pad), stride_(stride)
+    {
+    }
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vy = y_->view();
+        if(bn_->applied_) {
+            const SagaTensorView vx = bn_->y_->view();
+            chkSaga(saga_hip_maxpool_fwd_codes(&vx, &vy, (uint8_t *)codes_->deviceMem(), size_, pad_, stride_, S(p)));
+            return;
+        }
+        const SagaTensorView vx = bn_->x_->view();
+        chkSaga(saga_hip_maxpool_fwd_codes_bn(&vx, &vy, (uint8_t *)codes_->deviceMem(), size_, pad_, stride_,
+                                              (const float *)bn_->ss_->deviceMem(), bn_->flags_, S(p)));
+    }
+    HipOpArgs listInputs() const override { return {{"x", bn_->y_}, {"bn-x", bn_->x_}, {"ss", bn_->ss_}}; }
+    HipOpArgs listOutputs() const override { return {{"y", y_}, {"codes", codes_}}; }
+    std::string info() const override { return "max+codes on bn input"; }
+    double bytes() const override { return nbytes(bn_->x_) + nbytes(y_) + nbytes(codes_); }
+};
+
+// what saga_hip_maxpool_*_codes accept (anything else takes the x / y based kernels)
+static bool maxpool_codes_fit(const HipTensor &x, const HipTensor &y, const HipTensor *dx, const HipTensor *dy, int size,
+                              int pad, int stride)
+{
+    if(getenv("SAGA_HIP_NO_POOL_CODES"))
+        return false;
+    if(size < 2 || size > 3 || stride < 1 || stride > size || pad >= size)
+        return false;
+    const int vn = x.m_data_type == Tensor::DataType::HALF ? 8 : x.m_data_type == Tensor::DataType::FLOAT ? 4 : 0;
+    if(!vn || x.m_dims.size() != 4 || (int)x.m_dims[1] % vn)
+        return false;
+    for(const HipTensor *t : {&x, &y, dx, dy}) {
+        if(!t || !t->cpacked() || t->m_data_type != x.m_data_type || t->m_dims.elements() >= ((size_t)1 << 31))
+            return false;
+        for(int i : {0, 2, 3})
+            if((int)t->m_dims[i] > 1 && t->m_strides[i] % vn)
+                return false;
+    }
+    return true;
+}
+
+void pooling_setup(HipProgram &p, HipProgramUnit &pu, const Node &n, int mode)
+{
+    auto x = p.lower(pu, n.m_inputs["x"]);
+    auto y = p.lowerLike(pu, n.m_outputs["y"], *x);
+    const int size = n.m_attributes.get("global", false) ? (int)x->m_dims[2] : n.m_attributes.get("size", 1);
+    const int pad = n.m_attributes.get("pad", 0);
+    const int stride = n.m_attributes.get("stride", 1);
+    if(p.m_pt == ProgramType::INFERENCE) {
+        pu.fwd(std::make_shared<PoolFwd>(x, y, mode, size, pad, stride));
+        return;
+    }
+    auto dx = p.lowerGrad(pu, n.m_inputs["x"]);
+    auto dy = p.lowerGrad(pu, n.m_outputs["y"]);
+    if(mode == SAGA_POOL_MAX && dx && dy && maxpool_codes_fit(*x, *y, dx.get(), dy.get(), size, pad, stride)) {
+        // dense N,H,W,C bytes whatever pitch y has
+        auto codes = std::make_shared<HipTensor>(Tensor::DataType::U8, y->m_dims, HipLayout::NHWC, p.m_ctx.get(),
+                                                 n.m_outputs["y"]->namePostfix("maxpos"));
+        pu.fwd(std::make_shared<MaxPoolFwdCodes>(x, y, codes, size, pad, stride));
+        pu.bwd(std::make_shared<MaxPoolBwdCodes>(codes, dy, dx, size, pad, stride));
+        return;
+    }
+    pu.fwd(std::make_shared<PoolFwd>(x, y, mode, size, pad, stride));
+    pu.bwd(std::make_shared<PoolBwd>(x, y, dx, dy, mode, size, pad, stride));
+}
+void maxpool_setup(HipProgram &p, HipProgramUnit &pu, const Node &n) { pooling_setup(p, pu, n, SAGA_POOL_MAX); }
+void avgpool_setup(HipProgram &p, HipProgramUnit &pu, const Node &n) { pooling_setup(p, pu, n, SAGA_POOL_AVG); }
+REGISTER_HIP_OP("maxpool", maxpool_setup);
+REGISTER_HIP_OP("avgpool", avgpool_setup);
 
 // ---------------------------------------------------------------- sum / add / softmax
 // reference: src/cuda/cuda_dnn.cpp:1830-1964
@@ -1696,5 +1755,64 @@ Nodes concat_transform(HipProgram &p, HipProgramUnit &pu, const Nodes &nodes)
 REGISTER_HIP_TRANSFORM(100, ProgramType::INFERENCE | ProgramType::TRAINING, concat_transform);
 
 }  // namespace
+
+// Training programs: a max pooling (with position codes) whose input is the output of a batch norm (+ relu) that
+// nothing else touches - no other operation of the program reads or writes that storage (a skip connection, a
+// concat buffer the norm writes a slice of), not the host, not the anomaly checks - normalises its windows on the
+// fly from the norm's input, and the norm's forward only finalises its statistics.  The norm must get its sums
+// from the producing convolution, have no residual, and a backward pass that rebuilds the relu mask from x.
+void fuse_bn_pooling(HipProgram &p, HipOps &ops)
+{
+    if(p.m_pc.disable_op_fusing || p.m_pc.anomaly_detect || getenv("SAGA_HIP_NO_BN_POOL_FUSE") ||
+       getenv("SAGA_HIP_BN_MASK_FROM_Y"))
+        return;
+    for(size_t ip = 0; ip < ops.size(); ip++) {
+        auto pool = std::dynamic_pointer_cast<MaxPoolFwdCodes>(ops[ip]);
+        if(!pool)
+            continue;
+        const T &x = pool->x_;
+        std::shared_ptr<BnTrain> bn;
+        bool clean = true;
+        for(size_t i = 0; i < ops.size() && clean; i++) {
+            if(i == ip)
+                continue;
+            for(const auto &o : ops[i]->listOutputs())
+                if(o.second->m_storage == x->m_storage) {
+                    auto f = std::dynamic_pointer_cast<BnTrain>(ops[i]);
+                    if(bn || !f || f->y_ != x || i > ip)
+                        clean = false;
+                    bn = f;
+                }
+        }
+        if(!clean || !bn || !bn->stats_ || bn->z_ || bn->mask_ || bn->ss_ || (bn->flags_ & ~SAGA_BN_RELU))
+            continue;
+        for(size_t i = 0; i < ops.size() && clean; i++) {
+            if(i == ip)
+                continue;
+            auto *bwd = dynamic_cast<BnBwd *>(ops[i].get());
+            if(bwd && bwd->fwd_ == bn) {
+                // the norm's own backward lists y but, with the bias at hand and channels-last tensors, does not read it
+                if((bn->flags_ & SAGA_BN_RELU) && (!bwd->dx_->cpacked() || !bwd->dy_->cpacked() || !bn->x_->cpacked()))
+                    clean = false;
+                continue;
+            }
+            for(const auto &in : ops[i]->listInputs())
+                if(in.second->m_storage == x->m_storage)
+                    clean = false;
+        }
+        const auto &ex = p.m_ctx->m_exported;
+        if(!clean || std::any_of(ex.begin(), ex.end(), [&](const auto &e) { return e == x->m_storage; }))
+            continue;
+        // the pooling reads the norm's input in place of its output: same shape, type and channels-last packing
+        const HipTensor &bx = *bn->x_;
+        if(bx.m_data_type != x->m_data_type || bx.m_dims.i64() != x->m_dims.i64() || !bx.cpacked() ||
+           !maxpool_codes_fit(bx, bx, &bx, &bx, pool->size_, pool->pad_, pool->stride_))
+            continue;
+        const Dims sd{(int64_t)2 * (int64_t)x->m_dims[1]};
+        bn->ss_ = std::make_shared<HipTensor>(Tensor::DataType::FLOAT, sd, HipLayout::NCHW, p.m_ctx.get(),
+                                              std::string("scaleshift"));
+        ops[ip] = std::make_shared<BnMaxPoolFwdCodes>(bn, pool->y_, pool->codes_, pool->size_, pool->pad_, pool->stride_);
+    }
+}
 
 }  // namespace saga

@@ -594,8 +594,10 @@ void HipProgram::finalize()
     m_opt.clear();
 
     eliminateDeadOps();
-    if(m_pt == ProgramType::TRAINING)
+    if(m_pt == ProgramType::TRAINING) {
         link_bn_backward(*this, m_ops);
+        fuse_bn_pooling(*this, m_ops);
+    }
 
     m_ctx->m_workspace.alloc();
     m_ctx->m_programs.push_back(this);

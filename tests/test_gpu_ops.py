@@ -732,6 +732,67 @@ def test_maxpool_with_position_codes(k, pad, stride, H, padc, dtype):
     assert rc == -3  # SAGA_HIP_EUNSUPPORTED
 
 
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("k,pad,stride,H,relu", [(3, 1, 2, 12, True), (3, 1, 2, 9, False), (2, 0, 2, 8, True), (3, 0, 2, 11, True)])
+def test_maxpool_on_a_batch_norm_that_is_never_written(k, pad, stride, H, relu, dtype):
+    """saga_hip_bn_train_fwd_partials with y NULL (statistics only, scale and shift left for the consumer) followed
+    by saga_hip_maxpool_fwd_codes_bn, against the same two operators run one after the other with the normalised
+    tensor in between: pooled values and position codes bit for bit, saved and running statistics equal."""
+    rng = np.random.default_rng(k * 10 + H)
+    Cc = 16 if dtype == torch.float16 else 8
+    shape = (3, Cc, H, H + 1)
+    x = rnd(rng, *shape, dtype=dtype)
+    P, Q = ref.pool_out(H, k, pad, stride), ref.pool_out(H + 1, k, pad, stride)
+    s, b = (1 + 0.3 * rng.standard_normal(Cc)).astype(np.float32), (0.2 * rng.standard_normal(Cc)).astype(np.float32)
+    s[1] = -s[1]  # a negative scale: the maximum of the normalised values sits at the minimum of x
+    L = K.lib()
+    xd = dev(x, dtype, "nhwc")
+    rows = 3 * H * (H + 1)
+    # partial sums as a producing convolution would leave them: two rows that add up to the sums over x
+    xr = host(xd).astype(np.float64).transpose(0, 2, 3, 1).reshape(rows, Cc)
+    half_rows = rows // 2
+    part = np.stack([np.stack([xr[:half_rows].sum(0), (xr[:half_rows] ** 2).sum(0)], 1),
+                     np.stack([xr[half_rows:].sum(0), (xr[half_rows:] ** 2).sum(0)], 1)]).astype(np.float32)
+    partial = dev(part.reshape(-1))
+    flags = K.BN_RELU if relu else 0
+
+    def run(fused):
+        sd, bd = dev(s), dev(b)
+        md, vd = dev(np.zeros(Cc, np.float32)), dev(np.ones(Cc, np.float32))
+        sm, sv = dev(np.zeros(Cc, np.float32)), dev(np.zeros(Cc, np.float32))
+        ws = torch.zeros(2 * Cc, dtype=torch.float32, device="cuda")
+        yp = dev(np.zeros((3, Cc, P, Q), np.float32), dtype, "nhwc")
+        codes = torch.full((3, P, Q, Cc), 255, dtype=torch.uint8, device="cuda")
+        if fused:
+            K.check(L.saga_hip_bn_train_fwd_partials(C.byref(K.view(xd)), None, None, K.ptr(sd), K.ptr(bd), K.ptr(md),
+                                                     K.ptr(vd), K.ptr(sm), K.ptr(sv), 1e-5, 0.1, flags, K.ptr(partial), 2,
+                                                     None, K.ptr(ws), ws.numel() * 4, S()))
+            K.check(L.saga_hip_maxpool_fwd_codes_bn(C.byref(K.view(xd)), C.byref(K.view(yp)), K.ptr(codes), k, pad, stride,
+                                                    K.ptr(ws), flags, S()))
+        else:
+            yd = dev(np.zeros(shape, np.float32), dtype, "nhwc")
+            K.check(L.saga_hip_bn_train_fwd_partials(C.byref(K.view(xd)), None, C.byref(K.view(yd)), K.ptr(sd), K.ptr(bd),
+                                                     K.ptr(md), K.ptr(vd), K.ptr(sm), K.ptr(sv), 1e-5, 0.1, flags,
+                                                     K.ptr(partial), 2, None, K.ptr(ws), ws.numel() * 4, S()))
+            K.check(L.saga_hip_maxpool_fwd_codes(C.byref(K.view(yd)), C.byref(K.view(yp)), K.ptr(codes), k, pad, stride, S()))
+        return host(yp), codes.cpu().numpy(), [host(t) for t in (md, vd, sm, sv)]
+
+    y1, c1, st1 = run(True)
+    y0, c0, st0 = run(False)
+    np.testing.assert_array_equal(y1, y0)
+    np.testing.assert_array_equal(c1, c0)
+    for a_, b_ in zip(st1, st0):
+        np.testing.assert_array_equal(a_, b_)
+    # and against the oracle: batch norm, relu, max pooling
+    mean, var = xr.mean(0), xr.var(0)
+    yn = (host(xd).astype(np.float64) - mean[None, :, None, None]) / np.sqrt(var + 1e-5)[None, :, None, None]
+    yn = yn * s[None, :, None, None] + b[None, :, None, None]
+    if relu:
+        yn = np.maximum(yn, 0)
+    want = ref.maxpool_fwd(ref.round_half(yn.astype(np.float32)) if dtype == torch.float16 else yn.astype(np.float32), k, pad, stride)
+    assert_close(y1, want, dtype, "pooled batch norm")
+
+
 def test_pooling_golden(golden):
     g = golden["ops"]
     x = T(g, "pooling_input")
