@@ -2181,6 +2181,239 @@ template <int R, int MODE> __global__ void __launch_bounds__(256, 2) conv_thin_r
     }
 }
 
+// ---------------------------------------------------------------- 3x3, 64 -> 64 channels, whole image rows in LDS
+//
+// The 3x3 layers with 64 input and 64 output channels over large images (ResNet-50's first stage, 56x56) have too
+// little arithmetic per byte for the gather kernel's scheme - every output pixel's input is fetched into LDS nine
+// times, once per tap, and a 256 x 64 tile leaves the matrix unit waiting for those fills (114 us for 59 GFLOP).
+// Same idea as conv_thin_rows: a persistent block owns TR whole output rows of an image (TR * W <= 256 pixels),
+// copies the TR + 2 input rows they read ONCE into LDS - pixel slots of 144 bytes (128 of data + 16 of padding, so
+// that the 16-byte operand reads of 16 neighbouring pixels fall into 64 different banks), with a zero slot left
+// and right and zero rows above / below the image, all by out-of-range load offsets - and an MFMA operand of tap
+// (dr, ds) is the 16 bytes at ((orow + dr) * (W + 2) + ox + ds) * 144 + 16 * (k / 8): nine taps are nine
+// immediate offsets on one address.  Eight wavefronts: four groups of 64 pixels x two halves of the output
+// channels; a wavefront keeps its half of the filter (32 x 9 x 64 halves) in 144 registers for the whole launch.
+// FLIP reads the taps in reverse order: backward data of such a layer is this convolution of dy with the
+// transposed filter (C,R,S,K, which backward data keeps in its workspace anyway) mirrored.
+struct Rows64Args {
+    int H, W;
+    int TR;          // output rows per tile
+    int tpi;         // tiles per image
+    int ntiles;
+    int npix;        // TR * W
+    int slots_row;   // W + 2 pixel slots per LDS row
+    int chunks_tile; // (TR + 2) * slots_row * 9: 16-byte chunks of a tile's copy
+    int buf_bytes;   // one LDS buffer (chunks_tile * 16 rounded up to the 1 KB a load instruction fills)
+    int epi_off;     // where the epilogue's LDS scratch starts, minus what gather_epilogue adds itself
+};
+
+template <int MODE, bool FLIP, int WGM> __global__ void __launch_bounds__(128 * WGM, 4 / WGM) conv_rows64(GatherArgs g, Rows64Args t)
+{
+    float *const stats = MODE == 2 ? g.stats : nullptr;
+    g.stats = nullptr;
+    if constexpr(MODE != 1)
+        g.bn_s = nullptr;
+    else
+        g.bn_flags &= SAGA_BN_RELU; // (no residual here: its registers would not fit beside the filter's)
+    if constexpr(MODE != 0)
+        g.beta = 0.0f;
+    float run_s = 0.0f, run_q = 0.0f;
+    constexpr int TM = 2, TN = 1, NLD_MAX = 10, SLOT = 144, NW = 2 * WGM;
+    constexpr unsigned OOB = 0x7fffff00u;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int hi = lane >> 5;
+    const int wmi = wave >> 1, cj = wave & 1; // pixel group, channel half
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void *)g.a, 0, g.a_bytes, 0x00020000);
+
+    // this wavefront's half of the filter: fragment (tap, kk) = halves 16*kk + 8*hi .. +8 of that tap of output
+    // channel 32*cj + lane%32
+    half8_t fb[9][4];
+    {
+        const int o = cj * 32 + (lane & 31);
+        const bool ok = o < g.Ngemm;
+        const half_t *src = g.b + (int64_t)(ok ? o : 0) * 9 * 64 + hi * 8;
+#pragma unroll
+        for(int tp = 0; tp < 9; tp++)
+#pragma unroll
+            for(int kk = 0; kk < 4; kk++) {
+                const half8_t v = *(const half8_t *)(src + (FLIP ? 8 - tp : tp) * 64 + kk * 16);
+                const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+                fb[tp][kk] = ok ? v : zero;
+            }
+    }
+    const int my_nld = t.chunks_tile > wave * 64 ? (t.chunks_tile - wave * 64 + NW * 64 - 1) / (NW * 64) : 0;
+    // LDS chunk L = (q * 8 + wave) * 64 + lane of a tile's copy: pixel slot L / 9 (row r, column p of the padded
+    // rows), chunk L % 9 of the slot (the ninth is padding).  It has a source - channels 8*(L%9).. of input pixel
+    // (oy0 - 1 + r, p - 1) - unless that lies outside the image, and reads as zeros otherwise.
+    auto request = [&](int tile, int b) {
+        const int n = tile / t.tpi;
+        const int oy0 = (tile - n * t.tpi) * t.TR;
+        char *dst = smem + b * t.buf_bytes + wave * 1024;
+#pragma unroll
+        for(int q = 0; q < NLD_MAX; q++)
+            if(q < my_nld) {
+                const int L = (q * NW + wave) * 64 + lane;
+                const int slot = L / 9, kpos = L - slot * 9;
+                const int r = slot / t.slots_row, pcol = slot - r * t.slots_row;
+                const int iy = oy0 - 1 + r, ix = pcol - 1;
+                const bool ok = L < t.chunks_tile && kpos < 8 && ix >= 0 && ix < t.W && iy >= 0 && iy < t.H;
+                const unsigned off = ok ? (unsigned)((((n * t.H + iy) * t.W + ix) * g.lda + kpos * 8) * 2) : OOB;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(dst + q * (NW * 1024)), 16, off, 0, 0, 0);
+            }
+    };
+    // this lane's two pixels (row blocks i of the wavefront's 64) inside a tile: byte offset of the top left tap
+    int abase[TM], prow[TM]; // prow: the pixel's output row inside the tile, or a row beyond every image
+#pragma unroll
+    for(int i = 0; i < TM; i++) {
+        const int pp0 = wmi * 64 + i * 32 + (lane & 31);
+        const int pp = pp0 < t.npix ? pp0 : 0;
+        const int orow = pp / t.W;
+        abase[i] = (orow * t.slots_row + (pp - orow * t.W)) * SLOT + hi * 16;
+        prow[i] = pp0 < t.npix ? orow : 0x40000000;
+    }
+    char *epi = smem + t.epi_off;
+    const int G = gridDim.x;
+    int tile = xcd_remap(blockIdx.x, G);
+    const int first_tile = tile;
+    if(tile < t.ntiles)
+        request(tile, 0);
+    if(tile + G < t.ntiles)
+        request(tile + G, 1);
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    int b = 0;
+    for(; tile < t.ntiles; tile += G) {
+        const char *buf = smem + b * t.buf_bytes;
+        float16_t acc[TM][TN];
+#pragma unroll
+        for(int i = 0; i < TM; i++)
+#pragma unroll
+            for(int v = 0; v < 16; v++)
+                acc[i][0][v] = 0.0f;
+#pragma unroll
+        for(int dr = 0; dr < 3; dr++)
+#pragma unroll
+            for(int ds = 0; ds < 3; ds++) {
+                const int tapoff = (dr * t.slots_row + ds) * SLOT;
+                half8_t fa[4][TM];
+#pragma unroll
+                for(int kk = 0; kk < 4; kk++)
+#pragma unroll
+                    for(int i = 0; i < TM; i++)
+                        fa[kk][i] = *(const half8_t *)(buf + abase[i] + tapoff + kk * 32);
+#pragma unroll
+                for(int kk = 0; kk < 4; kk++)
+#pragma unroll
+                    for(int i = 0; i < TM; i++)
+                        acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[dr * 3 + ds][kk], fa[kk][i], acc[i][0], 0, 0, 0);
+            }
+        // the next tile's rows (requested a whole multiplication ago) and the previous tile's stores
+        asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+        const int n = tile / t.tpi;
+        const int oy0 = (tile - n * t.tpi) * t.TR;
+        const int64_t pix0 = ((int64_t)n * t.H + oy0) * t.W;
+        // (mrow is one of this lane's two rows: no division here, the epilogue's arithmetic is a large part of a tile)
+        auto rowpix = [&](int mrow, bool &ok, int64_t &pix) {
+            const int pr = ((mrow - wmi * 64) & 32) ? prow[1] : prow[0];
+            ok = oy0 + pr < t.H;
+            pix = pix0 + (ok ? mrow : 0);
+        };
+        gather_epilogue<TM, TN, WGM, 2, 64, false, true, true>(g, acc, epi, tid, lane, wave, wmi * 64, cj * 32, 0, tile, rowpix);
+        if constexpr(MODE == 2) {
+            bool okr[TM];
+#pragma unroll
+            for(int i = 0; i < TM; i++) {
+                int64_t pix;
+                rowpix(wmi * 64 + i * 32 + (lane & 31), okr[i], pix);
+            }
+            float s0, q0;
+            stats_lane_totals<TM, TN, true>(g.alpha, acc, okr, lane, s0, q0);
+            run_s += s0;
+            run_q += q0;
+        }
+        // every wavefront is past the barrier, so nobody reads this tile's buffer any more
+        if(tile + 2 * G < t.ntiles)
+            request(tile + 2 * G, b);
+        b ^= 1;
+    }
+    if constexpr(MODE == 2) {
+        g.stats = stats;
+        __syncthreads();
+        stats_block_write<TN, WGM, 2, 64>(g, epi + WGM * 8192, tid, lane, wave, cj * 32, 0, first_tile, run_s, run_q);
+    }
+}
+
+// Launches conv_rows64 if the geometry is its: returns false (and launches nothing) otherwise.  g: as for
+// launch_gather, with a = the NHWC input (pixel pitch lda), b = [Ngemm][9][64].
+template <bool FLIP> static bool launch_rows64(GatherArgs &g, const CLInfo &lout, hipStream_t st, size_t stats_floats, int *rc)
+{
+    static const bool off = getenv("SAGA_HIP_ROWS64") && atoi(getenv("SAGA_HIP_ROWS64")) == 0;
+    if(off || g.R != 3 || g.S != 3 || g.Cred != 64 || g.Ngemm > 64 || g.Ngemm % 8 || g.stride != 1 || g.pad != 1 ||
+       g.dil != 1 || g.IH != g.OH || g.IW != g.OW || g.OW < 8 || (g.bn_s && (g.bn_flags & SAGA_BN_ADD)) || g.bq_partial || !g.a_bytes || !g.b_bytes)
+        return false;
+    Rows64Args t;
+    t.H = g.OH;
+    t.W = g.OW;
+    static const int wgm = getenv("SAGA_HIP_ROWS64_WGM") ? atoi(getenv("SAGA_HIP_ROWS64_WGM")) : 4;
+    const int bm = wgm == 2 ? 128 : 256;
+    if(t.W > bm)
+        return false;
+    t.TR = std::min(bm / t.W, t.H);
+    t.tpi = (t.H + t.TR - 1) / t.TR;
+    const int64_t nimg = (int64_t)g.M / ((int64_t)t.H * t.W);
+    if(nimg * t.tpi > 0x7fffffff || nimg * t.tpi < 2 * num_cus()) // small problems: too few tiles to walk
+        return false;
+    t.ntiles = (int)(nimg * t.tpi);
+    t.npix = t.TR * t.W;
+    t.slots_row = t.W + 2;
+    t.chunks_tile = (t.TR + 2) * t.slots_row * 9;
+    t.buf_bytes = (t.chunks_tile * 16 + 1023) & ~1023;
+    const int epi_back = wgm == 2 ? 16384 : 32768; // gather_epilogue's scratch sits this far behind its base
+    const int epi_at = std::max(2 * t.buf_bytes, epi_back);
+    t.epi_off = epi_at - epi_back;
+    const int lds = epi_at + 4096;
+    const int blocks = std::min(t.ntiles, (wgm == 2 ? 2 : 1) * num_cus());
+    const bool vec_ok = (lout.pitch & 7) == 0 && aligned16(g.out) && ((lout.rows - 1) * lout.pitch + g.Ngemm) * 2 < 0x7fffff00ll &&
+                        (g.lda & 7) == 0 && aligned16(g.a);
+    if(!vec_ok || t.chunks_tile > 10 * (wgm == 2 ? 256 : 512) || lds > (wgm == 2 ? 76 : 150) * 1024 || (g.stats && (size_t)blocks * g.Ngemm * 2 > stats_floats))
+        return false;
+    static bool once = false;
+    if(!once) {
+        for(const void *k : {(const void *)conv_rows64<0, FLIP, 4>, (const void *)conv_rows64<1, FLIP, 4>,
+                             (const void *)conv_rows64<2, FLIP, 4>, (const void *)conv_rows64<0, FLIP, 2>,
+                             (const void *)conv_rows64<1, FLIP, 2>, (const void *)conv_rows64<2, FLIP, 2>}) {
+            const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+            if(e != hipSuccess) {
+                *rc = (int)e;
+                return true;
+            }
+        }
+        once = true;
+    }
+    g.classes = 1;
+    g.no_stage = 1;
+    g.nblk_n = 1;
+    g.out_bytes = (unsigned)(((lout.rows - 1) * lout.pitch + g.Ngemm) * 2);
+    g.stats_rows = blocks;
+#define GO_ROWS64(W_)                                                        \
+    do {                                                                     \
+        if(g.bn_s)                                                           \
+            conv_rows64<1, FLIP, W_><<<blocks, 128 * W_, lds, st>>>(g, t);    \
+        else if(g.stats)                                                     \
+            conv_rows64<2, FLIP, W_><<<blocks, 128 * W_, lds, st>>>(g, t);    \
+        else                                                                 \
+            conv_rows64<0, FLIP, W_><<<blocks, 128 * W_, lds, st>>>(g, t);    \
+    } while(0)
+    if(wgm == 2)
+        GO_ROWS64(2);
+    else
+        GO_ROWS64(4);
+#undef GO_ROWS64
+    *rc = 0;
+    return true;
+}
+
 // out[row][0..C) = 0 for rows of pitch `pitch` elements (C and pitch multiples of 8, 16-byte aligned)
 __global__ void __launch_bounds__(256) zero_rows(half_t *__restrict__ out, int64_t rows, int C, int64_t pitch)
 {
@@ -2565,7 +2798,9 @@ int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTe
     a.bq_partial = nullptr;
     if(!set_bn(a, bn, y, ly))
         return SAGA_HIP_EUNSUPPORTED;
-    const int rc = launch_gather<false>(a, st);
+    int rc = 0;
+    if(!(dma_stages() >= 2 && !pad && launch_rows64<false>(a, ly, st, stats_floats, &rc)))
+        rc = launch_gather<false>(a, st);
     if(stats_rows)
         *stats_rows = a.stats_rows;
     return rc;
@@ -2665,7 +2900,9 @@ int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const 
         a.bq_relu = link->relu ? 1 : 0;
         a.bq_partial = link->partial;
     }
-    const int rc = launch_gather<true>(a, st);
+    int rc = 0;
+    if(!(dma_stages() >= 2 && !link && launch_rows64<true>(a, ldx, st, 0, &rc)))
+        rc = launch_gather<true>(a, st);
     if(link && link->partial_rows)
         *link->partial_rows = a.stats_rows;
     return rc;

@@ -50,6 +50,10 @@ CONV_CASES = [
     # thin inputs under a 7-row filter: whole output rows per block, several tiles per image, a partial last tile
     (2, 3, 56, 56, 64, 7, 3, 2, 1),
     (1, 4, 33, 29, 24, 7, 3, 2, 1),
+    # 3x3 on 64 -> 64 channels with enough images for the kernel that keeps whole rows in LDS: four full tiles
+    # per image; a partial last tile, a row length that is no multiple of anything and 56 output channels
+    (37, 64, 56, 56, 64, 3, 1, 1, 1),
+    (130, 64, 30, 27, 56, 3, 1, 1, 1),
     # dilated (a tenth entry: dilation)
     (2, 16, 13, 12, 24, 3, 2, 1, 1, 2),
     (2, 32, 15, 15, 16, 3, 3, 2, 1, 3),
@@ -118,6 +122,8 @@ def test_conv_nonsquare_filter(R, S, layout, dtype):
                                   (2, 3, 30, 64, 7, 3, 2, 3), (2, 16, 8, 20, 3, 1, 1, 3),
                                   # the stem kernel: partial last tile; more tiles than blocks and a ragged channel tile
                                   (2, 3, 56, 64, 7, 3, 2, 3), (130, 3, 64, 40, 7, 3, 2, 1),
+                                  # 3x3 64 -> 64 with whole rows in LDS (see CONV_CASES)
+                                  (37, 64, 56, 64, 3, 1, 1, 3), (130, 64, 30, 56, 3, 1, 1, 1), (40, 64, 56, 64, 3, 1, 1, 0),
                                   # 3x3 layers of the last stages: many channels, tiles with dead rows, 7x7 images
                                   (3, 128, 14, 256, 3, 1, 1, 3), (6, 64, 7, 136, 3, 1, 1, 1), (2, 64, 28, 64, 3, 1, 1, 2)])
 def test_conv_with_folded_bn_inference(case):
@@ -159,6 +165,8 @@ BNSTATS_CASES = [
     (2, 3, 30, 64, 7, 3, 2, False),
     (2, 3, 56, 64, 7, 3, 2, False),
     (130, 3, 64, 64, 7, 3, 2, True),
+    (37, 64, 56, 64, 3, 1, 1, False),
+    (130, 64, 30, 56, 3, 1, 1, True),
     # 3x3 layers of the last stages: row counts that are no multiple of the tile, 7x7 images, 56x56 at 64 channels
     (3, 128, 14, 256, 3, 1, 1, True),
     (6, 64, 7, 136, 3, 1, 1, False),
