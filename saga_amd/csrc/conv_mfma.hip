@@ -1904,6 +1904,40 @@ __global__ void __launch_bounds__(256)
     }
 }
 
+// The same copy for dense 3-channel rows whose byte length is a multiple of 16 (W * 6 bytes: the RGB stem): one
+// block per padded row.  The source row comes into LDS through aligned 16-byte loads, every thread then builds
+// two padded pixels (16 bytes, one store) from six halves of the LDS copy - instead of three 2-byte global loads
+// and one 8-byte store per pixel.
+__global__ void __launch_bounds__(128)
+    pad_thin_rgb_rows(const half_t *__restrict__ x, int H, int W, int pad, half_t *__restrict__ x4, int Hp, int Wp)
+{
+    extern __shared__ __attribute__((aligned(16))) half_t row[];
+    const int hp = blockIdx.x % Hp, n = blockIdx.x / Hp;
+    const int h = hp - pad;
+    const bool inside = h >= 0 && h < H;
+    const int chunks = W * 6 / 16;
+    if(inside) {
+        const uint4_t *src = (const uint4_t *)(x + ((int64_t)n * H + h) * W * 3);
+        for(int i = threadIdx.x; i < chunks; i += blockDim.x)
+            ((uint4_t *)row)[i] = src[i];
+    }
+    __syncthreads();
+    half_t *dst = x4 + ((int64_t)n * Hp + hp) * Wp * 4;
+    for(int j = threadIdx.x; j < Wp / 2; j += blockDim.x) {
+        half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for(int e = 0; e < 2; e++) {
+            const int w = 2 * j + e - pad;
+            if(inside && w >= 0 && w < W) {
+                v[4 * e + 0] = row[3 * w + 0];
+                v[4 * e + 1] = row[3 * w + 1];
+                v[4 * e + 2] = row[3 * w + 2];
+            }
+        }
+        *(half8_t *)(dst + 8 * j) = v;
+    }
+}
+
 // wv[k][r][s*4 + c] = w[k][r][s][c] (s < S, c < C), 0 elsewhere; 32 halves per (k, r)
 __global__ void __launch_bounds__(256)
     repack_thin_filter(const half_t *__restrict__ w, half_t *__restrict__ wv, int C, int S, int64_t total)
@@ -1969,6 +2003,9 @@ struct ThinGeom {
     int Hp, Wp;
     size_t x4_bytes, wv_bytes;
 };
+
+static void launch_pad_thin(const half_t *x, int64_t pitch, const ConvGeom &g, half_t *x4, const ThinGeom &tg, int64_t px,
+                            hipStream_t st);
 
 static bool thin_ok(const ConvGeom &g, ThinGeom *t)
 {
@@ -2414,6 +2451,17 @@ template <bool FLIP> static bool launch_rows64(GatherArgs &g, const CLInfo &lout
     return true;
 }
 
+static void launch_pad_thin(const half_t *x, int64_t pitch, const ConvGeom &g, half_t *x4, const ThinGeom &tg, int64_t px,
+                            hipStream_t st)
+{
+    const int64_t blocks = (int64_t)g.N * tg.Hp;
+    if(g.C == 3 && pitch == 3 && (g.W * 6) % 16 == 0 && aligned16(x) && tg.Wp % 2 == 0 && blocks < (1ll << 31) &&
+       (size_t)g.W * 6 <= 48 * 1024)
+        pad_thin_rgb_rows<<<(int)blocks, 128, (size_t)g.W * 6, st>>>(x, g.H, g.W, g.pad, x4, tg.Hp, tg.Wp);
+    else
+        pad_thin<<<grid_for(px, 256, 1 << 20), 256, 0, st>>>(x, pitch, g.C, g.H, g.W, g.pad, x4, tg.Hp, tg.Wp, px);
+}
+
 // out[row][0..C) = 0 for rows of pitch `pitch` elements (C and pitch multiples of 8, 16-byte aligned)
 __global__ void __launch_bounds__(256) zero_rows(half_t *__restrict__ out, int64_t rows, int C, int64_t pitch)
 {
@@ -2679,8 +2727,7 @@ int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTe
             return SAGA_HIP_EWORKSPACE;
         half_t *x4 = (half_t *)ws, *wv = (half_t *)((char *)ws + tg.x4_bytes);
         const int64_t px = (int64_t)g.N * tg.Hp * tg.Wp, wn = (int64_t)g.K * g.R * 32;
-        pad_thin<<<grid_for(px, 256, 1 << 20), 256, 0, st>>>((const half_t *)x->ptr, lx.pitch, g.C, g.H, g.W, g.pad, x4,
-                                                              tg.Hp, tg.Wp, px);
+        launch_pad_thin((const half_t *)x->ptr, lx.pitch, g, x4, tg, px, st);
         repack_thin_filter<<<grid_for(wn, 256, 256 * 16), 256, 0, st>>>((const half_t *)w->ptr, wv, g.C, g.S, wn);
         GatherArgs a;
         a.a = x4;
@@ -2932,8 +2979,7 @@ int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, cons
             return SAGA_HIP_EUNSUPPORTED;
         half_t *x4 = (half_t *)ws;
         const int64_t px = (int64_t)g.N * tg.Hp * tg.Wp;
-        pad_thin<<<grid_for(px, 256, 1 << 20), 256, 0, st>>>((const half_t *)x->ptr, lx.pitch, g.C, g.H, g.W, g.pad, x4,
-                                                              tg.Hp, tg.Wp, px);
+        launch_pad_thin((const half_t *)x->ptr, lx.pitch, g, x4, tg, px, st);
         FilterArgs a;
         a.x = x4;
         a.ldx = 4;
