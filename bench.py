@@ -36,7 +36,7 @@ CONV_KINDS = ("convfwd", "convbwddata", "convbwddata.bn", "convbwdfilter")
 # the most GPU time in the training step.
 FAMILIES = {
     "conv": ("convfwd", "convfwd.bn", "convbwddata", "convbwddata.bn", "convbwdfilter"),
-    "batchnorm": ("bntrain", "bntrain.fused", "bnbwd", "bnbwd.fused", "bnbwd.linked"),
+    "batchnorm": ("bntrain", "bntrain.fused", "bnbwd", "bnbwd.fused", "bnbwd.linked", "bnbwd.pooled"),
     "pool": ("poolfwd", "poolfwd.bn", "poolbwd"),
 }
 

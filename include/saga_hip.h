@@ -298,6 +298,21 @@ int saga_hip_maxpool_fwd_codes(const SagaTensorView *x, const SagaTensorView *y,
  * ResNet stem - is neither written nor read.  flags: SAGA_BN_RELU or 0. */
 int saga_hip_maxpool_fwd_codes_bn(const SagaTensorView *x, const SagaTensorView *y, uint8_t *codes, int size, int pad,
                                   int stride, const float *scale_shift, int flags, saga_stream_t stream);
+
+/* Backward of that pair in one: cudnnPoolingBackward followed by cudnnBatchNormalizationBackwardEx
+ * (src/cuda/cuda_dnn.cpp:873-899, :2138-2163) without the tensor between them.  dp is the gradient of the POOLED
+ * output, codes the bytes the forward left, x the norm's input; both passes of the norm's backward gather their
+ * gradient from dp through the codes (rounded to the tensor's type as the pooling's backward would have stored
+ * it, masked by the relu recomputed from x when flags has SAGA_BN_RELU - b is then required).  Writes ds, db
+ * (beta_p) and dx = s*invstd*(g - db/M - (x - mean)*invstd*ds/M) + beta_dx*dx.  3x3 windows at stride 2 on
+ * channels-last tensors with whole 16-byte channel vectors; SAGA_HIP_EUNSUPPORTED otherwise (the size query
+ * returns 0 then). */
+size_t saga_hip_bn_bwd_pooled_workspace_size(const SagaTensorView *x, const SagaTensorView *dp, int size, int pad,
+                                             int stride);
+int saga_hip_bn_bwd_pooled(const SagaTensorView *x, const SagaTensorView *dp, const uint8_t *codes,
+                           const SagaTensorView *dx, const float *s, const float *b, const float *save_mean,
+                           const float *save_invstd, float *ds, float *db, float beta_dx, float beta_p, int flags,
+                           int size, int pad, int stride, void *workspace, size_t ws_bytes, saga_stream_t stream);
 int saga_hip_maxpool_bwd_codes(const uint8_t *codes, const SagaTensorView *dy, const SagaTensorView *dx, int size,
                                int pad, int stride, float beta, saga_stream_t stream);
 

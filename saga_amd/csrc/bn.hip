@@ -774,6 +774,14 @@ static size_t ws_floats(int64_t rows, int C, int dtype)
 
 } // namespace
 
+int bn_launch_bwd_finalize(const float *partial, int rows, const float *s, const float *save_invstd, float *ds, float *db,
+                           float *coef, double M, int C, float beta_p, hipStream_t st)
+{
+    bn_bwd_finalize<<<C, 256, 0, st>>>(partial, rows, s, save_invstd, ds, db, coef, M, C, beta_p);
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
 extern "C" {
 
 size_t saga_hip_bn_workspace_size(const SagaTensorView *x)

@@ -162,3 +162,9 @@ static inline int grid_for(int64_t work, int block, int cap = 256 * 64)
         g = cap;
     return (int)g;
 }
+
+// bn.hip: the per-channel step between the two passes of a batch norm's backward (bn_bwd_finalize), for kernels
+// in other files that produce the partial sums [rows][C][2] themselves
+int bn_launch_bwd_finalize(const float *partial, int rows, const float *s, const float *save_invstd, float *ds, float *db,
+                           float *coef, double M, int C, float beta_p, hipStream_t st);
+

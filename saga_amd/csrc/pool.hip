@@ -576,6 +576,142 @@ __global__ void __launch_bounds__(256)
     }
 }
 
+// Backward of max pooling (3x3, stride 2, position codes) and of the batch norm (+ relu) in front of it in one:
+// the pooled gradient is gathered as in maxpool_bwd_codes_3x3s2_k - a thread owns a 2x2 input patch and the four
+// windows that reach it - rounded to T as the unfused pooling would have stored it, masked by the norm's relu
+// (recomputed from the norm's input x as half(fma(x, sc, sh)) > 0, the forward's own expression), and goes
+// straight into the norm's backward: MODE 0 leaves per block and channel the sums of g and g * (x - mean),
+// MODE 1 writes dx = a * (g - k0 - (x - mean) * k1) (+ beta * dx).  The norm's output gradient never exists.
+// A block walks AG consecutive patch rows, so that there are few partial rows.
+// blockIdx.z = sample, blockIdx.y = group of patch rows, threadIdx.x = channel vector, threadIdx.y (+ blockIdx.x) = b
+constexpr int BNPOOL_AG = 16; // patch rows per block (measured on the 112x112 stem: 1 row 579 us, 8 rows 450 us, 16 or 64 rows 430 us)
+template <typename T, int VN, int MODE, int AG>
+__global__ void __launch_bounds__(256)
+    bn_pool_bwd_3x3s2_k(const uint8_t *__restrict__ codes, DView dp, DView x, DView dx, int pad, int na,
+                        const float *__restrict__ mean_, const float *__restrict__ s_, const float *__restrict__ invstd_,
+                        const float *__restrict__ b_, int relu, const float *__restrict__ coef, float *__restrict__ partial,
+                        float beta)
+{
+    __shared__ float red[MODE == 0 ? 256 * VN * 2 : 1];
+    const int C = x.d[1], H = x.d[2], W = x.d[3], P = dp.d[2], Q = dp.d[3];
+    const int n = blockIdx.z;
+    const int b = blockIdx.x * blockDim.y + threadIdx.y;
+    const int c = threadIdx.x * VN;
+    const bool live = c < C && 2 * b - 1 - pad < W;
+    float mean[VN], sc[VN], sh[VN], k0[VN], k1[VN], a0[VN], a1[VN];
+#pragma unroll
+    for(int j = 0; j < VN; j++) {
+        a0[j] = a1[j] = 0.0f;
+        mean[j] = sc[j] = sh[j] = k0[j] = k1[j] = 0.0f;
+        if(live) {
+            mean[j] = mean_[c + j];
+            sc[j] = MODE == 1 ? coef[c + j] : s_[c + j] * invstd_[c + j]; // s * invstd, also the forward's scale
+            sh[j] = relu ? __builtin_fmaf(-mean[j], sc[j], b_[c + j]) : 0.0f;
+            if(MODE == 1) {
+                k0[j] = coef[C + c + j];
+                k1[j] = coef[2 * C + c + j];
+            }
+        }
+    }
+    const int a_end = (blockIdx.y + 1) * AG < na ? (blockIdx.y + 1) * AG : na;
+    if(live)
+        for(int a = blockIdx.y * AG; a < a_end; a++) {
+            float g[4][VN];
+            typename CodeVec<VN>::type cd[4];
+            bool okw[4];
+#pragma unroll
+            for(int e = 0; e < 4; e++) {
+                const int p = a - 1 + (e >> 1), q = b - 1 + (e & 1);
+                okw[e] = p >= 0 && p < P && q >= 0 && q < Q;
+                const int pc = p < 0 ? 0 : p >= P ? P - 1 : p, qc = q < 0 ? 0 : q >= Q ? Q - 1 : q;
+                PV<T, VN>::load((const T *)dp.ptr + off4(dp, n, c, pc, qc), g[e]);
+                cd[e] = *(const typename CodeVec<VN>::type *)(codes + ((((size_t)n * P + pc) * Q + qc) * C + c));
+            }
+            float xv[4][VN];
+            bool in[4];
+#pragma unroll
+            for(int e = 0; e < 4; e++) {
+                const int h = 2 * a - 1 + (e >> 1) - pad, w = 2 * b - 1 + (e & 1) - pad;
+                in[e] = h >= 0 && h < H && w >= 0 && w < W;
+                const int hc = h < 0 ? 0 : h >= H ? H - 1 : h, wc = w < 0 ? 0 : w >= W ? W - 1 : w;
+                PV<T, VN>::load((const T *)x.ptr + off4(x, n, c, hc, wc), xv[e]);
+            }
+            auto code = [&](int e, int j) -> unsigned {
+                if constexpr(VN == 8)
+                    return (cd[e][j >> 2] >> (8 * (j & 3))) & 255u;
+                else
+                    return (cd[e] >> (8 * j)) & 255u;
+            };
+            auto term = [&](int e, unsigned k, int j) { return (okw[e] && code(e, j) == k) ? g[e][j] : 0.0f; };
+            float out[4][VN];
+#pragma unroll
+            for(int j = 0; j < VN; j++) {
+                out[0][j] = term(0, 4, j);
+                out[1][j] = term(0, 5, j) + term(1, 3, j);
+                out[2][j] = term(0, 7, j) + term(2, 1, j);
+                out[3][j] = term(0, 8, j) + term(1, 6, j) + term(2, 2, j) + term(3, 0, j);
+            }
+#pragma unroll
+            for(int e = 0; e < 4; e++) {
+                if(!in[e])
+                    continue;
+                float res[VN];
+#pragma unroll
+                for(int j = 0; j < VN; j++) {
+                    float gv = (float)(T)out[e][j]; // as the pooling's backward would have stored it
+                    if(relu && !((float)(T)__builtin_fmaf(xv[e][j], sc[j], sh[j]) > 0.0f))
+                        gv = 0.0f;
+                    const float xm = xv[e][j] - mean[j];
+                    if(MODE == 0) {
+                        a0[j] += gv;
+                        a1[j] += gv * xm;
+                    } else {
+                        res[j] = sc[j] * (gv - k0[j] - xm * k1[j]);
+                    }
+                }
+                if(MODE == 1) {
+                    const int h = 2 * a - 1 + (e >> 1) - pad, w = 2 * b - 1 + (e & 1) - pad;
+                    T *o = (T *)dx.ptr + off4(dx, n, c, h, w);
+                    if(beta != 0.0f) {
+                        float old[VN];
+                        PV<T, VN>::load(o, old);
+#pragma unroll
+                        for(int j = 0; j < VN; j++)
+                            res[j] += beta * old[j];
+                    }
+                    PV<T, VN>::store(o, res);
+                }
+            }
+        }
+    if constexpr(MODE == 0) {
+        // threads along y hold different columns of the same channels: add them up in a fixed order
+        const int t = threadIdx.y * blockDim.x + threadIdx.x;
+#pragma unroll
+        for(int j = 0; j < VN; j++) {
+            red[t * VN * 2 + j] = a0[j];
+            red[t * VN * 2 + VN + j] = a1[j];
+        }
+        __syncthreads();
+        if(threadIdx.y == 0 && c < C) {
+            for(int ty = 1; ty < (int)blockDim.y; ty++) {
+                const int u = ty * blockDim.x + threadIdx.x;
+#pragma unroll
+                for(int j = 0; j < VN; j++) {
+                    a0[j] += red[u * VN * 2 + j];
+                    a1[j] += red[u * VN * 2 + VN + j];
+                }
+            }
+            const int64_t row = ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+            float *o = partial + (row * C + c) * 2;
+#pragma unroll
+            for(int j = 0; j < VN; j++) {
+                o[j * 2] = a0[j];
+                o[j * 2 + 1] = a1[j];
+            }
+        }
+    }
+}
+
 static int vec_for(int dtype, std::initializer_list<const SagaTensorView *> vs)
 {
     const int vn = dtype == SAGA_HALF ? 8 : 4;
@@ -838,3 +974,85 @@ int saga_hip_maxpool_bwd_codes(const uint8_t *codes, const SagaTensorView *dy, c
 
 } // extern "C"
 
+// Shape of the fused launch: patches along rows in groups of BNPOOL_AG; returns the number of partial rows.
+static int64_t bn_pool_launch_shape(const SagaTensorView *x, int pad, dim3 &grid, dim3 &block, int *na_out, int ag = BNPOOL_AG)
+{
+    const int vn = x->dtype == SAGA_HALF ? 8 : 4;
+    const int na = (x->dims[2] + pad) / 2 + 1, nb = (x->dims[3] + pad) / 2 + 1;
+    codes_launch_shape(x->dims[1] / vn, nb, (na + ag - 1) / ag, x->dims[0], grid, block);
+    if(na_out)
+        *na_out = na;
+    return (int64_t)grid.x * grid.y * grid.z;
+}
+
+static bool bn_pool_ok(const SagaTensorView *x, const SagaTensorView *dp, const SagaTensorView *dx, int size, int pad, int stride)
+{
+    if(!valid_view(x) || !valid_view(dp) || size != 3 || stride != 2 || pad < 0 || pad > 2)
+        return false;
+    if(dx && (!valid_view(dx) || !same_dims(x, dx) || dx->dtype != x->dtype))
+        return false;
+    if(dp->dims[0] != x->dims[0] || dp->dims[1] != x->dims[1] || dp->dims[2] != pool_dim(x->dims[2], size, pad, stride) ||
+       dp->dims[3] != pool_dim(x->dims[3], size, pad, stride) || dp->dtype != x->dtype)
+        return false;
+    return codes_ok(x, dp, size, pad, stride) && (!dx || codes_ok(dx, dp, size, pad, stride));
+}
+
+extern "C" {
+
+size_t saga_hip_bn_bwd_pooled_workspace_size(const SagaTensorView *x, const SagaTensorView *dp, int size, int pad, int stride)
+{
+    if(!x || !dp || !bn_pool_ok(x, dp, nullptr, size, pad, stride))
+        return 0;
+    dim3 grid, block;
+    const int64_t rows = bn_pool_launch_shape(x, pad, grid, block, nullptr);
+    return ((size_t)rows * x->dims[1] * 2 + 3 * (size_t)x->dims[1] + 64) * sizeof(float);
+}
+
+int saga_hip_bn_bwd_pooled(const SagaTensorView *x, const SagaTensorView *dp, const uint8_t *codes, const SagaTensorView *dx,
+                           const float *s, const float *b, const float *save_mean, const float *save_invstd, float *ds,
+                           float *db, float beta_dx, float beta_p, int flags, int size, int pad, int stride, void *workspace,
+                           size_t ws_bytes, saga_stream_t stream)
+{
+    if(!x || !dp || !dx || !codes || !s || !save_mean || !save_invstd || !ds || !db)
+        return SAGA_HIP_EINVAL;
+    if(flags & ~SAGA_BN_RELU)
+        return SAGA_HIP_EUNSUPPORTED;
+    const int relu = flags & SAGA_BN_RELU ? 1 : 0;
+    if(relu && !b)
+        return SAGA_HIP_EINVAL; // the mask is rebuilt from x, which takes the bias
+    if(!bn_pool_ok(x, dp, dx, size, pad, stride) || ((uintptr_t)codes & 7))
+        return SAGA_HIP_EUNSUPPORTED;
+    const size_t need = saga_hip_bn_bwd_pooled_workspace_size(x, dp, size, pad, stride);
+    if(!workspace || ws_bytes < need)
+        return SAGA_HIP_EWORKSPACE;
+    dim3 grid, block;
+    int na = 0;
+    const int64_t rows = bn_pool_launch_shape(x, pad, grid, block, &na);
+    if(rows >= (1ll << 31))
+        return SAGA_HIP_EUNSUPPORTED;
+
+    const int C = x->dims[1];
+    float *partial = (float *)workspace, *coef = partial + (size_t)rows * C * 2;
+    hipStream_t st = as_stream(stream);
+    const DView dvp = dview(dp), dvx = dview(x), dvdx = dview(dx);
+    const double M = (double)x->dims[0] * x->dims[2] * x->dims[3];
+#define GO(T, VN)                                                                                                       \
+    do {                                                                                                                \
+        bn_pool_bwd_3x3s2_k<T, VN, 0, BNPOOL_AG><<<grid, block, 0, st>>>(codes, dvp, dvx, dvdx, pad, na, save_mean, s,     \
+                                                                        save_invstd, b, relu, nullptr, partial, 0.0f); \
+        const int rc = bn_launch_bwd_finalize(partial, (int)rows, s, save_invstd, ds, db, coef, M, C, beta_p, st);       \
+        if(rc)                                                                                                          \
+            return rc;                                                                                                  \
+        bn_pool_bwd_3x3s2_k<T, VN, 1, BNPOOL_AG><<<grid, block, 0, st>>>(codes, dvp, dvx, dvdx, pad, na, save_mean, s,           \
+                                                                  save_invstd, b, relu, coef, nullptr, beta_dx);        \
+    } while(0)
+    if(x->dtype == SAGA_HALF)
+        GO(half_t, 8);
+    else
+        GO(float, 4);
+#undef GO
+    SAGA_CHECK_LAUNCH();
+    return 0;
+}
+
+} // extern "C"

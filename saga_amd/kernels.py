@@ -87,6 +87,8 @@ SIGNATURES = {
     "saga_hip_maxpool_fwd_codes": (_I, [_TV, _TV, _VP, _I, _I, _I, _VP]),
     "saga_hip_maxpool_bwd_codes": (_I, [_VP, _TV, _TV, _I, _I, _I, _F, _VP]),
     "saga_hip_maxpool_fwd_codes_bn": (_I, [_TV, _TV, _VP, _I, _I, _I, _VP, _I, _VP]),
+    "saga_hip_bn_bwd_pooled_workspace_size": (_SZ, [_TV, _TV, _I, _I, _I]),
+    "saga_hip_bn_bwd_pooled": (_I, [_TV, _TV, _VP, _TV, _VP, _VP, _VP, _VP, _VP, _VP, _F, _F, _I, _I, _I, _I, _VP, _SZ, _VP]),
     "saga_hip_softmax": (_I, [_TV, _TV, _VP]),
     "saga_hip_spatial_transform": (_I, [_TV, _VP, _TV, _VP]),
     "saga_hip_dropout_fwd": (_I, [_TV, _TV, _F, C.c_uint64, C.c_uint64, _VP]),

@@ -1315,6 +1315,53 @@ struct BnMaxPoolFwdCodes : public HipOperation {
     double bytes() const override { return nbytes(bn_->x_) + nbytes(y_) + nbytes(codes_); }
 };
 
+// The backward of that pair in one operation: the gradient of the pooled output goes through the position codes
+// straight into the two passes of the norm's backward, and the gradient of the norm's output is never stored.
+struct BnBwdPooled : public HipOperation {
+    const std::shared_ptr<BnTrain> fwd_;
+    const T codes_, dp_, dx_, ds_, db_;
+    const int flags_, size_, pad_, stride_;
+    float dx_beta_ = 0, ds_beta_ = 0, db_beta_ = 0;
+    BnBwdPooled(HipProgram &p, std::shared_ptr<BnTrain> fwd, T codes, T dp, T dx, T ds, T db, int flags, int size, int pad,
+                int stride)
+      : HipOperation("bnbwd.pooled"), fwd_(fwd), codes_(codes), dp_(dp), dx_(dx), ds_(ds), db_(db), flags_(flags)
+      , size_(size), pad_(pad), stride_(stride)
+    {
+        const SagaTensorView vx = fwd->x_->shapeView(), vdp = dp->shapeView();
+        p.m_ctx->m_workspace.request(saga_hip_bn_bwd_pooled_workspace_size(&vx, &vdp, size, pad, stride));
+    }
+    void exec(HipProgram &p) override
+    {
+        const SagaTensorView vx = fwd_->x_->view(), vdp = dp_->view(), vdx = dx_->view();
+        chkSaga(saga_hip_bn_bwd_pooled(&vx, &vdp, (const uint8_t *)codes_->deviceMem(), &vdx,
+                                       (const float *)fwd_->s_->deviceMem(), (const float *)fwd_->b_->deviceMem(),
+                                       (const float *)fwd_->sm_->deviceMem(), (const float *)fwd_->sv_->deviceMem(),
+                                       (float *)ds_->deviceMem(), (float *)db_->deviceMem(), dx_beta_, ds_beta_, flags_, size_,
+                                       pad_, stride_, p.m_ctx->m_workspace.ptr(), p.m_ctx->m_workspace.size(), S(p)));
+    }
+    HipOpArgs listInputs() const override
+    {
+        return {{"x", fwd_->x_}, {"dp", dp_}, {"codes", codes_}, {"s", fwd_->s_}, {"b", fwd_->b_}, {"sm", fwd_->sm_},
+                {"sv", fwd_->sv_}};
+    }
+    HipOpArgs listOutputs() const override { return {{"dx", dx_}, {"ds", ds_}, {"db", db_}}; }
+    // both passes read x, the pooled gradient and the codes; the second writes dx
+    double bytes() const override
+    {
+        return nbytes(dx_) * (3 + (dx_beta_ != 0 ? 1 : 0)) + 2 * (nbytes(dp_) + nbytes(codes_));
+    }
+    float *getBeta(const T &t) override
+    {
+        if(t == dx_)
+            return &dx_beta_;
+        if(t == ds_)
+            return &ds_beta_;
+        if(t == db_)
+            return &db_beta_;
+        return nullptr;
+    }
+};
+
 // what saga_hip_maxpool_*_codes accept (anything else takes the x / y based kernels)
 static bool maxpool_codes_fit(const HipTensor &x, const HipTensor &y, const HipTensor *dx, const HipTensor *dy, int size,
                               int pad, int stride)
@@ -1761,6 +1808,53 @@ REGISTER_HIP_TRANSFORM(100, ProgramType::INFERENCE | ProgramType::TRAINING, conc
 // concat buffer the norm writes a slice of), not the host, not the anomaly checks - normalises its windows on the
 // fly from the norm's input, and the norm's forward only finalises its statistics.  The norm must get its sums
 // from the producing convolution, have no residual, and a backward pass that rebuilds the relu mask from x.
+// The backward half: the pooling's backward (codes -> gradient of the norm's output) and the norm's backward that
+// alone reads that gradient become one operation, if the fused kernels take the geometry.
+static void fuse_bn_pooling_backward(HipProgram &p, HipOps &ops, const std::shared_ptr<BnTrain> &bn, const T &codes, int size,
+                                     int pad, int stride)
+{
+    if(getenv("SAGA_HIP_NO_BN_POOL_BWD_FUSE"))
+        return;
+    ssize_t ipb = -1, ibn = -1;
+    for(size_t i = 0; i < ops.size(); i++) {
+        if(auto *pb = dynamic_cast<MaxPoolBwdCodes *>(ops[i].get()); pb && pb->codes_ == codes)
+            ipb = (ssize_t)i;
+        if(auto *bb = dynamic_cast<BnBwd *>(ops[i].get()); bb && bb->fwd_ == bn)
+            ibn = (ssize_t)i;
+    }
+    if(ipb < 0 || ibn < 0 || ipb > ibn)
+        return;
+    auto *pb = static_cast<MaxPoolBwdCodes *>(ops[ipb].get());
+    auto *bb = static_cast<BnBwd *>(ops[ibn].get());
+    const T &g = pb->dx_; // gradient of the norm's output
+    if(bb->dy_ != g || bb->link_ || bb->dz_ || pb->beta_ != 0.0f)
+        return;
+    // nobody else reads or writes that gradient, and the host does not hold it
+    for(size_t i = 0; i < ops.size(); i++) {
+        if((ssize_t)i == ipb || (ssize_t)i == ibn)
+            continue;
+        for(const auto &o : ops[i]->listOutputs())
+            if(o.second->m_storage == g->m_storage)
+                return;
+        for(const auto &in : ops[i]->listInputs())
+            if(in.second->m_storage == g->m_storage)
+                return;
+    }
+    const auto &ex = p.m_ctx->m_exported;
+    if(std::any_of(ex.begin(), ex.end(), [&](const auto &e) { return e == g->m_storage; }))
+        return;
+    const SagaTensorView vx = bn->x_->shapeView(), vdp = pb->dy_->shapeView();
+    if(bb->dx_->m_data_type != bn->x_->m_data_type || !bb->dx_->cpacked() || !pb->dy_->cpacked() ||
+       saga_hip_bn_bwd_pooled_workspace_size(&vx, &vdp, size, pad, stride) == 0)
+        return;
+    auto fused = std::make_shared<BnBwdPooled>(p, bn, codes, pb->dy_, bb->dx_, bb->ds_, bb->db_, bb->flags_, size, pad, stride);
+    fused->dx_beta_ = bb->dx_beta_;
+    fused->ds_beta_ = bb->ds_beta_;
+    fused->db_beta_ = bb->db_beta_;
+    ops[ibn] = fused;
+    ops.erase(ops.begin() + ipb);
+}
+
 void fuse_bn_pooling(HipProgram &p, HipOps &ops)
 {
     if(p.m_pc.disable_op_fusing || p.m_pc.anomaly_detect || getenv("SAGA_HIP_NO_BN_POOL_FUSE") ||
@@ -1812,6 +1906,7 @@ void fuse_bn_pooling(HipProgram &p, HipOps &ops)
         bn->ss_ = std::make_shared<HipTensor>(Tensor::DataType::FLOAT, sd, HipLayout::NCHW, p.m_ctx.get(),
                                               std::string("scaleshift"));
         ops[ip] = std::make_shared<BnMaxPoolFwdCodes>(bn, pool->y_, pool->codes_, pool->size_, pool->pad_, pool->stride_);
+        fuse_bn_pooling_backward(p, ops, bn, pool->codes_, pool->size_, pool->pad_, pool->stride_);
     }
 }
 

@@ -801,6 +801,63 @@ def test_maxpool_on_a_batch_norm_that_is_never_written(k, pad, stride, H, relu, 
     assert_close(y1, want, dtype, "pooled batch norm")
 
 
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("pad,H,W,relu,beta", [(1, 12, 14, True, 0.0), (1, 9, 11, True, 1.0), (1, 16, 16, False, 0.0), (0, 11, 13, True, 0.0)])
+def test_batch_norm_backward_through_a_max_pooling(pad, H, W, relu, beta, dtype):
+    """saga_hip_bn_bwd_pooled - the backward of a max pooling (3x3, stride 2) and of the batch norm (+ relu) in front
+    of it without the gradient tensor between them - against saga_hip_maxpool_bwd_codes followed by
+    saga_hip_bn_bwd_ex: dx equal to the last bit or two of the type, ds and db to 1e-5."""
+    rng = np.random.default_rng(H * 31 + W + pad)
+    Cc = 16 if dtype == torch.float16 else 8
+    N = 3
+    shape = (N, Cc, H, W)
+    x = rnd(rng, *shape, dtype=dtype)
+    P, Q = ref.pool_out(H, 3, pad, 2), ref.pool_out(W, 3, pad, 2)
+    s, b = (1 + 0.3 * rng.standard_normal(Cc)).astype(np.float32), (0.2 * rng.standard_normal(Cc)).astype(np.float32)
+    flags = K.BN_RELU if relu else 0
+    L = K.lib()
+    xd = dev(x, dtype, "nhwc")
+    xh = host(xd).astype(np.float64)
+    mean, var = xh.mean((0, 2, 3)), xh.var((0, 2, 3))
+    sm, sv = dev(mean.astype(np.float32)), dev((1.0 / np.sqrt(var + 1e-5)).astype(np.float32))
+    sd, bd = dev(s), dev(b)
+    # forward: the norm's output and the pooling's codes, by the unfused operators
+    yd = dev(np.zeros(shape, np.float32), dtype, "nhwc")
+    md, vd = dev(mean.astype(np.float32)), dev(var.astype(np.float32))
+    K.check(L.saga_hip_bn_infer(C.byref(K.view(xd)), None, C.byref(K.view(yd)), K.ptr(sd), K.ptr(bd), K.ptr(md), K.ptr(vd),
+                                1e-5, flags, S()))
+    yp = dev(np.zeros((N, Cc, P, Q), np.float32), dtype, "nhwc")
+    codes = torch.full((N, P, Q, Cc), 255, dtype=torch.uint8, device="cuda")
+    K.check(L.saga_hip_maxpool_fwd_codes(C.byref(K.view(yd)), C.byref(K.view(yp)), K.ptr(codes), 3, pad, 2, S()))
+    dp = rnd(rng, N, Cc, P, Q, dtype=dtype)
+    dpd = dev(dp, dtype, "nhwc")
+    init = rnd(rng, *shape, dtype=dtype)
+
+    # unfused: pooling backward into dy, then the norm's backward
+    dyd = dev(np.zeros(shape, np.float32), dtype, "nhwc")
+    K.check(L.saga_hip_maxpool_bwd_codes(K.ptr(codes), C.byref(K.view(dpd)), C.byref(K.view(dyd)), 3, pad, 2, 0.0, S()))
+    dx0 = dev(init, dtype, "nhwc")
+    ds0, db0 = dev(np.ones(Cc, np.float32)), dev(np.ones(Cc, np.float32))
+    wsb = torch.zeros(L.saga_hip_bn_workspace_size(C.byref(K.view(xd))), dtype=torch.uint8, device="cuda")
+    K.check(L.saga_hip_bn_bwd_ex(C.byref(K.view(xd)), None if relu else None, C.byref(K.view(dyd)), C.byref(K.view(dx0)), None,
+                                 K.ptr(sd), K.ptr(bd), K.ptr(sm), K.ptr(sv), K.ptr(ds0), K.ptr(db0), beta, 0.0, 0.0, flags,
+                                 None, K.ptr(wsb), wsb.numel(), S()))
+    # fused
+    need = L.saga_hip_bn_bwd_pooled_workspace_size(C.byref(K.view(xd)), C.byref(K.view(dpd)), 3, pad, 2)
+    assert need > 0
+    ws = torch.full((need,), 0x7f, dtype=torch.uint8, device="cuda")
+    dx1 = dev(init, dtype, "nhwc")
+    ds1, db1 = dev(np.ones(Cc, np.float32)), dev(np.ones(Cc, np.float32))
+    K.check(L.saga_hip_bn_bwd_pooled(C.byref(K.view(xd)), C.byref(K.view(dpd)), K.ptr(codes), C.byref(K.view(dx1)), K.ptr(sd),
+                                     K.ptr(bd), K.ptr(sm), K.ptr(sv), K.ptr(ds1), K.ptr(db1), beta, 0.0, flags, 3, pad, 2,
+                                     K.ptr(ws), need, S()))
+    np.testing.assert_allclose(host(ds1), host(ds0), rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(host(db1), host(db0), rtol=1e-5, atol=1e-5)
+    assert_close(host(dx1), host(dx0), dtype, "dx", 2e-3 if dtype == torch.float16 else 1e-5)
+    # what it does not take is refused by the size query and by the call
+    assert L.saga_hip_bn_bwd_pooled_workspace_size(C.byref(K.view(xd)), C.byref(K.view(dpd)), 2, pad, 2) == 0
+
+
 def test_pooling_golden(golden):
     g = golden["ops"]
     x = T(g, "pooling_input")
