@@ -4,7 +4,8 @@ The kernel library reads its switches once per process, so every case runs a sel
 test files in a child process with the switch set: the register-staged fp16 convolution kernels, the
 direct (one output per lane) convolutions, the table-driven fp32 convolutions, batch-norm backward with
 the relu mask read from y, and the engine without relu bit masks / position codes / arena / batched
-filter transposes / batch-norm backward link / reordering of fan-in writers."""
+filter transposes / batch-norm backward link / reordering of fan-in writers / row-resident convolution kernels /
+pooled batch norm."""
 import os
 import subprocess
 import sys
@@ -29,6 +30,13 @@ CASES = [
     ("SAGA_HIP_NO_BATCHED_TRANSPOSE", "1", ["tests/test_gpu_networks.py", "-k", "training and not links"]),
     ("SAGA_HIP_NO_BNBWD_LINK", "1", ["tests/test_gpu_networks.py", "-k", "training and not links"]),
     ("SAGA_HIP_NO_WRITER_REORDER", "1", ["tests/test_gpu_networks.py", "-k", "training"]),
+    # the stem and the 3x3 64 -> 64 layers through the gather kernel instead of the row-resident ones
+    ("SAGA_HIP_THIN_ROWS", "0", ["tests/test_gpu_ops.py", "-k", "test_conv_fwd_bwd or folded_bn or bnstats"]),
+    ("SAGA_HIP_ROWS64", "0", ["tests/test_gpu_ops.py", "-k", "test_conv_fwd_bwd or folded_bn or bnstats"]),
+    ("SAGA_HIP_ROWS64_WGM", "2", ["tests/test_gpu_ops.py", "-k", "test_conv_fwd_bwd or folded_bn or bnstats"]),
+    # batch norm and max pooling as separate operations (forward and backward; backward only)
+    ("SAGA_HIP_NO_BN_POOL_FUSE", "1", ["tests/test_gpu_networks.py", "-k", "resnet50"]),
+    ("SAGA_HIP_NO_BN_POOL_BWD_FUSE", "1", ["tests/test_gpu_networks.py", "-k", "resnet50"]),
 ]
 
 
