@@ -472,6 +472,22 @@ template <int TM, int TN, int BN, bool BWD> __device__ __forceinline__ bool stor
     return TM == 2 && TN == 2 && BN >= 128 && vec_ok && !(BWD && g.classes > 1) && !g.no_stage;
 }
 
+// Inference with a folded batch norm: scale = s/sqrt(v+eps) and shift = b - m*scale of the block's BN channels
+// as a table in LDS (bnp: 2 * BN floats).  The caller puts barriers around it.
+template <int BN> __device__ __forceinline__ void bnfold_table(const GatherArgs &g, float *bnp, int tid, int n0)
+{
+    if(tid < BN) {
+        const int n = n0 + tid;
+        float sc = 0.0f, sh = 0.0f;
+        if(n < g.Ngemm) {
+            sc = g.bn_s[n] * rsqrtf(g.bn_v[n] + g.bn_eps);
+            sh = g.bn_b[n] - g.bn_m[n] * sc;
+        }
+        bnp[tid] = sc;
+        bnp[BN + tid] = sh;
+    }
+}
+
 // BUFST: the direct 16-byte stores go through a range-checked buffer with an out-of-range offset for the lanes that
 // have nothing to store, so that every wavefront issues the same number of store instructions whatever its rows
 // (a caller that counts outstanding memory operations needs that).
@@ -479,23 +495,13 @@ template <int TM, int TN, int WGM, int WGN, int BN, bool BWD, bool MASK, bool BU
 __device__ __forceinline__ void gather_epilogue(const GatherArgs &g, float16_t (&acc)[TM][TN], char *smem, int tid, int lane,
                                                 int wave, int wm, int wn, int n0, int stats_row, RowPix rowpix)
 {
-    // Inference with a folded batch norm: scale = s/sqrt(v+eps) and shift = b - m*scale of the
-    // block's BN channels go into LDS once (the stage memory is free after the last slice).
-    // (behind the tiles that the wavefronts stage their outputs in)
+    // (the table sits behind the tiles that the wavefronts stage their outputs in; the stage memory is free
+    // after the last slice)
     float *bnp = (float *)(smem + WGM * WGN * TM * 32 * TN * 64);
     if constexpr(!BWD) {
         if(g.bn_s) {
             __syncthreads(); // every wavefront is done reading the last slice
-            if(tid < BN) {
-                const int n = n0 + tid;
-                float sc = 0.0f, sh = 0.0f;
-                if(n < g.Ngemm) {
-                    sc = g.bn_s[n] * rsqrtf(g.bn_v[n] + g.bn_eps);
-                    sh = g.bn_b[n] - g.bn_m[n] * sc;
-                }
-                bnp[tid] = sc;
-                bnp[BN + tid] = sh;
-            }
+            bnfold_table<BN>(g, bnp, tid, n0);
             __syncthreads();
         }
     }
@@ -2381,6 +2387,338 @@ template <int MODE, bool FLIP, int WGM> __global__ void __launch_bounds__(128 * 
     }
 }
 
+// s_waitcnt vmcnt(n) for a count known only at run time (the same for the whole wavefront)
+__device__ __forceinline__ void wait_vmcnt(int n)
+{
+#define SAGA_VMCNT_CASE(k) case k: asm volatile("s_waitcnt vmcnt(" #k ")" ::: "memory"); break;
+    switch(__builtin_amdgcn_readfirstlane(n)) {
+        SAGA_VMCNT_CASE(1) SAGA_VMCNT_CASE(2) SAGA_VMCNT_CASE(3) SAGA_VMCNT_CASE(4) SAGA_VMCNT_CASE(5) SAGA_VMCNT_CASE(6)
+        SAGA_VMCNT_CASE(7) SAGA_VMCNT_CASE(8) SAGA_VMCNT_CASE(9) SAGA_VMCNT_CASE(10) SAGA_VMCNT_CASE(11) SAGA_VMCNT_CASE(12)
+        SAGA_VMCNT_CASE(13) SAGA_VMCNT_CASE(14) SAGA_VMCNT_CASE(15) SAGA_VMCNT_CASE(16) SAGA_VMCNT_CASE(17) SAGA_VMCNT_CASE(18)
+        SAGA_VMCNT_CASE(19) SAGA_VMCNT_CASE(20) SAGA_VMCNT_CASE(21) SAGA_VMCNT_CASE(22) SAGA_VMCNT_CASE(23) SAGA_VMCNT_CASE(24)
+        SAGA_VMCNT_CASE(25) SAGA_VMCNT_CASE(26) SAGA_VMCNT_CASE(27) SAGA_VMCNT_CASE(28) SAGA_VMCNT_CASE(29) SAGA_VMCNT_CASE(30)
+    default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    }
+#undef SAGA_VMCNT_CASE
+}
+
+// Epilogue of conv_rows64_wide: a wavefront's 64 pixels x 64 channels.  alpha / beta, the folded batch norm
+// (MODE 1, table at bnp), rounding to fp16 - and the stores go out as whole pixels: the accumulator layout gives a
+// lane 16-byte pieces of 32 different pixels, i.e. 32 cache lines touched per store instruction; the pieces are
+// exchanged through LDS (stg: this wavefront's kilobyte q at stg + 4096 * q, rows of 128 bytes with the 16-byte
+// chunks XOR-swizzled by the row) so that a store instruction writes 8 whole pixels.  soff[it]: byte offset in the
+// output of chunk lane%8 of pixel 8*it + lane/8 of the wavefront, or out of range.
+template <int MODE>
+__device__ __forceinline__ void rows64_wide_epilogue(const GatherArgs &g, float16_t (&acc)[2][2], const float *bnp, char *stg,
+                                                     int lane, const bool (&okr)[2], const int64_t (&pix)[2],
+                                                     const unsigned (&soff)[8])
+{
+    typedef unsigned u4 __attribute__((ext_vector_type(4)));
+    const int hi = lane >> 5;
+#pragma unroll
+    for(int i = 0; i < 2; i++)
+#pragma unroll
+        for(int j = 0; j < 2; j++) {
+            float f[16];
+#pragma unroll
+            for(int v = 0; v < 16; v++)
+                f[v] = g.alpha * acc[i][j][v];
+            if(g.beta != 0.0f) {
+                float old[16];
+                load_row32(g.out + pix[i] * g.ldo, okr[i], j * 32, g.Ngemm, hi, old);
+#pragma unroll
+                for(int v = 0; v < 16; v++)
+                    f[v] += g.beta * old[v];
+            }
+            if constexpr(MODE == 1) {
+#pragma unroll
+                for(int q = 0; q < 4; q++) {
+                    const int cl = j * 32 + 8 * q + 4 * hi;
+                    const float4_t sc = *(const float4_t *)(bnp + cl), sh = *(const float4_t *)(bnp + 64 + cl);
+#pragma unroll
+                    for(int e = 0; e < 4; e++) {
+                        float t = __builtin_fmaf(f[4 * q + e], sc[e], sh[e]);
+                        if(g.bn_flags & SAGA_BN_RELU)
+                            t = (t != t) ? t : fmaxf(t, 0.0f);
+                        f[4 * q + e] = t;
+                    }
+                }
+            }
+            const int row = i * 32 + (lane & 31);
+            char *srow = stg + (row >> 3) * 4096 + (row & 7) * 128;
+#pragma unroll
+            for(int q = 0; q < 2; q++) {
+                const unsigned x0 = pack2(f[8 * q + 0], f[8 * q + 1]), x1 = pack2(f[8 * q + 2], f[8 * q + 3]);
+                const unsigned y0 = pack2(f[8 * q + 4], f[8 * q + 5]), y1 = pack2(f[8 * q + 6], f[8 * q + 7]);
+                const auto s0_ = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+                const auto s1_ = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+                const u4 o = {s0_[0], s1_[0], s0_[1], s1_[1]};
+                const int chunk = 4 * j + 2 * q + hi;
+                *(u4 *)(srow + ((chunk ^ (row & 7)) << 4)) = o;
+            }
+        }
+    // LDS operations of one wavefront complete in order: its reads below see its writes above
+    const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc((void *)g.out, 0, g.out_bytes, 0x00020000);
+    const int r8 = lane >> 3, chunk = lane & 7;
+#pragma unroll
+    for(int it = 0; it < 8; it++) {
+        const u4 o = *(const u4 *)(stg + it * 4096 + r8 * 128 + ((chunk ^ r8) << 4));
+        const unsigned off = soff[it]; // (a local: see the loads)
+        __builtin_amdgcn_raw_buffer_store_b128(o, ro, off, 0, 0);
+    }
+}
+
+// the loads of one tile's rows (conv_rows64_wide)
+struct Rows64Req {
+    const char *img; // the tile's image
+    unsigned base;   // byte offset of the tile's first input row inside it (may be negative: rows above the image)
+    char *dst;       // this wavefront's first kilobyte of the tile's LDS buffer
+};
+
+// The same convolution with one wavefront per SIMD: four wavefronts, each with 64 pixels x ALL 64 output channels
+// and the whole filter in registers (288 of the 512 a lone wavefront may use).  In conv_rows64 every matrix
+// instruction needs a 16-byte LDS read of its own, which is exactly what a CU's LDS delivers while the matrix units
+// run flat out - two pipelines that would both have to be 100 % busy; here one pixel operand feeds two
+// instructions.  No other wavefront fills a SIMD's gaps any more, so the matrix phase is scheduled by hand (LDS
+// reads one tap ahead, pinned between the matrix instructions: it then runs at the matrix unit's rate) and the
+// rest of a tile's work is kept short:
+// - the byte offsets of a lane's row loads are computed once (a tile's position is one scalar added to them, and
+//   the rows above and below an image fall outside a buffer that covers just that image);
+// - the rows go through THREE LDS buffers; the loads of the tile after the next are issued one at a time between
+//   the matrix instructions, and the wait in front of a tile's barrier leaves them and the previous tile's stores
+//   in flight;
+// - the filter reaches the registers through LDS (fetched straight from memory a lane's fragments are 1152 bytes
+//   from its neighbour's, 64 cache lines per load instruction, times four wavefronts: 10 us before the first tile);
+// - the outputs are exchanged through LDS so that a store instruction writes whole pixels (rows64_wide_epilogue).
+template <int MODE, bool FLIP> __global__ void __launch_bounds__(256, 1) conv_rows64_wide(GatherArgs g, Rows64Args t)
+{
+    float *const stats = MODE == 2 ? g.stats : nullptr;
+    g.stats = nullptr;
+    if constexpr(MODE != 1)
+        g.bn_s = nullptr;
+    else
+        g.bn_flags &= SAGA_BN_RELU;
+    if constexpr(MODE != 0)
+        g.beta = 0.0f;
+    float run_s = 0.0f, run_q = 0.0f;
+    constexpr int TM = 2, TN = 2, NLD_MAX = 13, SLOT = 144, NW = 4;
+    constexpr unsigned OOB = 0x7fffff00u;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int hi = lane >> 5;
+
+    // LDS chunk L = (q * 4 + wave) * 64 + lane of a tile's copy: pixel slot L / 9 (row r, column p of the padded
+    // rows), chunk L % 9 of the slot (the ninth is padding): channels 8*(L%9).. of the pixel p - 1 of row r of the
+    // tile's TR + 2 input rows, as a byte offset from the tile's first input row (which may lie above the image).
+    // Every wavefront issues the same nld loads per tile (a buffer is a whole number of 4 KB rounds).
+    const int nld = t.buf_bytes >> 12; // NLD_MAX - 1 or NLD_MAX (the host's condition)
+    unsigned roff[NLD_MAX];
+    {
+        // (from one load to the next L grows by 256 = 28 * 9 + 4: no division per load)
+        const int L0 = wave * 64 + lane;
+        int slot = L0 / 9, kpos = L0 - slot * 9;
+        int r = slot / t.slots_row, pcol = slot - r * t.slots_row;
+#pragma unroll
+        for(int q = 0; q < NLD_MAX; q++) {
+            const int ix = pcol - 1;
+            const bool ok = slot * 9 + kpos < t.chunks_tile && kpos < 8 && ix >= 0 && ix < t.W;
+            roff[q] = ok ? (unsigned)(((r * t.W + ix) * g.lda + kpos * 8) * 2) : OOB;
+            kpos += 4;
+            const int step = kpos >= 9 ? 29 : 28;
+            kpos -= kpos >= 9 ? 9 : 0;
+            slot += step;
+            pcol += step;
+#pragma unroll
+            for(int w = 0; w < 3; w++) { // (slots_row >= 10: at most three rows further)
+                const bool wrap = pcol >= t.slots_row;
+                pcol -= wrap ? t.slots_row : 0;
+                r += wrap ? 1 : 0;
+            }
+        }
+    }
+    const unsigned img_bytes = (unsigned)(t.H * t.W * g.lda * 2);
+    const int row_bytes = t.W * g.lda * 2;
+    // a tile's loads: rows outside the image are outside the buffer that covers just the image (a negative offset
+    // is a huge unsigned one) and read as zeros
+    // (a tile beyond the last one: every offset out of range - the loads are issued all the same, so that the count
+    // of outstanding memory operations does not depend on it, and write zeros into a buffer that nobody reads)
+    auto req_setup = [&](int tile, int buffer) {
+        Rows64Req r;
+        const bool real = tile < t.ntiles;
+        const int tl = real ? tile : 0;
+        const int n = tl / t.tpi;
+        const int oy0 = (tl - n * t.tpi) * t.TR;
+        r.img = (const char *)g.a + (int64_t)n * img_bytes;
+        r.base = real ? (unsigned)((oy0 - 1) * row_bytes) : OOB;
+        r.dst = smem + buffer * t.buf_bytes + wave * 1024;
+        return r;
+    };
+    auto req_piece = [&](const Rows64Req &r, int q) {
+        const __amdgpu_buffer_rsrc_t ri = __builtin_amdgcn_make_buffer_rsrc((void *)r.img, 0, img_bytes, 0x00020000);
+        // (the offset goes through a local: a captured array element passed directly makes the host pass drop the kernel)
+        const unsigned off = roff[q];
+        if(q < NLD_MAX - 1 || nld == NLD_MAX)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ri, (lds_ptr_t)(r.dst + q * (NW * 1024)), 16, off + r.base, 0, 0, 0);
+    };
+    // this lane's two pixels (row blocks i of the wavefront's 64) inside a tile: byte offset of the top left tap
+    int abase[TM], prow[TM]; // prow: the pixel's output row inside the tile, or a row beyond every image
+#pragma unroll
+    for(int i = 0; i < TM; i++) {
+        const int pp0 = wave * 64 + i * 32 + (lane & 31);
+        const int pp = pp0 < t.npix ? pp0 : 0;
+        const int orow = pp / t.W;
+        abase[i] = (orow * t.slots_row + (pp - orow * t.W)) * SLOT + hi * 16;
+        prow[i] = pp0 < t.npix ? orow : 0x40000000;
+    }
+    // the stores' side: store instruction it writes chunk lane%8 of pixel 8*it + lane/8 of the wavefront's 64
+    int srow[8];       // that pixel's output row inside the tile, or a row beyond every image
+    unsigned sconst[8]; // its byte offset from the tile's first output pixel
+#pragma unroll
+    for(int it = 0; it < 8; it++) {
+        const int pp0 = wave * 64 + it * 8 + (lane >> 3);
+        const bool ok = pp0 < t.npix && (lane & 7) * 8 < g.Ngemm;
+        srow[it] = ok ? pp0 / t.W : 0x40000000;
+        sconst[it] = (unsigned)((pp0 * g.ldo + (lane & 7) * 8) * 2);
+    }
+    char *epi = smem + t.epi_off;
+    const int G = gridDim.x;
+    int tile = xcd_remap(blockIdx.x, G);
+    const int first_tile = tile;
+    {
+        const Rows64Req r0 = req_setup(tile, 0);
+#pragma unroll
+        for(int q = 0; q < NLD_MAX; q++)
+            req_piece(r0, q);
+    }
+    // The filter, [channel][tap][64] in memory.  A lane's fragments lie 1152 bytes from its neighbour's, so loading
+    // them straight into registers touches 64 cache lines per instruction (and four wavefronts do it): the block
+    // copies the filter through LDS instead - whole kilobytes per load instruction, into the two buffers that are
+    // still free, as rows of 73 sixteen-byte chunks (72 + 1 of padding: a fragment read then hits 64 different
+    // banks) - and every wavefront picks its fragments there.  Channels beyond the filter's read as zeros.
+    {
+        const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void *)g.b, 0, g.b_bytes, 0x00020000);
+        char *stage = smem + t.buf_bytes + wave * 1024;
+#pragma unroll
+        for(int q = 0; q < 19; q++) { // 64 * 73 = 4672 chunks, 256 per round
+            const int L = (q * NW + wave) * 64 + lane;
+            const int row = L / 73, cpos = L - row * 73;
+            const unsigned off = (cpos < 72 && row < g.Ngemm && row < 64) ? (unsigned)((row * 576 + cpos * 8) * 2) : OOB;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(stage + q * (NW * 1024)), 16, off, 0, 0, 0);
+        }
+    }
+    if constexpr(MODE == 1) // the folded norm's table: the same for every tile
+        bnfold_table<64>(g, (float *)(epi + 32768), tid, 0);
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    // fragment (tap, kk, j) = halves 16*kk + 8*hi .. +8 of that tap of output channel 32*j + lane%32
+    half8_t fb[9][4][TN];
+#pragma unroll
+    for(int j = 0; j < TN; j++) {
+        const char *src = smem + t.buf_bytes + (j * 32 + (lane & 31)) * (73 * 16) + hi * 16;
+#pragma unroll
+        for(int tp = 0; tp < 9; tp++)
+#pragma unroll
+            for(int kk = 0; kk < 4; kk++)
+                fb[tp][kk][j] = *(const half8_t *)(src + (FLIP ? 8 - tp : tp) * 128 + kk * 32);
+    }
+    // (everybody has its fragments before the second tile's rows overwrite them)
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    const Rows64Req r1 = req_setup(tile + G, 1);
+#pragma unroll
+    for(int q = 0; q < NLD_MAX; q++)
+        req_piece(r1, q);
+    // (the first tile's rows arrived with the filter)
+    constexpr int NST = TM * TN * 2; // the epilogue's stores per tile (always all of them: BUFST)
+    int b = 0;      // buffer of the current tile; the next tile's is b + 1, the one after goes to b + 2 (mod 3)
+    int behind = 0; // this wavefront's memory operations issued after the next tile's loads and before this tile's
+    for(; tile < t.ntiles; tile += G) {
+        const char *buf = smem + b * t.buf_bytes;
+        // the rows of the tile after the next go out between this tile's multiplications, into the buffer that the
+        // previous tile has left (every wavefront has passed that tile's barrier)
+        const Rows64Req rq = req_setup(tile + 2 * G, b >= 1 ? b - 1 : 2);
+        float16_t acc[TM][TN];
+#pragma unroll
+        for(int i = 0; i < TM; i++)
+#pragma unroll
+            for(int j = 0; j < TN; j++)
+#pragma unroll
+                for(int v = 0; v < 16; v++)
+                    acc[i][j][v] = 0.0f;
+        // one tap ahead: the reads of tap + 1 go out between the multiplications of tap, two per four matrix
+        // instructions (the scheduling barriers pin LDS reads, loads and matrix instructions, other instructions
+        // may move: left to itself the compiler issues each read right in front of its first use and waits for it)
+        half8_t fa[2][4][TM];
+#pragma unroll
+        for(int kk = 0; kk < 4; kk++)
+#pragma unroll
+            for(int i = 0; i < TM; i++)
+                fa[0][kk][i] = *(const half8_t *)(buf + abase[i] + kk * 32);
+        __builtin_amdgcn_sched_barrier(0x6);
+#pragma unroll
+        for(int tp = 0; tp < 9; tp++) {
+            const int tapoff = tp + 1 < 9 ? (((tp + 1) / 3) * t.slots_row + (tp + 1) % 3) * SLOT : 0;
+#pragma unroll
+            for(int kk = 0; kk < 4; kk++) {
+                if(tp + 1 < 9) {
+#pragma unroll
+                    for(int i = 0; i < TM; i++)
+                        fa[(tp + 1) & 1][kk][i] = *(const half8_t *)(buf + abase[i] + tapoff + kk * 32);
+                }
+                __builtin_amdgcn_sched_barrier(0x6);
+#pragma unroll
+                for(int i = 0; i < TM; i++)
+#pragma unroll
+                    for(int j = 0; j < TN; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[tp][kk][j], fa[tp & 1][kk][i], acc[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0x6);
+                // (a load every second or third group of four)
+#pragma unroll
+                for(int q = 0; q < NLD_MAX; q++)
+                    if((q * 36) / NLD_MAX == tp * 4 + kk) {
+                        req_piece(rq, q);
+                        __builtin_amdgcn_sched_barrier(0x6);
+                    }
+            }
+        }
+        // The NEXT tile's rows must have arrived before the barrier that lets everybody read them.  Behind them this
+        // wavefront has issued the previous tile's stores and this tile's loads: those may stay in flight.
+        wait_vmcnt(behind + nld);
+        asm volatile("s_barrier" ::: "memory");
+        behind = NST;
+        const int n = tile / t.tpi;
+        const int oy0 = (tile - n * t.tpi) * t.TR;
+        const int64_t pix0 = ((int64_t)n * t.H + oy0) * t.W;
+        bool okr[TM];
+        int64_t pix[TM];
+#pragma unroll
+        for(int i = 0; i < TM; i++) {
+            okr[i] = oy0 + prow[i] < t.H;
+            pix[i] = pix0 + (okr[i] ? wave * 64 + i * 32 + (lane & 31) : 0);
+        }
+        unsigned soff[8];
+        const unsigned tile_off = (unsigned)(pix0 * g.ldo * 2); // (the output's bytes fit 31 bits: the host's condition)
+#pragma unroll
+        for(int it = 0; it < 8; it++)
+            soff[it] = oy0 + srow[it] < t.H ? sconst[it] + tile_off : OOB;
+        // (staged in this tile's buffer: every wavefront is past the barrier, so nobody reads it any more, and
+        // the kilobytes a wavefront stages in are the ones that only its own later loads write)
+        rows64_wide_epilogue<MODE>(g, acc, (const float *)(epi + 32768), smem + b * t.buf_bytes + wave * 1024, lane, okr, pix, soff);
+        if constexpr(MODE == 2) {
+            float s0, q0;
+            stats_lane_totals<TM, TN, true>(g.alpha, acc, okr, lane, s0, q0);
+            run_s += s0;
+            run_q += q0;
+        }
+        b = b == 2 ? 0 : b + 1;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // (loads into this block's LDS may still be in flight)
+    if constexpr(MODE == 2) {
+        g.stats = stats;
+        __syncthreads();
+        stats_block_write<TN, 4, 1, 64>(g, epi + 32768, tid, lane, wave, 0, 0, first_tile, run_s, run_q);
+    }
+}
+
 // Launches conv_rows64 if the geometry is its: returns false (and launches nothing) otherwise.  g: as for
 // launch_gather, with a = the NHWC input (pixel pitch lda), b = [Ngemm][9][64].
 template <bool FLIP> static bool launch_rows64(GatherArgs &g, const CLInfo &lout, hipStream_t st, size_t stats_floats, int *rc)
@@ -2406,13 +2744,57 @@ template <bool FLIP> static bool launch_rows64(GatherArgs &g, const CLInfo &lout
     t.slots_row = t.W + 2;
     t.chunks_tile = (t.TR + 2) * t.slots_row * 9;
     t.buf_bytes = (t.chunks_tile * 16 + 1023) & ~1023;
+    const int buf_narrow = t.buf_bytes;
     const int epi_back = wgm == 2 ? 16384 : 32768; // gather_epilogue's scratch sits this far behind its base
+    const bool vec_ok = (lout.pitch & 7) == 0 && aligned16(g.out) && ((lout.rows - 1) * lout.pitch + g.Ngemm) * 2 < 0x7fffff00ll &&
+                        (g.lda & 7) == 0 && aligned16(g.a);
+    // one wavefront per SIMD with the whole filter in registers, where a block may have the LDS for three buffers
+    static const bool wide_on = !(getenv("SAGA_HIP_ROWS64_WIDE") && atoi(getenv("SAGA_HIP_ROWS64_WIDE")) == 0);
+    static const int lds_max = [] {
+        int dev = 0, v = 0;
+        if(hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess)
+            return 64 * 1024;
+        return std::min(v, 160 * 1024);
+    }();
+    t.buf_bytes = (t.chunks_tile * 16 + 4095) & ~4095; // (a whole number of rounds of the four wavefronts' loads)
+    if(wide_on && wgm == 4 && vec_ok && t.chunks_tile <= 13 * 256 && t.chunks_tile > 11 * 256 && (int64_t)t.H * t.W * g.lda * 2 < 0x7fff0000ll) {
+        const int epi_at = std::max(3 * t.buf_bytes, epi_back);
+        t.epi_off = epi_at - epi_back;
+        const int lds = epi_at + 4096;
+        const int blocks = std::min(t.ntiles, num_cus());
+        if(lds <= lds_max && !(g.stats && (size_t)blocks * g.Ngemm * 2 > stats_floats)) {
+            static bool once = false;
+            if(!once) {
+                for(const void *k : {(const void *)conv_rows64_wide<0, FLIP>, (const void *)conv_rows64_wide<1, FLIP>,
+                                     (const void *)conv_rows64_wide<2, FLIP>}) {
+                    const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds_max);
+                    if(e != hipSuccess) {
+                        *rc = (int)e;
+                        return true;
+                    }
+                }
+                once = true;
+            }
+            g.classes = 1;
+            g.no_stage = 1;
+            g.nblk_n = 1;
+            g.out_bytes = (unsigned)(((lout.rows - 1) * lout.pitch + g.Ngemm) * 2);
+            g.stats_rows = blocks;
+            if(g.bn_s)
+                conv_rows64_wide<1, FLIP><<<blocks, 256, lds, st>>>(g, t);
+            else if(g.stats)
+                conv_rows64_wide<2, FLIP><<<blocks, 256, lds, st>>>(g, t);
+            else
+                conv_rows64_wide<0, FLIP><<<blocks, 256, lds, st>>>(g, t);
+            *rc = 0;
+            return true;
+        }
+    }
+    t.buf_bytes = buf_narrow;
     const int epi_at = std::max(2 * t.buf_bytes, epi_back);
     t.epi_off = epi_at - epi_back;
     const int lds = epi_at + 4096;
     const int blocks = std::min(t.ntiles, (wgm == 2 ? 2 : 1) * num_cus());
-    const bool vec_ok = (lout.pitch & 7) == 0 && aligned16(g.out) && ((lout.rows - 1) * lout.pitch + g.Ngemm) * 2 < 0x7fffff00ll &&
-                        (g.lda & 7) == 0 && aligned16(g.a);
     if(!vec_ok || t.chunks_tile > 10 * (wgm == 2 ? 256 : 512) || lds > (wgm == 2 ? 76 : 150) * 1024 || (g.stats && (size_t)blocks * g.Ngemm * 2 > stats_floats))
         return false;
     static bool once = false;
