@@ -1561,6 +1561,20 @@ __device__ __forceinline__ half8_t tr_read8(const char *lo, const char *hi)
     return __builtin_bit_cast(half8_t, v);
 }
 
+// The same two reads as instructions of our own: addr = LDS byte address, LO / HI = immediate offsets.  The
+// compiler does not know that they read LDS, which is the point - in front of a ds_read that it has emitted itself
+// it waits for EVERY outstanding buffer_load ... lds whose target it cannot tell apart from the read's address (a
+// stage picked at run time), the slice just requested included, and the loads of the pipelined kernel below are
+// then never in flight while it multiplies.  The caller waits for the data (s_waitcnt lgkmcnt) before it uses it.
+template <int LO, int HI> __device__ __forceinline__ half8_t tr_read8_raw(unsigned addr)
+{
+    short4_t a, b;
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(a) : "v"(addr), "n"(LO) : "memory");
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(b) : "v"(addr), "n"(HI) : "memory");
+    const short8_t v = __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(half8_t, v);
+}
+
 template <int BM, int BN, int STAGES, int NW>
 __global__ void __launch_bounds__(64 * NW) conv_bwd_filter_dma(FilterArgs g, unsigned x_bytes, unsigned dy_bytes)
 {
@@ -1680,6 +1694,7 @@ __global__ void __launch_bounds__(64 * NW) conv_bwd_filter_dma(FilterArgs g, uns
         fob[j] = BK * ROWA + fp * ROWB + (((c >> 3) ^ fswb) << 4) + (c & 7) * 2;
     }
 
+    const unsigned lds0 = (unsigned)(uintptr_t)(lds_ptr_t)smem;
     const int KT = (m_end - m_begin + BK - 1) / BK;
 #pragma unroll
     for(int st = 0; st < STAGES - 1; st++)
@@ -1693,21 +1708,42 @@ __global__ void __launch_bounds__(64 * NW) conv_bwd_filter_dma(FilterArgs g, uns
             asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
         if(kt + STAGES - 1 < KT)
             issue((kt + STAGES - 1) % STAGES);
-        const char *sbase = smem + (kt % STAGES) * STAGE_BYTES;
+        // the slice's fragments: all reads go out, then each 16-pixel step waits for its own (tr_read8_raw)
+        const unsigned sbase = lds0 + (kt % STAGES) * STAGE_BYTES;
+        static_assert(BK == 32, "two 16-pixel steps per slice");
+        half8_t fa[2][TM], fb[2][TN];
 #pragma unroll
-        for(int kk = 0; kk < BK; kk += 16) {
-            half8_t fa[TM], fb[TN];
+        for(int i = 0; i < TM; i++) {
+            fa[0][i] = tr_read8_raw<0, 4 * ROWA>(sbase + foa[i]);
+        }
+#pragma unroll
+        for(int j = 0; j < TN; j++)
+            fb[0][j] = tr_read8_raw<0, 4 * ROWB>(sbase + fob[j]);
+#pragma unroll
+        for(int i = 0; i < TM; i++)
+            fa[1][i] = tr_read8_raw<16 * ROWA, 20 * ROWA>(sbase + foa[i]);
+#pragma unroll
+        for(int j = 0; j < TN; j++)
+            fb[1][j] = tr_read8_raw<16 * ROWB, 20 * ROWB>(sbase + fob[j]);
+#pragma unroll
+        for(int kk = 0; kk < 2; kk++) {
+            if(kk == 0)
+                asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(2 * (TM + TN)) : "memory");
+            else
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            // (the multiplications must stay behind the wait: their operands pass through it)
 #pragma unroll
             for(int i = 0; i < TM; i++)
-                fa[i] = tr_read8(sbase + foa[i] + kk * ROWA, sbase + foa[i] + (kk + 4) * ROWA);
+                asm volatile("" : "+v"(fa[kk][i]));
 #pragma unroll
             for(int j = 0; j < TN; j++)
-                fb[j] = tr_read8(sbase + fob[j] + kk * ROWB, sbase + fob[j] + (kk + 4) * ROWB);
+                asm volatile("" : "+v"(fb[kk][j]));
 #pragma unroll
             for(int i = 0; i < TM; i++)
 #pragma unroll
                 for(int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kk][i], fb[kk][j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0); // (or the first step's multiplications sink below the second wait)
         }
     }
 
@@ -1813,7 +1849,8 @@ static FilterPlan plan_filter(const ConvGeom &g, bool big_ok = true, bool thin =
     // SAGA_HIP_FILTER_TILE=128 keeps the small tiles everywhere, =256 takes the large one wherever it fits
     static const char *env = getenv("SAGA_HIP_FILTER_TILE");
     static const int forced = env ? atoi(env) : 0;
-    int target = 768; // three blocks fit a CU: 768 blocks are one full round of the chip (measured best of 512..2048)
+    static const int target_env = getenv("SAGA_HIP_FILTER_TARGET") ? atoi(getenv("SAGA_HIP_FILTER_TARGET")) : 0;
+    int target = 512; // two blocks per CU (three fit): measured best of 256 / 512 / 640 / 768 / 1024
     // 256x256 on sixteen wavefronts, one block per CU: half the LDS fill traffic per flop.  Measured
     // 25-35 % faster where the reduction per tile is long enough to pay for the smaller grid (3x3
     // filters, or 1x1 with >= 1024 input and >= 512 output channels), slower on the other 1x1 layers.
@@ -1832,6 +1869,8 @@ static FilterPlan plan_filter(const ConvGeom &g, bool big_ok = true, bool thin =
         p.bn = 256; // the stem: all 7 x 32 virtual channels in one tile, so dy (the large operand) is read once
         target = 1024;
     }
+    if(target_env && p.bn == 256)
+        target = target_env;
     p.tiles_k = (g.K + p.bm - 1) / p.bm;
     p.tiles_c = (RSC + p.bn - 1) / p.bn;
     const int tiles = p.tiles_k * p.tiles_c;
