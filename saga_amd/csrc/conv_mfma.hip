@@ -1637,21 +1637,24 @@ __global__ void __launch_bounds__(64 * NW) conv_bwd_filter_dma(FilterArgs g, uns
     }
     int ms = m_begin; // first pixel of the next slice to be issued
 
-    auto issue = [&](int stage) {
+    // one slice = RA + RB load instructions ("pieces"): piece p < RA is round p of the dy rows, the others are rounds
+    // of the x rows; after the last piece of a slice the cursor moves on
+    auto issue_piece = [&](int stage, int p) {
         char *sa = smem + stage * STAGE_BYTES;
         char *sb = sa + BK * ROWA;
-#pragma unroll
-        for(int j = 0; j < RA; j++) {
+        if(p < RA) {
+            const int j = p;
             const int m = ms + pa0 + j * NW * RPA;
             const unsigned off = (ka_ok && m < m_end) ? (unsigned)((m * g.ldy + ka) * 2) : OOB;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(ry, (lds_ptr_t)(sa + (wave + NW * j) * 1024), 16, off, 0, 0, 0);
-        }
-#pragma unroll
-        for(int j = 0; j < RB; j++) {
+        } else {
+            const int j = p - RA;
             const int m = ms + pb0 + j * NW * RPB;
-            const int iy = by_[j] * g.stride + offy, ix = bx_[j] * g.stride + offx;
+            // (through locals: a captured array element passed directly makes the host pass drop the kernel)
+            const int byj = by_[j], bxj = bx_[j], bnj = bn_[j];
+            const int iy = byj * g.stride + offy, ix = bxj * g.stride + offx;
             const bool ok = cb_ok && m < m_end && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
-            const unsigned off = ok ? (unsigned)((((bn_[j] * g.H + iy) * g.W + ix) * g.ldx + cc) * 2) : OOB;
+            const unsigned off = ok ? (unsigned)((((bnj * g.H + iy) * g.W + ix) * g.ldx + cc) * 2) : OOB;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(sb + (wave + NW * j) * 1024), 16, off, 0, 0, 0);
             bx_[j] += BK;
             while(bx_[j] >= g.Q) {
@@ -1663,7 +1666,13 @@ __global__ void __launch_bounds__(64 * NW) conv_bwd_filter_dma(FilterArgs g, uns
                 bn_[j]++;
             }
         }
-        ms += BK;
+        if(p == RA + RB - 1)
+            ms += BK;
+    };
+    auto issue = [&](int stage) {
+#pragma unroll
+        for(int p = 0; p < RA + RB; p++)
+            issue_piece(stage, p);
     };
 
     float16_t acc[TM][TN];
@@ -1706,8 +1715,8 @@ __global__ void __launch_bounds__(64 * NW) conv_bwd_filter_dma(FilterArgs g, uns
             asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((RA + RB) * (STAGES - 2)) : "memory");
         else
             asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-        if(kt + STAGES - 1 < KT)
-            issue((kt + STAGES - 1) % STAGES);
+        const bool more = kt + STAGES - 1 < KT;
+        const int nst = (kt + STAGES - 1) % STAGES;
         // the slice's fragments: all reads go out, then each 16-pixel step waits for its own (tr_read8_raw)
         const unsigned sbase = lds0 + (kt % STAGES) * STAGE_BYTES;
         static_assert(BK == 32, "two 16-pixel steps per slice");
@@ -1725,26 +1734,37 @@ __global__ void __launch_bounds__(64 * NW) conv_bwd_filter_dma(FilterArgs g, uns
 #pragma unroll
         for(int j = 0; j < TN; j++)
             fb[1][j] = tr_read8_raw<16 * ROWB, 20 * ROWB>(sbase + fob[j]);
+        // The loads of the slice STAGES - 1 ahead go out between the multiplications: the address unit takes a
+        // kilobyte in 16 cycles, and right behind the barrier every wavefront of the block would stand in line for
+        // it with nothing running on the matrix units (0.4 us of a 1.3 us iteration on sixteen wavefronts).
+        constexpr int NP = RA + RB, NQ = 2 * TM * TN;
 #pragma unroll
-        for(int kk = 0; kk < 2; kk++) {
-            if(kk == 0)
-                asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(2 * (TM + TN)) : "memory");
-            else
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            // (the multiplications must stay behind the wait: their operands pass through it)
+        for(int q = 0; q < NQ; q++) {
+            const int kk = q / (TM * TN), i = (q / TN) % TM, j = q % TN;
+            if(q % (TM * TN) == 0) {
+                if(kk == 0)
+                    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(2 * (TM + TN)) : "memory");
+                else
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                // (the multiplications must stay behind the wait: their operands pass through it)
 #pragma unroll
-            for(int i = 0; i < TM; i++)
-                asm volatile("" : "+v"(fa[kk][i]));
+                for(int ii = 0; ii < TM; ii++)
+                    asm volatile("" : "+v"(fa[kk][ii]));
 #pragma unroll
-            for(int j = 0; j < TN; j++)
-                asm volatile("" : "+v"(fb[kk][j]));
+                for(int jj = 0; jj < TN; jj++)
+                    asm volatile("" : "+v"(fb[kk][jj]));
+            }
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kk][i], fb[kk][j], acc[i][j], 0, 0, 0);
 #pragma unroll
-            for(int i = 0; i < TM; i++)
-#pragma unroll
-                for(int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kk][i], fb[kk][j], acc[i][j], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0); // (or the first step's multiplications sink below the second wait)
+            for(int p = 0; p < NP; p++)
+                if(q == ((p + 1) * NQ) / (NP + 1)) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    if(more)
+                        issue_piece(nst, p);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
         }
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     float *out = g.partial + (int64_t)split * g.K * g.RSC;
@@ -1849,7 +1869,6 @@ static FilterPlan plan_filter(const ConvGeom &g, bool big_ok = true, bool thin =
     // SAGA_HIP_FILTER_TILE=128 keeps the small tiles everywhere, =256 takes the large one wherever it fits
     static const char *env = getenv("SAGA_HIP_FILTER_TILE");
     static const int forced = env ? atoi(env) : 0;
-    static const int target_env = getenv("SAGA_HIP_FILTER_TARGET") ? atoi(getenv("SAGA_HIP_FILTER_TARGET")) : 0;
     int target = 512; // two blocks per CU (three fit): measured best of 256 / 512 / 640 / 768 / 1024
     // 256x256 on sixteen wavefronts, one block per CU: half the LDS fill traffic per flop.  Measured
     // 25-35 % faster where the reduction per tile is long enough to pay for the smaller grid (3x3
@@ -1869,8 +1888,6 @@ static FilterPlan plan_filter(const ConvGeom &g, bool big_ok = true, bool thin =
         p.bn = 256; // the stem: all 7 x 32 virtual channels in one tile, so dy (the large operand) is read once
         target = 1024;
     }
-    if(target_env && p.bn == 256)
-        target = target_env;
     p.tiles_k = (g.K + p.bm - 1) / p.bm;
     p.tiles_c = (RSC + p.bn - 1) / p.bn;
     const int tiles = p.tiles_k * p.tiles_c;
