@@ -2775,6 +2775,219 @@ template <int MODE, bool FLIP> __global__ void __launch_bounds__(256, 1) conv_ro
     }
 }
 
+// ---------------------------------------------------------------- backward filter of those layers, whole image rows in LDS
+//
+// dw[k][tap][c] = sum over pixels of dy[p][k] * x[p + tap][c] for the 3x3, stride-1 layers with 64 input channels and
+// at most 64 output channels.  conv_bwd_filter_dma treats the nine taps as nine column blocks of a GEMM: x goes
+// from L2 to LDS nine times, dy three times (three column tiles), and the partial tiles of a thousand blocks are
+// 50 MB to write and read back.  Here, as in conv_rows64_wide, a persistent block of four wavefronts (one per SIMD)
+// walks tiles of TR whole image rows: the TR + 2 rows of x (144-byte pixel slots with zero borders, the same copy
+// as conv_rows64_wide's) and the TR rows of dy (128-byte pixel rows, 16-byte granules XOR-swizzled as in
+// conv_bwd_filter_dma) are copied ONCE per tile, the x operand of tap (dr, ds) is the same copy read (dr, ds) slots
+// further on, and the whole 64 x 9 x 64 result stays in the block's registers for the launch: wavefront (mt, nt)
+// holds output channels 32*mt.. x input channels 32*nt.. of all nine taps (144 accumulator registers), and one
+// partial per BLOCK goes to the second pass (filter_reduce_v4: 256 partials instead of 1000).
+// The reduction index of an MFMA is the pixel: operands come from the transposing LDS read (tr_read8_raw), 16
+// pixels per step, one dy operand and nine x operands for nine instructions.  One wavefront per SIMD: the reads run
+// three operands ahead of the multiplications that use them, in program order (they are instructions of our own,
+// and the waits in front of the multiplications count them), and a tile's loads go out between the multiplications
+// of the tile before.  NSTEPS = pixels of a tile / 16 (the host's condition: a whole number).
+struct FilterRowsArgs {
+    const half_t *x, *dy;
+    float *partial;      // [block][K][9][64]
+    int ldx, ldy, H, W, K;
+    int TR, tpi, ntiles; // output rows per tile, tiles per image, tiles
+    int slots_row;       // W + 2 pixel slots per LDS row of x
+    int xchunks;         // (TR + 2) * slots_row * 9: 16-byte chunks of a tile's x copy
+    int x_bytes, y_bytes; // one LDS buffer of each (whole rounds of the four wavefronts' loads)
+};
+
+template <int NSTEPS> __global__ void __launch_bounds__(256, 1) conv_bwd_filter_rows64(FilterRowsArgs t)
+{
+    constexpr int NW = 4, SLOT = 144, NLX = 13, NLY = (NSTEPS * 16 * 8 + 255) / 256;
+    constexpr unsigned OOB = 0x7fffff00u;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int mt = wave >> 1, nt = wave & 1;
+    const int npix = NSTEPS * 16;
+
+    // x rows: as in conv_rows64_wide (chunk L = (q * 4 + wave) * 64 + lane: slot L / 9, chunk L % 9 of it)
+    const int nlx = t.x_bytes >> 12;
+    unsigned roffx[NLX];
+    {
+        const int L0 = wave * 64 + lane;
+        int slot = L0 / 9, kpos = L0 - slot * 9;
+        int r = slot / t.slots_row, pcol = slot - r * t.slots_row;
+#pragma unroll
+        for(int q = 0; q < NLX; q++) {
+            const int ix = pcol - 1;
+            const bool ok = slot * 9 + kpos < t.xchunks && kpos < 8 && ix >= 0 && ix < t.W;
+            roffx[q] = ok ? (unsigned)(((r * t.W + ix) * t.ldx + kpos * 8) * 2) : OOB;
+            kpos += 4;
+            const int step = kpos >= 9 ? 29 : 28;
+            kpos -= kpos >= 9 ? 9 : 0;
+            slot += step;
+            pcol += step;
+#pragma unroll
+            for(int w = 0; w < 3; w++) {
+                const bool wrap = pcol >= t.slots_row;
+                pcol -= wrap ? t.slots_row : 0;
+                r += wrap ? 1 : 0;
+            }
+        }
+    }
+    // dy rows: chunk L: pixel L / 8 of the tile, physical granule L % 8 = logical granule ^ 4 * bit 1 of the pixel
+    unsigned roffy[NLY];
+#pragma unroll
+    for(int q = 0; q < NLY; q++) {
+        const int L = (q * NW + wave) * 64 + lane;
+        const int pp = L >> 3, gran = (L & 7) ^ (((pp >> 1) & 1) << 2);
+        roffy[q] = (pp < npix && gran * 8 < t.K) ? (unsigned)((pp * t.ldy + gran * 8) * 2) : OOB;
+    }
+    const unsigned ximg = (unsigned)(t.H * t.W * t.ldx * 2), yimg = (unsigned)(t.H * t.W * t.ldy * 2);
+    char *const xbuf = smem, *const ybuf = smem + 2 * t.x_bytes;
+    // piece p of a tile's loads: the first NLX are x, the others dy.  A tile beyond the last one: every offset out
+    // of range (the loads are issued all the same and write zeros into a buffer that nobody reads)
+    auto req_piece = [&](int tile, int b, int p) {
+        const bool real = tile < t.ntiles;
+        const int tl = real ? tile : 0;
+        const int n = tl / t.tpi;
+        const int oy0 = (tl - n * t.tpi) * t.TR;
+        if(p < NLX) {
+            const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)((const char *)t.x + (int64_t)n * ximg), 0, ximg, 0x00020000);
+            const unsigned base = real ? (unsigned)((oy0 - 1) * t.W * t.ldx * 2) : OOB;
+            const unsigned off = roffx[p]; // (a local: a captured array element passed directly makes the host pass drop the kernel)
+            if(p < NLX - 1 || nlx == NLX)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(xbuf + b * t.x_bytes + (p * NW + wave) * 1024), 16, off + base, 0, 0, 0);
+        } else {
+            const int q = p - NLX;
+            const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc((void *)((const char *)t.dy + (int64_t)n * yimg), 0, yimg, 0x00020000);
+            const unsigned base = real ? (unsigned)(oy0 * t.W * t.ldy * 2) : OOB;
+            const unsigned off = roffy[q];
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ry, (lds_ptr_t)(ybuf + b * t.y_bytes + (q * NW + wave) * 1024), 16, off + base, 0, 0, 0);
+        }
+    };
+    // Operand addresses.  A transposing read hands lane i (channel i of 16, 4 pixels): the lane points at pixel fp
+    // (the read's second half: fp + 4) of the 16-pixel step and at 4 channels of its 32-channel tile.
+    const int fp = 8 * (lane >> 5) + ((lane & 15) >> 2);
+    const int fc = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    const unsigned lds0 = (unsigned)(uintptr_t)(lds_ptr_t)smem;
+    const int ca = mt * 32 + fc, cb = nt * 32 + fc;
+    // dy: pixel rows of 128 bytes (the swizzle term is the same for every step: steps are 16 pixels apart)
+    const unsigned ya = (unsigned)(fp * 128 + (((ca >> 3) ^ (((fp >> 1) & 1) << 2)) << 4) + (ca & 7) * 2);
+    // x: the slot of the lane's two pixels in step 0, and their columns (a step moves 16 pixels on, across row ends)
+    const unsigned xc = (unsigned)((cb >> 3) * 16 + (cb & 7) * 2);
+    const int r0lo = fp / t.W, c0lo = fp - r0lo * t.W, r0hi = (fp + 4) / t.W, c0hi = fp + 4 - r0hi * t.W;
+    unsigned tapoff[9];
+#pragma unroll
+    for(int tp = 0; tp < 9; tp++)
+        tapoff[tp] = (unsigned)(((tp / 3) * t.slots_row + tp % 3) * SLOT);
+
+    float16_t acc[9];
+#pragma unroll
+    for(int tp = 0; tp < 9; tp++)
+#pragma unroll
+        for(int v = 0; v < 16; v++)
+            acc[tp][v] = 0.0f;
+
+    const int G = gridDim.x;
+    int tile = xcd_remap(blockIdx.x, G);
+#pragma unroll
+    for(int p = 0; p < NLX + NLY; p++)
+        req_piece(tile, 0, p);
+    int b = 0;
+    for(; tile < t.ntiles; tile += G) {
+        // this tile's rows have arrived (everybody's: the barrier), and everybody is done with the other buffer
+        asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+        const unsigned xb = lds0 + b * t.x_bytes + xc, yb = lds0 + 2 * t.x_bytes + b * t.y_bytes + ya;
+        int rlo = r0lo, clo = c0lo, rhi = r0hi, chi = c0hi; // the step's pixels: row inside the tile, column
+        auto xaddr = [&](int r, int c) { return xb + (unsigned)((r * t.slots_row + c) * SLOT); };
+        auto next_step = [&]() {
+            clo += 16;
+            const bool wl = clo >= t.W;
+            clo -= wl ? t.W : 0;
+            rlo += wl ? 1 : 0;
+            chi += 16;
+            const bool wh = chi >= t.W;
+            chi -= wh ? t.W : 0;
+            rhi += wh ? 1 : 0;
+        };
+        auto read_x = [&](unsigned alo, unsigned ahi, int tp) {
+            short4_t lo, hi;
+            asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo) : "v"(alo + tapoff[tp]) : "memory");
+            asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(hi) : "v"(ahi + tapoff[tp]) : "memory");
+            const short8_t v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            return __builtin_bit_cast(half8_t, v);
+        };
+        // the pipeline of operand reads: item (step, -1) is the step's dy operand, (step, tp) its x operand of tap
+        // tp; three x operands ahead of the multiplication that uses them
+        half8_t fa[2], fb[2][9];
+        unsigned alo = xaddr(rlo, clo), ahi = xaddr(rhi, chi);
+        fa[0] = tr_read8_raw<0, 512>(yb);
+        fb[0][0] = read_x(alo, ahi, 0);
+        fb[0][1] = read_x(alo, ahi, 1);
+        fb[0][2] = read_x(alo, ahi, 2);
+#pragma unroll
+        for(int st = 0; st < NSTEPS; st++) {
+            const int cur = st & 1, nxt = cur ^ 1;
+            unsigned nlo = alo, nhi = ahi;
+#pragma unroll
+            for(int tp = 0; tp < 9; tp++) {
+                // issue: the x operand three taps on; at the end of a step the next step's dy operand and first x
+                // operands (after the last step: the first step's again, never used - the waits count them)
+                if(tp < 6) {
+                    fb[cur][tp + 3] = read_x(alo, ahi, tp + 3);
+                } else if(tp == 6) {
+                    if(st + 1 < NSTEPS) {
+                        next_step();
+                        nlo = xaddr(rlo, clo);
+                        nhi = xaddr(rhi, chi);
+                    }
+                    fa[nxt] = st + 1 < NSTEPS ? tr_read8_raw<0, 512>(yb + (st + 1) * 2048) : tr_read8_raw<0, 512>(yb);
+                } else if(tp == 7) {
+                    fb[nxt][0] = read_x(nlo, nhi, 0);
+                } else {
+                    fb[nxt][1] = read_x(nlo, nhi, 1);
+                    fb[nxt][2] = read_x(nlo, nhi, 2);
+                }
+                // wait for this multiplication's operands: three items (two instructions each) were issued
+                // behind them, four at the last tap
+                if(tp == 8)
+                    asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
+                else
+                    asm volatile("s_waitcnt lgkmcnt(6)" ::: "memory");
+                asm volatile("" : "+v"(fa[cur]), "+v"(fb[cur][tp]));
+                acc[tp] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[cur], fb[cur][tp], acc[tp], 0, 0, 0);
+                // the next tile's loads: two per step, four multiplications apart, while there are any
+                constexpr int NP = NLX + NLY;
+                static_assert(2 * NSTEPS >= NP, "a step issues two of the next tile's loads");
+                if((tp == 2 || tp == 6) && 2 * st + (tp == 6) < NP) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    req_piece(tile + G, b ^ 1, 2 * st + (tp == 6));
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            alo = nlo;
+            ahi = nhi;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // (the reads that nobody uses)
+        b ^= 1;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // (loads into this block's LDS may still be in flight)
+    // the block's partial: acc[tp][v] = element (k = 32*mt + 8*(v/4) + 4*(lane/32) + v%4, tap tp, c = 32*nt + lane%32)
+    float *out = t.partial + (int64_t)blockIdx.x * t.K * 576;
+    const int ecol = nt * 32 + (lane & 31), erow = mt * 32 + (lane >> 5) * 4;
+#pragma unroll
+    for(int tp = 0; tp < 9; tp++)
+#pragma unroll
+        for(int v = 0; v < 16; v++) {
+            const int k = erow + (v >> 2) * 8 + (v & 3);
+            if(k < t.K)
+                out[(int64_t)k * 576 + tp * 64 + ecol] = acc[tp][v];
+        }
+}
+
 // Launches conv_rows64 if the geometry is its: returns false (and launches nothing) otherwise.  g: as for
 // launch_gather, with a = the NHWC input (pixel pitch lda), b = [Ngemm][9][64].
 template <bool FLIP> static bool launch_rows64(GatherArgs &g, const CLInfo &lout, hipStream_t st, size_t stats_floats, int *rc)
@@ -3454,6 +3667,50 @@ int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, cons
     const size_t need = xpad + (size_t)p.splits * g.K * g.R * g.S * Cp * sizeof(float);
     if(!ws || ws_bytes < need || !aligned16(ws))
         return SAGA_HIP_EWORKSPACE;
+    // the 3x3, stride-1 layers with 64 input channels over large images: whole image rows in LDS
+    static const bool rows_on = !(getenv("SAGA_HIP_FILTER_ROWS64") && atoi(getenv("SAGA_HIP_FILTER_ROWS64")) == 0);
+    if(rows_on && pipelined && !pad && g.R == 3 && g.S == 3 && g.stride == 1 && g.pad == 1 && g.dil == 1 && g.C == 64 && g.K <= 64 &&
+       g.P == g.H && g.Q == g.W && g.W >= 16 && g.W <= 256 && (lx.pitch & 7) == 0 && aligned16(x->ptr)) {
+        FilterRowsArgs t;
+        int tr = std::min(256 / g.W, g.H);
+        while(tr > 1 && (tr * g.W) % 16)
+            tr--;
+        const int nsteps = tr * g.W / 16;
+        t.TR = tr;
+        t.tpi = (g.H + tr - 1) / tr;
+        const int64_t ntiles = (int64_t)g.N * t.tpi;
+        t.slots_row = g.W + 2;
+        t.xchunks = (tr + 2) * t.slots_row * 9;
+        t.x_bytes = (t.xchunks * 16 + 4095) & ~4095;
+        t.y_bytes = nsteps * 16 * 128;
+        const int blocks = num_cus();
+        const int lds = 2 * t.x_bytes + 2 * t.y_bytes;
+        int dev = 0, lds_max = 0;
+        if((tr * g.W) % 16 == 0 && (nsteps == 14 || nsteps == 16) && ntiles >= 2 * blocks && ntiles < 0x7fffffff &&
+           (t.x_bytes >> 12) >= 12 && (t.x_bytes >> 12) <= 13 && (t.y_bytes & 4095) == 0 &&
+           (int64_t)g.H * g.W * lx.pitch * 2 < 0x7fff0000ll && (int64_t)g.H * g.W * ldy.pitch * 2 < 0x7fff0000ll &&
+           (size_t)blocks * n * sizeof(float) <= ws_bytes && hipGetDevice(&dev) == hipSuccess &&
+           hipDeviceGetAttribute(&lds_max, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) == hipSuccess && lds <= lds_max) {
+            t.x = (const half_t *)x->ptr;
+            t.dy = (const half_t *)dy->ptr;
+            t.partial = (float *)ws;
+            t.ldx = (int)lx.pitch;
+            t.ldy = (int)ldy.pitch;
+            t.H = g.H;
+            t.W = g.W;
+            t.K = g.K;
+            t.ntiles = (int)ntiles;
+            auto kern = nsteps == 14 ? conv_bwd_filter_rows64<14> : conv_bwd_filter_rows64<16>;
+            const hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+            if(e != hipSuccess)
+                return (int)e;
+            kern<<<blocks, 256, lds, st>>>(t);
+            SAGA_CHECK_LAUNCH();
+            filter_reduce_v4<<<(unsigned)((n / 4 + 15) / 16), 256, 0, st>>>(t.partial, (half_t *)dw->ptr, n, blocks, alpha, beta);
+            SAGA_CHECK_LAUNCH();
+            return 0;
+        }
+    }
     FilterArgs a;
     a.x = (const half_t *)x->ptr;
     a.ldx = (int)lx.pitch;

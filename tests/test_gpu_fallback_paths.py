@@ -36,6 +36,8 @@ CASES = [
     ("SAGA_HIP_ROWS64_WGM", "2", ["tests/test_gpu_ops.py", "-k", "test_conv_fwd_bwd or folded_bn or bnstats"]),
     # the 3x3 64 -> 64 layers with two wavefronts per SIMD (half the filter each) instead of one with all of it
     ("SAGA_HIP_ROWS64_WIDE", "0", ["tests/test_gpu_ops.py", "-k", "test_conv_fwd_bwd or folded_bn or bnstats"]),
+    # backward filter of those layers through the generic kernel
+    ("SAGA_HIP_FILTER_ROWS64", "0", ["tests/test_gpu_ops.py", "-k", "test_conv_fwd_bwd"]),
     # batch norm and max pooling as separate operations (forward and backward; backward only)
     ("SAGA_HIP_NO_BN_POOL_FUSE", "1", ["tests/test_gpu_networks.py", "-k", "resnet50"]),
     ("SAGA_HIP_NO_BN_POOL_BWD_FUSE", "1", ["tests/test_gpu_networks.py", "-k", "resnet50"]),

@@ -54,6 +54,10 @@ CONV_CASES = [
     # per image; a partial last tile, a row length that is no multiple of anything and 56 output channels
     (37, 64, 56, 56, 64, 3, 1, 1, 1),
     (130, 64, 30, 27, 56, 3, 1, 1, 1),
+    # ... and for the backward filter that does the same (tiles of a whole number of 16-pixel steps): 48 output
+    # channels and a last tile of two rows; eight rows of 32 pixels per tile
+    (64, 64, 30, 56, 48, 3, 1, 1, 1),
+    (128, 64, 32, 32, 64, 3, 1, 1, 1),
     # dilated (a tenth entry: dilation)
     (2, 16, 13, 12, 24, 3, 2, 1, 1, 2),
     (2, 32, 15, 15, 16, 3, 3, 2, 1, 3),
