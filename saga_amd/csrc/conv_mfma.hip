@@ -70,6 +70,7 @@ struct GatherArgs {
     int bq_relu;
     float *bq_partial;  // null: no link
     int no_stage;      // the epilogue stores straight from registers (experiment switch SAGA_HIP_NO_STAGED_STORES)
+    int b_krsc;        // conv_rows64_wide<.., FLIP>: b is the filter as the forward pass has it (K,R,S,C), not transposed
     unsigned out_bytes; // extent of out, for the epilogue variant that stores through a range-checked buffer (BUFST)
     float *stats;      // forward only, optional: per block row and output channel, sum and sum of
                        // squares of the stored outputs, [ceil(M / BM)][Ngemm][2]
@@ -2659,7 +2660,7 @@ template <int MODE, bool FLIP> __global__ void __launch_bounds__(256, 1) conv_ro
         for(int q = 0; q < 19; q++) { // 64 * 73 = 4672 chunks, 256 per round
             const int L = (q * NW + wave) * 64 + lane;
             const int row = L / 73, cpos = L - row * 73;
-            const unsigned off = (cpos < 72 && row < g.Ngemm && row < 64) ? (unsigned)((row * 576 + cpos * 8) * 2) : OOB;
+            const unsigned off = (cpos < 72 && row < (FLIP && g.b_krsc ? g.Cred : g.Ngemm) && row < 64) ? (unsigned)((row * 576 + cpos * 8) * 2) : OOB;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(stage + q * (NW * 1024)), 16, off, 0, 0, 0);
         }
     }
@@ -2668,14 +2669,34 @@ template <int MODE, bool FLIP> __global__ void __launch_bounds__(256, 1) conv_ro
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     // fragment (tap, kk, j) = halves 16*kk + 8*hi .. +8 of that tap of output channel 32*j + lane%32
     half8_t fb[9][4][TN];
+    if(FLIP && g.b_krsc) {
+        // Backward data straight from the forward filter w[k][tap][c] (no transposed copy: a stand-alone call saves
+        // the launch that makes one): a fragment is 8 consecutive k of one c, which is what the transposing LDS read
+        // delivers - the lane points at row k = 16*kk + fp (the read's second half: + 4) and 4 columns of its tile.
+        const int fp = 8 * (lane >> 5) + ((lane & 15) >> 2), fc = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+        const unsigned src = (unsigned)(uintptr_t)(lds_ptr_t)(smem + t.buf_bytes) + fp * (73 * 16) + fc * 2;
 #pragma unroll
-    for(int j = 0; j < TN; j++) {
-        const char *src = smem + t.buf_bytes + (j * 32 + (lane & 31)) * (73 * 16) + hi * 16;
+        for(int j = 0; j < TN; j++)
 #pragma unroll
-        for(int tp = 0; tp < 9; tp++)
+            for(int tp = 0; tp < 9; tp++) {
 #pragma unroll
-            for(int kk = 0; kk < 4; kk++)
-                fb[tp][kk][j] = *(const half8_t *)(src + (FLIP ? 8 - tp : tp) * 128 + kk * 32);
+                for(int kk = 0; kk < 4; kk++)
+                    fb[tp][kk][j] = tr_read8_raw<0, 4 * 73 * 16>(src + kk * (16 * 73 * 16) + ((8 - tp) * 64 + j * 32) * 2);
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+                for(int kk = 0; kk < 4; kk++)
+                    asm volatile("" : "+v"(fb[tp][kk][j]));
+            }
+    } else {
+#pragma unroll
+        for(int j = 0; j < TN; j++) {
+            const char *src = smem + t.buf_bytes + (j * 32 + (lane & 31)) * (73 * 16) + hi * 16;
+#pragma unroll
+            for(int tp = 0; tp < 9; tp++)
+#pragma unroll
+                for(int kk = 0; kk < 4; kk++)
+                    fb[tp][kk][j] = *(const half8_t *)(src + (FLIP ? 8 - tp : tp) * 128 + kk * 32);
+        }
     }
     // (everybody has its fragments before the second tile's rows overwrite them)
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -2990,8 +3011,12 @@ template <int NSTEPS> __global__ void __launch_bounds__(256, 1) conv_bwd_filter_
 
 // Launches conv_rows64 if the geometry is its: returns false (and launches nothing) otherwise.  g: as for
 // launch_gather, with a = the NHWC input (pixel pitch lda), b = [Ngemm][9][64].
-template <bool FLIP> static bool launch_rows64(GatherArgs &g, const CLInfo &lout, hipStream_t st, size_t stats_floats, int *rc)
+// krsc: b is the untransposed forward filter (backward data only): only the kernel that can read it that way may run.
+template <bool FLIP> static bool launch_rows64(GatherArgs &g, const CLInfo &lout, hipStream_t st, size_t stats_floats, int *rc, bool krsc = false)
 {
+    g.b_krsc = krsc ? 1 : 0;
+    if(krsc && (g.Ngemm != 64 || g.Cred != 64))
+        return false;
     static const bool off = getenv("SAGA_HIP_ROWS64") && atoi(getenv("SAGA_HIP_ROWS64")) == 0;
     if(off || g.R != 3 || g.S != 3 || g.Cred != 64 || g.Ngemm > 64 || g.Ngemm % 8 || g.stride != 1 || g.pad != 1 ||
        g.dil != 1 || g.IH != g.OH || g.IW != g.OW || g.OW < 8 || (g.bn_s && (g.bn_flags & SAGA_BN_ADD)) || g.bq_partial || !g.a_bytes || !g.b_bytes)
@@ -3059,6 +3084,8 @@ template <bool FLIP> static bool launch_rows64(GatherArgs &g, const CLInfo &lout
             return true;
         }
     }
+    if(krsc)
+        return false;
     t.buf_bytes = buf_narrow;
     const int epi_at = std::max(2 * t.buf_bytes, epi_back);
     t.epi_off = epi_at - epi_back;
@@ -3558,6 +3585,12 @@ int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const 
             return SAGA_HIP_EWORKSPACE;
     }
     const half_t *wt = (const half_t *)wt_ready;
+    // nobody has transposed the filter: the row-resident 3x3 kernel reads it as it is
+    bool krsc = false;
+    if(!wt && !link && dma_stages() >= 2 && aligned16(w->ptr)) {
+        wt = (const half_t *)w->ptr;
+        krsc = true;
+    }
     if(!wt) {
         const size_t need = (size_t)g.K * g.C * g.R * g.S * sizeof(half_t);
         if(!ws || ws_bytes < need || !aligned16(ws))
@@ -3599,6 +3632,19 @@ int conv_mfma_bwd_data(const SagaTensorView *dy, const SagaTensorView *w, const 
         a.bq_partial = link->partial;
     }
     int rc = 0;
+    if(krsc) {
+        if(launch_rows64<true>(a, ldx, st, 0, &rc, true))
+            return rc;
+        // (not that kernel's geometry: the transposed copy after all)
+        const size_t need = (size_t)g.K * g.C * g.R * g.S * sizeof(half_t);
+        if(!ws || ws_bytes < need || !aligned16(ws))
+            return SAGA_HIP_EWORKSPACE;
+        const int64_t total = (int64_t)g.K * g.C * g.R * g.S;
+        transpose_filter<<<grid_for(total, 256, 256 * 16), 256, 0, st>>>((const half_t *)w->ptr, (half_t *)ws, g.K, g.C,
+                                                                        g.R * g.S);
+        a.b = (const half_t *)ws;
+        a.b_krsc = 0;
+    }
     if(!(dma_stages() >= 2 && !link && launch_rows64<true>(a, ldx, st, 0, &rc)))
         rc = launch_gather<true>(a, st);
     if(link && link->partial_rows)
