@@ -3731,12 +3731,16 @@ int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, cons
         t.y_bytes = nsteps * 16 * 128;
         const int blocks = num_cus();
         const int lds = 2 * t.x_bytes + 2 * t.y_bytes;
-        int dev = 0, lds_max = 0;
+        static const int lds_max = [] {
+            int dev = 0, v = 0;
+            if(hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess)
+                return 64 * 1024;
+            return v;
+        }();
         if((tr * g.W) % 16 == 0 && (nsteps == 14 || nsteps == 16) && ntiles >= 2 * blocks && ntiles < 0x7fffffff &&
            (t.x_bytes >> 12) >= 12 && (t.x_bytes >> 12) <= 13 && (t.y_bytes & 4095) == 0 &&
            (int64_t)g.H * g.W * lx.pitch * 2 < 0x7fff0000ll && (int64_t)g.H * g.W * ldy.pitch * 2 < 0x7fff0000ll &&
-           (size_t)blocks * n * sizeof(float) <= ws_bytes && hipGetDevice(&dev) == hipSuccess &&
-           hipDeviceGetAttribute(&lds_max, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) == hipSuccess && lds <= lds_max) {
+           (size_t)blocks * n * sizeof(float) <= ws_bytes && lds <= lds_max) {
             t.x = (const half_t *)x->ptr;
             t.dy = (const half_t *)dy->ptr;
             t.partial = (float *)ws;
@@ -3747,9 +3751,13 @@ int conv_mfma_bwd_filter(const SagaTensorView *x, const SagaTensorView *dy, cons
             t.K = g.K;
             t.ntiles = (int)ntiles;
             auto kern = nsteps == 14 ? conv_bwd_filter_rows64<14> : conv_bwd_filter_rows64<16>;
-            const hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-            if(e != hipSuccess)
-                return (int)e;
+            static bool once[2] = {false, false};
+            if(!once[nsteps == 16]) {
+                const hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_max);
+                if(e != hipSuccess)
+                    return (int)e;
+                once[nsteps == 16] = true;
+            }
             kern<<<blocks, 256, lds, st>>>(t);
             SAGA_CHECK_LAUNCH();
             filter_reduce_v4<<<(unsigned)((n / 4 + 15) / 16), 256, 0, st>>>(t.partial, (half_t *)dw->ptr, n, blocks, alpha, beta);
