@@ -47,10 +47,10 @@ FAMILIES = {
 # lines, the per-kernel table and the commit the counters were taken at are in
 # profiles/resnet50_b256_fp16_hbm_counters.txt; they go stale when kernels change, hence the label.
 MEASURED_HBM_BYTES_PER_LAUNCH = {
-    "conv": 269518027,
-    "batchnorm": 415181333,
+    "conv": 268838015,
+    "batchnorm": 415183025,
 }
-TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE snapshot at commit 7786cee (profiles/resnet50_b256_fp16_hbm_counters.txt)"
+TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE snapshot at commit 827e3a2 (profiles/resnet50_b256_fp16_hbm_counters.txt)"
 
 
 def by_kind(rows):
