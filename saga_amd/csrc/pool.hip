@@ -448,6 +448,268 @@ __global__ void __launch_bounds__(256) maxpool_fwd_codes_k(DView x, DView y, uin
         *(typename CodeVec<VN>::type *)(codes + ((((size_t)n * P + p) * Q + q) * C + c)) = packed;
 }
 
+// The same pooling for 3x3 windows of stride 2 and padding 1 on fp16 channels-last tensors, whole image rows in LDS.
+// maxpool_fwd_codes_k loads every window for itself: an input element is fetched 2.25 times (the caches serve most
+// of that, but neighbouring output rows run on different dies and the rows they share come from memory twice: 618 MB
+// for the 411 MB stem output of ResNet-50) and, on a batch norm's input, normalised 2.25 times; and its comparisons,
+// two float compares and two selects per element and window position, make it bound by the vector ALU, not by memory
+// (236 us for that tensor, 2.4 TB/s).
+// Here one persistent block per CU owns strips of TR output rows of an image.  The 2 * TR + 1 input rows go to LDS
+// once (buffer_load ... lds; rows above / below the image fall outside a buffer resource that covers just the image),
+// the next strip's while this one is worked on.  Every element is normalised once, in place, and left there as a
+// 16-bit ORDER KEY, two to a register: 0x8000 + |v| for v >= 0 and 0x7fff - |v| for v < 0, minus 0x03ff, so that
+// unsigned integer order is the order of the values (-inf = 0 ... +inf = 0xf801), -0, raised to +0 before, shares
+// its key (a tie, as in a float compare) and every NaN, of either sign and any payload, is the one largest key
+// 0xf802 (the first NaN of a window wins, as there).  relu is max(key, key of 0).  The window maximum is then 8
+// packed integer maxima per register and the position code of the FIRST maximum is min over k of
+// (key_k == maximum ? k : 0xffff), also packed: 4 instructions per two elements and window position instead of
+// some 20.  A position outside the image reads the window's centre row / column instead and is numbered 16 + k.
+// Pooled values and codes equal maxpool_fwd_codes_k's, except that a pooled -0 comes out as +0 and a pooled NaN as
+// a quiet one of positive sign.  144 us for the tensor above.
+typedef __attribute__((address_space(3))) void *pool_lds_ptr_t;
+typedef unsigned short pool_u16x2 __attribute__((ext_vector_type(2)));
+typedef short pool_i16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 pool_h2 __attribute__((ext_vector_type(2)));
+typedef unsigned pool_u32x4 __attribute__((ext_vector_type(4)));
+constexpr int POOL_ROWS_NT = 1024; // threads per block
+constexpr int POOL_ROWS_NLD = 5;   // 16-byte chunks per lane of a strip's rows (at most 80 KB; two buffers of them)
+struct PoolRowsArgs {
+    const half_t *x;
+    half_t *y;
+    uint8_t *codes;
+    const float *ss;
+    int C, H, W, P, Q, CV;   // CV = C / 8 channel vectors per pixel (a power of two)
+    int xs0, xs2, xs3;       // pitches of x in elements: image, row, pixel
+    int64_t ys0, ys2, ys3;   // of y
+    int TR, spi, nstrips;    // output rows per strip, strips per image, strips
+    int chunks;              // (2 * TR + 1) * W * CV
+    int relu;
+    unsigned ximg_bytes;     // H * xs2 * 2
+};
+
+// (packed 16-bit integer operations as inline assembly: written as vector expressions the compiler recognises
+// min(x, 1) as a comparison and falls back to one compare and one select per half)
+__device__ __forceinline__ unsigned pk_max_u16(unsigned a, unsigned b)
+{
+    unsigned r;
+    asm("v_pk_max_u16 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ unsigned pk_min_u16(unsigned a, unsigned b)
+{
+    unsigned r;
+    asm("v_pk_min_u16 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+// a * b + c per half, saturating at 0xffff
+__device__ __forceinline__ unsigned pk_mad_sat_u16(unsigned a, unsigned b, unsigned c)
+{
+    unsigned r;
+    asm("v_pk_mad_u16 %0, %1, %2, %3 clamp" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+// a - b and a + b per half, wrapping
+__device__ __forceinline__ unsigned pk_sub_u16(unsigned a, unsigned b)
+{
+    unsigned r;
+    asm("v_pk_sub_u16 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ unsigned pk_add_u16(unsigned a, unsigned b)
+{
+    unsigned r;
+    asm("v_pk_add_u16 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+// per half: 0xffff when bit 15 is set, else 0
+__device__ __forceinline__ unsigned pk_sign_u16(unsigned a)
+{
+    return __builtin_bit_cast(unsigned, (pool_i16x2)(__builtin_bit_cast(pool_i16x2, a) >> (pool_i16x2){15, 15}));
+}
+
+// (LDS accesses of the kernel below as inline assembly: before an LDS access of its own the compiler waits for every
+// buffer_load ... lds in flight, the next strip's included)
+__device__ __forceinline__ pool_u32x4 lds_read16(unsigned addr)
+{
+    pool_u32x4 r;
+    asm volatile("ds_read_b128 %0, %1" : "=v"(r) : "v"(addr) : "memory");
+    return r;
+}
+__device__ __forceinline__ void lds_write16(unsigned addr, pool_u32x4 v)
+{
+    asm volatile("ds_write_b128 %0, %1" : : "v"(addr), "v"(v) : "memory");
+}
+
+template <bool RELU>
+__global__ void __launch_bounds__(POOL_ROWS_NT, 1) maxpool_3x3s2_rows_k(PoolRowsArgs t)
+{
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    constexpr unsigned OOB = 0xffffffffu; // (beyond every image: the load writes zeros)
+    constexpr int NT = POOL_ROWS_NT, NW = NT / 64;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const unsigned lds0 = (unsigned)(uintptr_t)(pool_lds_ptr_t)smem;
+    // chunk L = (q * NW + wave) * 64 + lane of a strip: channel vector L % CV of pixel (L / CV) % W of row L / CV / W
+    unsigned roff[POOL_ROWS_NLD];
+#pragma unroll
+    for(int q = 0; q < POOL_ROWS_NLD; q++) {
+        const int L = (q * NW + wave) * 64 + lane;
+        const int pix = L / t.CV, cv = L - pix * t.CV;
+        const int r = pix / t.W, w = pix - r * t.W;
+        roff[q] = L < t.chunks ? (unsigned)((r * t.xs2 + w * t.xs3 + cv * 8) * 2) : OOB;
+    }
+    // two buffers of whole 1 KB pieces (one load of a wave each)
+    const int buf_bytes = ((t.chunks + 63) >> 6) << 10;
+    // this thread's channel vector is the same for every chunk and output it handles (the block's size is a multiple of CV)
+    const int cv = tid & (t.CV - 1);
+    float sc[8], sh[8];
+#pragma unroll
+    for(int j = 0; j < 8; j++) {
+        sc[j] = t.ss ? t.ss[cv * 8 + j] : 1.0f;
+        sh[j] = t.ss ? t.ss[t.C + cv * 8 + j] : 0.0f;
+    }
+    const unsigned floor_key = 0x7c017c01u; // relu: no key below that of +0
+    const int nout = t.TR * t.Q * t.CV;
+    // a strip's rows into buffer b
+    auto request = [&](int strip, int b) {
+        const int n = strip / t.spi;
+        const int p0 = (strip - n * t.spi) * t.TR;
+        const __amdgpu_buffer_rsrc_t rx =
+            __builtin_amdgcn_make_buffer_rsrc((void *)(t.x + (int64_t)n * t.xs0), 0, t.ximg_bytes, 0x00020000);
+        const unsigned base = (unsigned)((2 * p0 - 1) * t.xs2 * 2); // (negative for the first strip: out of range)
+#pragma unroll
+        for(int q = 0; q < POOL_ROWS_NLD; q++) {
+            const unsigned off = roff[q] == OOB ? OOB : roff[q] + base;
+            if((q * NW + wave) * 64 < t.chunks)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (pool_lds_ptr_t)(smem + b * buf_bytes + (q * NW + wave) * 1024), 16, off, 0, 0, 0);
+        }
+    };
+    // the three window columns of output column q: LDS offset within a row (the centre column's for one outside the
+    // image: a duplicate changes no maximum) and 16 per half for a column outside, to number its positions 16 + k
+    auto columns = [&](int q, unsigned (&col)[3], unsigned (&kcc)[3]) {
+#pragma unroll
+        for(int c = 0; c < 3; c++) {
+            const int w = 2 * q - 1 + c;
+            const bool ok = w >= 0 && w < t.W;
+            col[c] = (unsigned)(((ok ? w : 2 * q) * t.CV + cv) * 16);
+            kcc[c] = ok ? 0u : 0x00100010u;
+        }
+    };
+    // output (p, q) of image n, p the strip's row pl, for this thread's 8 channels
+    auto pool_one = [&](unsigned buf, int n, int p, int pl, int q, const unsigned (&col)[3], const unsigned (&kcc)[3]) {
+        const unsigned row_bytes = (unsigned)(t.W * t.CV * 16);
+        pool_u32x4 v[9];
+        unsigned kc[9];
+#pragma unroll
+        for(int r = 0; r < 3; r++) {
+            const int h = 2 * p - 1 + r;
+            const bool okr = h >= 0 && h < t.H;
+            const unsigned row = buf + (unsigned)(2 * pl + (okr ? r : 1)) * row_bytes;
+            const unsigned kcr = okr ? 0u : 0x00100010u;
+#pragma unroll
+            for(int c = 0; c < 3; c++) {
+                v[r * 3 + c] = lds_read16(row + col[c]);
+                kc[r * 3 + c] = kcr | kcc[c] | (unsigned)(r * 3 + c) * 0x00010001u;
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]), "+v"(v[8])
+                     :
+                     : "memory");
+        pool_u32x4 out;
+        unsigned code[4];
+#pragma unroll
+        for(int i = 0; i < 4; i++) {
+            unsigned m = v[0][i];
+#pragma unroll
+            for(int k = 1; k < 9; k++)
+                m = pk_max_u16(m, v[k][i]);
+            // the first position that holds the maximum: min over k of (k, or 0xffff where v[k] differs from it)
+            unsigned first = 0xffffffffu;
+#pragma unroll
+            for(int k = 0; k < 9; k++)
+                first = pk_min_u16(first, pk_mad_sat_u16(v[k][i] ^ m, 0xffffffffu, kc[k]));
+            code[i] = (first & 0xffu) | (first >> 8 & 0xff00u);
+            // key -> fp16 bits (0xfc01 and above: NaN, made quiet)
+            unsigned ord = pk_add_u16(m, 0x03ff03ffu);
+            ord |= pk_sub_u16(pk_max_u16(ord, 0xfc00fc00u), 0xfc00fc00u) << 9; // (0xfc01 at most: 0 or 1 per half)
+            out[i] = ord ^ (~pk_sign_u16(ord) | 0x80008000u);
+        }
+        *(pool_u32x4 *)(t.y + n * t.ys0 + p * t.ys2 + q * t.ys3 + cv * 8) = out;
+        if(t.codes) {
+            typedef unsigned u2 __attribute__((ext_vector_type(2)));
+            u2 packed;
+            packed[0] = code[0] | code[1] << 16;
+            packed[1] = code[2] | code[3] << 16;
+            *(u2 *)(t.codes + ((((size_t)n * t.P + p) * t.Q + q) * t.C + cv * 8)) = packed;
+        }
+    };
+    // one output per thread and strip at most (the usual case): its row, column and column offsets, once
+    const bool one_pass = nout <= NT;
+    const int pl1 = (tid / t.CV) / t.Q, q1 = (tid / t.CV) - pl1 * t.Q;
+    unsigned col1[3], kcc1[3];
+    columns(q1, col1, kcc1);
+    int b = 0;
+    if((int)blockIdx.x < t.nstrips)
+        request(blockIdx.x, 0);
+    for(int strip = blockIdx.x; strip < t.nstrips; strip += gridDim.x, b ^= 1) {
+        const int n = strip / t.spi;
+        const int p0 = (strip - n * t.spi) * t.TR;
+        const unsigned buf = lds0 + b * buf_bytes;
+        // this strip's rows have landed; every wave is done with the other buffer (and the stores of its last strip)
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if(strip + (int)gridDim.x < t.nstrips)
+            request(strip + gridDim.x, b ^ 1);
+        // values -> order keys, in place
+        for(int L = tid; L < t.chunks; L += NT) {
+            pool_u32x4 win = lds_read16(buf + L * 16);
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(win) : : "memory"); // (the operand keeps the uses behind the wait)
+            // bn_apply_cl's expression, fma(float(x), scale, shift) rounded to fp16 (scale 1 and shift 0 without a norm: the
+            // value itself).  Not v_fma_mixlo_f16 / mixhi: they round the exact sum once, bn_apply_cl's fp32 fma and
+            // conversion round twice, and the results differ in one element of some ten thousand.
+            unsigned pair[4];
+#pragma unroll
+            for(int i = 0; i < 4; i++) {
+                const unsigned wi = win[i]; // (bit_cast of the element expression itself reads element 0 for every i)
+                const pool_h2 h = __builtin_bit_cast(pool_h2, wi);
+                const float f0 = __builtin_fmaf((float)h[0], sc[2 * i], sh[2 * i]);
+                const float f1 = __builtin_fmaf((float)h[1], sc[2 * i + 1], sh[2 * i + 1]);
+                asm("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(pair[i]) : "v"(f0), "v"(f1));
+            }
+            unsigned key[4];
+#pragma unroll
+            for(int i = 0; i < 4; i++) {
+                unsigned bits = pair[i];
+                if constexpr(!RELU) // -0 -> +0 (with relu the floor below does it)
+                    asm("v_pk_add_f16 %0, %1, 0" : "=v"(bits) : "v"(bits));
+                // order of the values: 0x8000 + |v| for v >= 0, 0x7fff - |v| for v < 0; shifted down by 0x03ff (wrapping)
+                // -inf becomes 0, +inf 0xf801 and every NaN, of either sign, lies above: all NaN -> 0xf802
+                const unsigned ord = bits ^ (pk_sign_u16(bits) | 0x80008000u);
+                key[i] = pk_min_u16(pk_sub_u16(ord, 0x03ff03ffu), 0xf802f802u);
+                if constexpr(RELU)
+                    key[i] = pk_max_u16(key[i], floor_key);
+            }
+            lds_write16(buf + L * 16, (pool_u32x4){key[0], key[1], key[2], key[3]});
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if(one_pass) {
+            if(tid < nout && p0 + pl1 < t.P)
+                pool_one(buf, n, p0 + pl1, pl1, q1, col1, kcc1);
+        } else {
+            for(int o = tid; o < nout; o += NT) {
+                const int pq = o / t.CV;
+                const int pl = pq / t.Q, q = pq - pl * t.Q;
+                if(p0 + pl >= t.P)
+                    continue;
+                unsigned col[3], kcc[3];
+                columns(q, col, kcc);
+                pool_one(buf, n, p0 + pl, pl, q, col, kcc);
+            }
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 // floor(a / S) for a that may be negative, S a compile-time constant
 template <int S> __device__ __forceinline__ int floor_div(int a) { return a >= 0 ? a / S : -((-a + S - 1) / S); }
 
@@ -897,10 +1159,85 @@ int saga_hip_maxpool_fwd_codes_bn(const SagaTensorView *x, const SagaTensorView 
 
 } // extern "C"
 
+// The row-resident kernel for 3x3 / stride 2 / padding 1 on fp16 channels-last tensors whose rows do not overlap;
+// false when the shapes do not fit it (SAGA_HIP_POOL_ROWS=0 switches it off).
+static bool launch_maxpool_rows(const SagaTensorView *x, const SagaTensorView *y, uint8_t *codes, int size, int pad,
+                                int stride, hipStream_t st, const float *ss, int relu)
+{
+    static const bool off = getenv("SAGA_HIP_POOL_ROWS") && atoi(getenv("SAGA_HIP_POOL_ROWS")) == 0;
+    if(off || x->dtype != SAGA_HALF || size != 3 || stride != 2 || pad != 1)
+        return false;
+    const int N = x->dims[0], C = x->dims[1], H = x->dims[2], W = x->dims[3], P = y->dims[2], Q = y->dims[3];
+    const int cv = C / 8;
+    if(C % 8 || (cv & (cv - 1)) || cv > 256)
+        return false;
+    const int64_t xs0 = x->strides[0], xs2 = x->strides[2], xs3 = x->strides[3];
+    if(H < 2 || W < 2 || P < 2 || Q < 2) // (a dimension of one element may carry any pitch)
+        return false;
+    if((C > 1 && (x->strides[1] != 1 || y->strides[1] != 1)) || xs3 < C || xs3 % 8 || xs2 % 8 ||
+       (int64_t)(W - 1) * xs3 + C > xs2 || (int64_t)H * xs2 * 2 >= 0x7fff0000)
+        return false;
+    if(N > 1 && (xs0 % 8 || (int64_t)H * xs2 > xs0 || xs0 >= 0x7fffffff || y->strides[0] % 8 || y->strides[0] < 0))
+        return false;
+    for(int i : {2, 3})
+        if(y->strides[i] % 8 || y->strides[i] < 0)
+            return false;
+    if(!aligned16(x->ptr) || !aligned16(y->ptr))
+        return false;
+    // the most output rows whose 2 * TR + 1 input rows fit the kernel's chunks per lane
+    const int64_t row_chunks = (int64_t)W * cv;
+    int tr = (int)((POOL_ROWS_NLD * POOL_ROWS_NT / row_chunks - 1) / 2);
+    tr = std::min(tr, P);
+    if(tr < 1)
+        return false;
+    static int cus = 0;
+    if(!cus) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if(hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
+            return false;
+        cus = prop.multiProcessorCount;
+        if(hipFuncSetAttribute((const void *)maxpool_3x3s2_rows_k<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                               2 * POOL_ROWS_NLD * POOL_ROWS_NT * 16) != hipSuccess ||
+           hipFuncSetAttribute((const void *)maxpool_3x3s2_rows_k<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                               2 * POOL_ROWS_NLD * POOL_ROWS_NT * 16) != hipSuccess) {
+            cus = 0;
+            return false;
+        }
+    }
+    PoolRowsArgs t;
+    t.x = (const half_t *)x->ptr;
+    t.y = (half_t *)y->ptr;
+    t.codes = codes;
+    t.ss = ss;
+    t.C = C, t.H = H, t.W = W, t.P = P, t.Q = Q, t.CV = cv;
+    t.xs0 = N > 1 ? (int)xs0 : 0, t.xs2 = (int)xs2, t.xs3 = (int)xs3;
+    t.ys0 = N > 1 ? y->strides[0] : 0, t.ys2 = y->strides[2], t.ys3 = y->strides[3];
+    t.TR = tr;
+    t.spi = (P + tr - 1) / tr;
+    if((int64_t)t.spi * N > 0x7fffffff)
+        return false;
+    t.nstrips = t.spi * N;
+    t.chunks = (int)((2 * tr + 1) * row_chunks);
+    t.relu = relu;
+    t.ximg_bytes = (unsigned)(H * xs2 * 2);
+    const int lds = 2 * (((t.chunks + 63) >> 6) << 10);
+    if(lds > 2 * POOL_ROWS_NLD * POOL_ROWS_NT * 16)
+        return false;
+    const int blocks = std::min(t.nstrips, cus);
+    if(relu)
+        maxpool_3x3s2_rows_k<true><<<blocks, POOL_ROWS_NT, lds, st>>>(t);
+    else
+        maxpool_3x3s2_rows_k<false><<<blocks, POOL_ROWS_NT, lds, st>>>(t);
+    return true;
+}
+
 static void launch_maxpool_codes(const SagaTensorView *x, const SagaTensorView *y, uint8_t *codes, int size, int pad,
                                  int stride, hipStream_t st, const float *ss, int relu)
 {
     const int vn = x->dtype == SAGA_HALF ? 8 : 4;
+    if(launch_maxpool_rows(x, y, codes, size, pad, stride, st, ss, relu))
+        return;
     dim3 grid, block;
     codes_launch_shape(y->dims[1] / vn, y->dims[3], y->dims[2], y->dims[0], grid, block);
     const DView dvx = dview(x), dvy = dview(y);

@@ -4,8 +4,8 @@ The kernel library reads its switches once per process, so every case runs a sel
 test files in a child process with the switch set: the register-staged fp16 convolution kernels, the
 direct (one output per lane) convolutions, the table-driven fp32 convolutions, batch-norm backward with
 the relu mask read from y, and the engine without relu bit masks / position codes / arena / batched
-filter transposes / batch-norm backward link / reordering of fan-in writers / row-resident convolution kernels /
-pooled batch norm."""
+filter transposes / batch-norm backward link / reordering of fan-in writers / row-resident convolution and pooling
+kernels / pooled batch norm."""
 import os
 import subprocess
 import sys
@@ -41,6 +41,8 @@ CASES = [
     # batch norm and max pooling as separate operations (forward and backward; backward only)
     ("SAGA_HIP_NO_BN_POOL_FUSE", "1", ["tests/test_gpu_networks.py", "-k", "resnet50"]),
     ("SAGA_HIP_NO_BN_POOL_BWD_FUSE", "1", ["tests/test_gpu_networks.py", "-k", "resnet50"]),
+    # 3x3 / stride 2 max pooling with one thread per window instead of whole image rows in LDS
+    ("SAGA_HIP_POOL_ROWS", "0", ["tests/test_gpu_ops.py", "-k", "pool"]),
 ]
 
 

@@ -702,33 +702,39 @@ def test_pooling(k, pad, stride, H, layout, padc, dtype):
         assert_close(host(dxd), dx_ref + 1, dtype, mode + "pool bwd")
 
 
+# (k, pad, stride, H, W, C); the last three: image rows in strips of 2, 1 and 7 output rows, the last strip short
+POOL_CODE_CASES = [(2, 0, 2, 8, 9, 16), (3, 1, 2, 9, 10, 16), (3, 1, 2, 12, 13, 16), (3, 0, 2, 11, 12, 16), (3, 0, 2, 8, 9, 16),
+                   (3, 1, 1, 6, 7, 16), (3, 0, 3, 10, 11, 16), (2, 1, 1, 5, 6, 16),
+                   (3, 1, 2, 37, 112, 64), (3, 1, 2, 10, 75, 128), (3, 1, 2, 43, 300, 8)]
+
+
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("padc", [0, 8])
-@pytest.mark.parametrize("k,pad,stride,H", [(2, 0, 2, 8), (3, 1, 2, 9), (3, 1, 2, 12), (3, 0, 2, 11), (3, 0, 2, 8), (3, 1, 1, 6), (3, 0, 3, 10), (2, 1, 1, 5)])
-def test_maxpool_with_position_codes(k, pad, stride, H, padc, dtype):
+@pytest.mark.parametrize("k,pad,stride,H,W,Cc", POOL_CODE_CASES)
+def test_maxpool_with_position_codes(k, pad, stride, H, W, Cc, padc, dtype):
     """The training pair saga_hip_maxpool_fwd_codes / _bwd_codes on channels-last tensors (dense and
     with a wider channel pitch): y and the recorded first-maximum positions bit-exact against the
     oracle's indices, dx against the oracle's backward - on post-relu data full of exact ties, with
     a NaN and with rows of -inf."""
     rng = np.random.default_rng(k * 100 + H + pad)
-    shape = (3, 16, H, H + 1)
+    shape = (3, Cc, H, W)
     x = np.maximum(rnd(rng, *shape, dtype=dtype), 0)
     x[0, 3, 1, 2] = np.nan
     x[1, 5] = -np.inf
-    P, Q = ref.pool_out(H, k, pad, stride), ref.pool_out(H + 1, k, pad, stride)
-    oshape = (3, 16, P, Q)
+    P, Q = ref.pool_out(H, k, pad, stride), ref.pool_out(W, k, pad, stride)
+    oshape = (3, Cc, P, Q)
     dy = rnd(rng, *oshape, dtype=dtype)
     y_ref, idx_ref = ref.maxpool_fwd(x, k, pad, stride, with_idx=True)
     L = K.lib()
     xd = dev(x, dtype, "nhwc", padc)
     yd = dev(np.zeros(oshape, np.float32), dtype, "nhwc", padc)
-    codes = torch.full((3, P, Q, 16), 255, dtype=torch.uint8, device="cuda")
+    codes = torch.full((3, P, Q, Cc), 255, dtype=torch.uint8, device="cuda")
     K.check(L.saga_hip_maxpool_fwd_codes(C.byref(K.view(xd)), C.byref(K.view(yd)), K.ptr(codes), k, pad, stride, S()))
     np.testing.assert_array_equal(host(yd), y_ref)
     # code r*k+s -> input position (p*stride-pad+r)*W + (q*stride-pad+s), the oracle's index
     cd = codes.cpu().numpy().astype(np.int64).transpose(0, 3, 1, 2)
     pp, qq = np.meshgrid(np.arange(P), np.arange(Q), indexing="ij")
-    pos = (pp * stride - pad + cd // k) * (H + 1) + (qq * stride - pad + cd % k)
+    pos = (pp * stride - pad + cd // k) * W + (qq * stride - pad + cd % k)
     np.testing.assert_array_equal(pos, idx_ref)
     dx_ref = ref.maxpool_bwd(x, dy, k, pad, stride)
     dyd = dev(dy, dtype, "nhwc", padc)
@@ -744,22 +750,67 @@ def test_maxpool_with_position_codes(k, pad, stride, H, padc, dtype):
     assert rc == -3  # SAGA_HIP_EUNSUPPORTED
 
 
+def test_maxpool_codes_on_zeros_of_both_signs_and_several_nans():
+    """The fp16 3x3 / stride 2 pooling compares 16-bit order keys, not floats.  What a float comparison decides
+    without being asked has to hold there too: -0 and +0 tie (the first one is the maximum), the first NaN of a
+    window wins whatever its sign or payload and whatever follows it (+inf, a 'larger' NaN), a window of -inf
+    reports its first position.  Positions bit-exact against the oracle's indices, values equal."""
+    H, W, Cc = 7, 9, 8
+    bits = np.full((2, Cc, H, W), 0xbc00, np.uint16)  # -1 everywhere
+    neg0, pos0, pinf, ninf = 0x8000, 0x0000, 0x7c00, 0xfc00
+    bits[0, 0, 2, 2], bits[0, 0, 2, 3] = neg0, pos0      # -0 first, then +0
+    bits[0, 1, 2, 2], bits[0, 1, 2, 3] = pos0, neg0      # +0 first, then -0
+    bits[0, 2, 2, 2], bits[0, 2, 2, 3] = 0xfe00, 0x7e00  # a negative NaN, then a positive one
+    bits[0, 3, 2, 2], bits[0, 3, 2, 3] = 0x7c01, 0x7fff  # a signalling NaN, then the one with every bit set
+    bits[0, 4, 2, 2], bits[0, 4, 2, 3] = pinf, 0x7e00    # +inf, then a NaN
+    bits[0, 5, 2, 3], bits[0, 5, 3, 2] = 0xfe00, pinf    # a negative NaN, +inf a row below
+    bits[0, 6] = ninf                                    # nothing but -inf
+    bits[0, 7, 0, 0], bits[0, 7, 6, 8] = neg0, 0xffff    # in the corners, next to the padding
+    bits[1] = bits[0][:, ::-1, ::-1]                     # and everything met from the other side
+    x16 = bits.view(np.float16)
+    x = x16.astype(np.float32)
+    P, Q = ref.pool_out(H, 3, 1, 2), ref.pool_out(W, 3, 1, 2)
+    y_ref, idx_ref = ref.maxpool_fwd(x, 3, 1, 2, with_idx=True)
+    L = K.lib()
+    for flags, fn in ((None, "plain"), (0, "norm"), (K.BN_RELU, "norm + relu")):
+        xd = dev(x16, torch.float16, "nhwc")
+        assert np.array_equal(xd.cpu().numpy().view(np.uint16), bits)
+        yd = dev(np.zeros((2, Cc, P, Q), np.float32), torch.float16, "nhwc")
+        codes = torch.full((2, P, Q, Cc), 255, dtype=torch.uint8, device="cuda")
+        if flags is None:
+            K.check(L.saga_hip_maxpool_fwd_codes(C.byref(K.view(xd)), C.byref(K.view(yd)), K.ptr(codes), 3, 1, 2, S()))
+            want_y, want_idx = y_ref, idx_ref
+        else:  # through the norm's arithmetic with scale 1 and shift 0
+            ss = dev(np.concatenate([np.ones(Cc, np.float32), np.zeros(Cc, np.float32)]))
+            K.check(L.saga_hip_maxpool_fwd_codes_bn(C.byref(K.view(xd)), C.byref(K.view(yd)), K.ptr(codes), 3, 1, 2,
+                                                    K.ptr(ss), flags, S()))
+            xr = np.where(np.isnan(x), x, np.maximum(x, 0)) if flags else x
+            want_y, want_idx = ref.maxpool_fwd(xr, 3, 1, 2, with_idx=True)
+        np.testing.assert_array_equal(host(yd), want_y, err_msg=fn)
+        cd = codes.cpu().numpy().astype(np.int64).transpose(0, 3, 1, 2)
+        pp, qq = np.meshgrid(np.arange(P), np.arange(Q), indexing="ij")
+        pos = (pp * 2 - 1 + cd // 3) * W + (qq * 2 - 1 + cd % 3)
+        np.testing.assert_array_equal(pos, want_idx, err_msg=fn)
+
+
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("k,pad,stride,H,relu", [(3, 1, 2, 12, True), (3, 1, 2, 9, False), (2, 0, 2, 8, True), (3, 0, 2, 11, True)])
-def test_maxpool_on_a_batch_norm_that_is_never_written(k, pad, stride, H, relu, dtype):
+@pytest.mark.parametrize("k,pad,stride,H,relu,W,Cw", [(3, 1, 2, 12, True, 13, 16), (3, 1, 2, 9, False, 10, 16), (2, 0, 2, 8, True, 9, 16),
+                                                     (3, 0, 2, 11, True, 12, 16), (3, 1, 2, 37, True, 112, 64), (3, 1, 2, 10, False, 75, 128),
+                                                     (3, 1, 2, 43, True, 300, 8)])
+def test_maxpool_on_a_batch_norm_that_is_never_written(k, pad, stride, H, relu, W, Cw, dtype):
     """saga_hip_bn_train_fwd_partials with y NULL (statistics only, scale and shift left for the consumer) followed
     by saga_hip_maxpool_fwd_codes_bn, against the same two operators run one after the other with the normalised
     tensor in between: pooled values and position codes bit for bit, saved and running statistics equal."""
     rng = np.random.default_rng(k * 10 + H)
-    Cc = 16 if dtype == torch.float16 else 8
-    shape = (3, Cc, H, H + 1)
+    Cc = Cw if dtype == torch.float16 else 8
+    shape = (3, Cc, H, W)
     x = rnd(rng, *shape, dtype=dtype)
-    P, Q = ref.pool_out(H, k, pad, stride), ref.pool_out(H + 1, k, pad, stride)
+    P, Q = ref.pool_out(H, k, pad, stride), ref.pool_out(W, k, pad, stride)
     s, b = (1 + 0.3 * rng.standard_normal(Cc)).astype(np.float32), (0.2 * rng.standard_normal(Cc)).astype(np.float32)
     s[1] = -s[1]  # a negative scale: the maximum of the normalised values sits at the minimum of x
     L = K.lib()
     xd = dev(x, dtype, "nhwc")
-    rows = 3 * H * (H + 1)
+    rows = 3 * H * W
     # partial sums as a producing convolution would leave them: two rows that add up to the sums over x
     xr = host(xd).astype(np.float64).transpose(0, 2, 3, 1).reshape(rows, Cc)
     half_rows = rows // 2
