@@ -8,7 +8,8 @@ wherever samples are independent.
    images against the oracle (samples do not interact);
  * batch norm (training): per-channel mean and variance of the output are b and s^2; the
    gradient has zero sum and zero correlation with the normalised input per channel;
- * max pooling: every dy lands on exactly one input position;
+ * max pooling: every dy lands on exactly one input position; on a batch norm's input, values and
+   first-maximum position codes against torch on the whole tensor;
  * ResNet-50 b256 at 224x224 through the engine: inference logits of the first images against
    the oracle network (running statistics make samples independent), finite loss and a
    loss-scale step after one training step.
@@ -239,6 +240,38 @@ def test_maxpool_full_size_routes_every_gradient_once():
         for c in (ia, ib):
             holds |= x == y[:, :, r][:, :, :, c]
     assert bool(holds[won].all())
+
+
+def test_maxpool_on_batch_norm_full_size_values_and_first_maximum_codes():
+    """saga_hip_maxpool_fwd_codes_bn on the stem's tensor (256 x 64 x 112 x 112).  Scales that are powers of two
+    make fma(x, scale, shift) exact before its one rounding to fp32, so torch's multiply-add is the same number
+    and the normalised tensor can be built outside the library: pooled values bit for bit, and every position
+    code equal to the FIRST maximum of its window (relu leaves zeros in every window: ties everywhere)."""
+    Cc, H, P = 64, 112, 56
+    g = torch.Generator(device="cuda").manual_seed(12)
+    x = nhwc(torch.randn(N256, Cc, H, H, dtype=HALF, device="cuda", generator=g))
+    sc = (2.0 ** torch.randint(-2, 3, (Cc,), generator=torch.Generator().manual_seed(3)).float())
+    sc[1::3] = -sc[1::3]  # negative scales: the maximum sits at the minimum of x
+    sh = torch.randn(Cc, generator=torch.Generator().manual_seed(4))
+    ss = torch.cat([sc, sh]).cuda()
+    y = nhwc(torch.zeros(N256, Cc, P, P, dtype=HALF, device="cuda"))
+    codes = torch.full((N256, P, P, Cc), 255, dtype=torch.uint8, device="cuda")
+    L = K.lib()
+    K.check(L.saga_hip_maxpool_fwd_codes_bn(C.byref(K.view(x)), C.byref(K.view(y)), K.ptr(codes), 3, 1, 2, K.ptr(ss),
+                                            K.BN_RELU, None))
+    z = torch.relu(x.float() * sc.cuda()[None, :, None, None] + sh.cuda()[None, :, None, None]).to(HALF)
+    assert torch.equal(y, nhwc(torch.nn.functional.max_pool2d(z.float(), 3, 2, 1).to(HALF)))
+    # the nine window positions as nine strided views of the padded tensor; torch.max reports the first maximum
+    zp = torch.nn.functional.pad(z, (1, 1, 1, 1), value=float("-inf"))
+    best = torch.full_like(y, float("-inf"))
+    first = torch.zeros(y.shape, dtype=torch.uint8, device="cuda")
+    for k in range(9):
+        v = zp[:, :, k // 3:k // 3 + 2 * P:2, k % 3:k % 3 + 2 * P:2]
+        take = v > best
+        best = torch.where(take, v, best)
+        first = torch.where(take, torch.full_like(first, k), first)
+    assert torch.equal(best, y)
+    assert torch.equal(codes.permute(0, 3, 1, 2), first)
 
 
 def test_resnet50_b256_through_the_engine():
