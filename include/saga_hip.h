@@ -287,7 +287,11 @@ int saga_hip_pool_bwd(int mode, const SagaTensorView *x, const SagaTensorView *y
  * the forward pass leaves one byte per output element (window position r*size + s of the first maximum,
  * dense N,P,Q,C order, 8-byte aligned buffer of N*C*P*Q bytes) and the backward pass reads only those and
  * dy - same result, less than half the traffic.  Channels-last tensors with whole 16-byte channel vectors,
- * size 2 or 3; SAGA_HIP_EUNSUPPORTED otherwise (use saga_hip_pool_fwd / saga_hip_pool_bwd). */
+ * size 2 or 3; SAGA_HIP_EUNSUPPORTED otherwise (use saga_hip_pool_fwd / saga_hip_pool_bwd).
+ * Zeros of both signs tie (the first one is the maximum, as under a float comparison) and the first NaN of a
+ * window is its maximum.  For fp16 tensors with 3x3 windows, stride 2 and padding 1 (also through
+ * saga_hip_pool_fwd without idx, and in the _bn form below) a pooled -0 is stored as +0 and a pooled NaN as a
+ * quiet NaN of positive sign, whatever the input's sign and payload were. */
 int saga_hip_maxpool_fwd_codes(const SagaTensorView *x, const SagaTensorView *y, uint8_t *codes, int size, int pad,
                                int stride, saga_stream_t stream);
 /* The same on the OUTPUT of a batch norm (+ relu) that is never written: x is the norm's input and every window
