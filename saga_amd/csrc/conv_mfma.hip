@@ -3152,6 +3152,321 @@ __global__ void __launch_bounds__(256) zero_rows(half_t *__restrict__ out, int64
     }
 }
 
+// ---------------------------------------------------------------- 1x1, 64 -> 256 channels: a streaming kernel
+//
+// The 1x1 convolutions that widen 64 channels to 256 over large images (ResNet-50's first stage, 56x56: 103 MB in,
+// 411 MB out at batch 256) are stores and little else: 64 multiply-adds per output.  Through the gather kernel a
+// block lives for two slices of the reduction, and its prologue, its barriers and the drain of its stores are not
+// hidden by the one other block of the CU: 132 - 145 us, 3.6 TB/s, where plain stores reach 6.9 TB/s.  Here the
+// whole filter stays in registers and a WAVEFRONT, not a block, is the unit: it owns strips of 64 pixels and one half
+// of the output channels (the two wavefronts of a pair copy the same strip, the second time from L2), copies a
+// strip into its own LDS (144-byte pixel slots, as in conv_rows64), multiplies and stores - no barrier after the
+// set-up, the next strip's copy in flight behind this strip's stores.  Eight wavefronts per CU, two per SIMD: one
+// converts and stores while the other multiplies.
+template <int MODE>
+__device__ __forceinline__ void c64_epilogue(const GatherArgs &g, float16_t (&acc)[2][2], const float *bnp, char *stg, int lane,
+                                             int c0, const bool (&okr)[2], const int64_t (&pix)[2], const unsigned (&soff)[8],
+                                             float (&st)[16])
+{
+    // (rows64_wide_epilogue for channels c0 .. c0 + 63 of a wider output, this wavefront's kilobytes contiguous,
+    // no beta, and the residual of the folded norm)
+    typedef unsigned u4 __attribute__((ext_vector_type(4)));
+    const int hi = lane >> 5;
+#pragma unroll
+    for(int i = 0; i < 2; i++)
+#pragma unroll
+        for(int j = 0; j < 2; j++) {
+            float f[16];
+#pragma unroll
+            for(int v = 0; v < 16; v++)
+                f[v] = acc[i][j][v];
+            if(g.alpha != 1.0f) {
+#pragma unroll
+                for(int v = 0; v < 16; v++)
+                    f[v] *= g.alpha;
+            }
+            if constexpr(MODE == 1) {
+                float zz[16];
+                if(g.bn_flags & SAGA_BN_ADD)
+                    load_row32(g.z + pix[i] * g.ldz, okr[i], c0 + j * 32, g.Ngemm, hi, zz);
+#pragma unroll
+                for(int q = 0; q < 4; q++) {
+                    const int cl = j * 32 + 8 * q + 4 * hi;
+                    const float4_t sc = *(const float4_t *)(bnp + cl), sh = *(const float4_t *)(bnp + 64 + cl);
+#pragma unroll
+                    for(int e = 0; e < 4; e++) {
+                        float t = __builtin_fmaf(f[4 * q + e], sc[e], sh[e]);
+                        if(g.bn_flags & SAGA_BN_ADD)
+                            t += zz[4 * q + e];
+                        if(g.bn_flags & SAGA_BN_RELU)
+                            t = (t != t) ? t : fmaxf(t, 0.0f);
+                        f[4 * q + e] = t;
+                    }
+                }
+            }
+            const int row = i * 32 + (lane & 31);
+            char *srow = stg + (row >> 3) * 1024 + (row & 7) * 128;
+#pragma unroll
+            for(int q = 0; q < 2; q++) {
+                const unsigned x0 = pack2(f[8 * q + 0], f[8 * q + 1]), x1 = pack2(f[8 * q + 2], f[8 * q + 3]);
+                const unsigned y0 = pack2(f[8 * q + 4], f[8 * q + 5]), y1 = pack2(f[8 * q + 6], f[8 * q + 7]);
+                const auto s0_ = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+                const auto s1_ = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+                const u4 o = {s0_[0], s1_[0], s0_[1], s1_[1]};
+                const int chunk = 4 * j + 2 * q + hi;
+                *(u4 *)(srow + ((chunk ^ (row & 7)) << 4)) = o;
+            }
+        }
+    // LDS operations of one wavefront complete in order: its reads below see its writes above
+    const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc((void *)g.out, 0, g.out_bytes, 0x00020000);
+    const int r8 = lane >> 3, chunk = lane & 7;
+#pragma unroll
+    for(int it = 0; it < 8; it++) {
+        const u4 o = *(const u4 *)(stg + it * 1024 + r8 * 128 + ((chunk ^ r8) << 4));
+        const unsigned off = soff[it]; // (a local: an element of a captured array passed directly makes the host pass drop the kernel)
+        // (plain stores: with the non-temporal hint this kernel alone writes at 6.3 TB/s instead of 5.0, but inside a
+        // network the next operation no longer finds the tail of the tensor in the last-level cache and the step as a
+        // whole takes longer)
+        __builtin_amdgcn_raw_buffer_store_b128(o, ro, off, 0, 0);
+        if constexpr(MODE == 2) {
+            // Statistics of the values as stored: here a lane holds 8 channels of ONE pixel, so sums over pixels are
+            // sums in the lane's own registers (st: 8 sums, 8 sums of squares; a pixel past the tensor's end holds
+            // zeros) and the lanes are added up once, at the end of the launch.
+            typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+            for(int e = 0; e < 4; e++) {
+                const unsigned w = o[e]; // (bit_cast of the element expression itself reads element 0 for every e)
+                const h2 v = __builtin_bit_cast(h2, w);
+                const float a = (float)v[0], b = (float)v[1];
+                st[2 * e] += a;
+                st[2 * e + 1] += b;
+                st[8 + 2 * e] = __builtin_fmaf(a, a, st[8 + 2 * e]);
+                st[8 + 2 * e + 1] = __builtin_fmaf(b, b, st[8 + 2 * e + 1]);
+            }
+        }
+    }
+}
+
+constexpr int C64_BUF = 9216;                       // a strip in LDS: 64 pixel slots of 144 bytes
+constexpr int C64_LDS = 8 * 2 * C64_BUF + 256 * 8;  // two strips per wavefront, the folded norm's table behind them
+
+template <int MODE> __global__ void __launch_bounds__(512, 1) conv1x1_c64_n256(GatherArgs g, int nstrips)
+{
+    float *const stats = MODE == 2 ? g.stats : nullptr;
+    g.stats = nullptr;
+    if constexpr(MODE != 1)
+        g.bn_s = nullptr;
+    constexpr int SLOT = 144, NLD = 9, NST = 16;
+    constexpr unsigned OOB = 0x7fffff00u;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int hi = lane >> 5;
+    const int half = wave & 1, slot = wave >> 1; // which half of the output channels, which of the block's four strips
+    float *bnp = (float *)(smem + 8 * 2 * C64_BUF);
+
+    // The filter, [256][64] halves: through LDS (whole kilobytes per load instruction, rows of 144 bytes so that a
+    // fragment read hits 64 different banks), then this wavefront's 128 channels into registers.
+    {
+        const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void *)g.b, 0, g.b_bytes, 0x00020000);
+#pragma unroll
+        for(int q = 0; q < 5; q++) { // 256 * 9 = 2304 chunks, 512 per round
+            const int L = q * 512 + tid;
+            const int row = L / 9, k = L - row * 9;
+            const unsigned off = (k < 8 && row < 256) ? (unsigned)((row * 64 + k * 8) * 2) : OOB;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr_t)(smem + (q * 8 + wave) * 1024), 16, off, 0, 0, 0);
+        }
+    }
+    if constexpr(MODE == 1) {
+#pragma unroll
+        for(int cb = 0; cb < 4; cb++)
+            bnfold_table<64>(g, bnp + cb * 128, tid, cb * 64);
+    }
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    // fragment (cb, kk, j) = halves 16*kk + 8*hi .. +8 of output channel 128*half + 64*cb + 32*j + lane%32
+    half8_t fb[2][4][2];
+#pragma unroll
+    for(int cb = 0; cb < 2; cb++)
+#pragma unroll
+        for(int j = 0; j < 2; j++) {
+            const char *src = smem + (half * 128 + cb * 64 + j * 32 + (lane & 31)) * SLOT + hi * 16;
+#pragma unroll
+            for(int kk = 0; kk < 4; kk++)
+                fb[cb][kk][j] = *(const half8_t *)(src + kk * 32);
+        }
+    // (everybody has its fragments before the first strips overwrite the staged filter)
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+
+    // Chunk L = q * 64 + lane of a strip's copy: chunk L % 9 of pixel L / 9 (the ninth is the slot's padding), as a
+    // byte offset from the strip's first pixel.  Pixels past the tensor's end are out of the buffer's range.
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void *)g.a, 0, g.a_bytes, 0x00020000);
+    unsigned roff[NLD];
+#pragma unroll
+    for(int q = 0; q < NLD; q++) {
+        const int L = q * 64 + lane;
+        const int p = L / 9, k = L - p * 9;
+        roff[q] = k < 8 ? (unsigned)((p * g.lda + k * 8) * 2) : OOB;
+    }
+    char *const mybuf = smem + wave * 2 * C64_BUF;
+    auto request = [&](int strip, int b) {
+        // (a strip beyond the last: every offset out of range - the loads are issued all the same, so that the count of
+        // outstanding memory operations does not depend on it)
+        const unsigned base = strip < nstrips ? (unsigned)strip * 64u * (unsigned)g.lda * 2u : OOB;
+#pragma unroll
+        for(int q = 0; q < NLD; q++) {
+            const unsigned r = roff[q];
+            const unsigned off = (r == OOB || base == OOB) ? OOB : r + base;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(mybuf + b * C64_BUF + q * 1024), 16, off, 0, 0, 0);
+        }
+    };
+    // this lane's two pixels (row blocks i of the strip) as byte offsets into the copy
+    unsigned abase[2];
+#pragma unroll
+    for(int i = 0; i < 2; i++)
+        abase[i] = (unsigned)(uintptr_t)(lds_ptr_t)mybuf + (i * 32 + (lane & 31)) * SLOT + hi * 16;
+    // the stores' side: store instruction it writes chunk lane%8 of pixel 8*it + lane/8 of the strip
+    unsigned sconst[8];
+#pragma unroll
+    for(int it = 0; it < 8; it++)
+        sconst[it] = (unsigned)(((it * 8 + (lane >> 3)) * g.ldo + half * 128 + (lane & 7) * 8) * 2);
+    const int step = gridDim.x * 4;
+    int strip = blockIdx.x * 4 + slot;
+    float st[2][16];
+#pragma unroll
+    for(int cb = 0; cb < 2; cb++)
+#pragma unroll
+        for(int e = 0; e < 16; e++)
+            st[cb][e] = 0.0f;
+    request(strip, 0);
+    int b = 0, behind = 0;
+    for(; strip < nstrips; strip += step, b ^= 1) {
+        // the next strip's copy goes out behind the previous strip's stores; then this strip's must have landed
+        request(strip + step, b ^ 1);
+        static_assert(NST + NLD == 25 && NLD == 9, "the waits below");
+        if(behind)
+            asm volatile("s_waitcnt vmcnt(25)" ::: "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+        behind = NST;
+        typedef unsigned u4 __attribute__((ext_vector_type(4)));
+        u4 fa[4][2];
+#pragma unroll
+        for(int kk = 0; kk < 4; kk++)
+#pragma unroll
+            for(int i = 0; i < 2; i++)
+                asm volatile("ds_read_b128 %0, %1" : "=v"(fa[kk][i]) : "v"(abase[i] + b * C64_BUF + kk * 32) : "memory");
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(fa[0][0]), "+v"(fa[0][1]), "+v"(fa[1][0]), "+v"(fa[1][1]), "+v"(fa[2][0]), "+v"(fa[2][1]),
+                       "+v"(fa[3][0]), "+v"(fa[3][1])
+                     :
+                     : "memory");
+        bool okr[2];
+        int64_t pix[2];
+#pragma unroll
+        for(int i = 0; i < 2; i++) {
+            const int64_t p = (int64_t)strip * 64 + i * 32 + (lane & 31);
+            okr[i] = p < g.M;
+            pix[i] = okr[i] ? p : 0;
+        }
+        const unsigned strip_off = (unsigned)strip * 64u * (unsigned)g.ldo * 2u; // (the output's bytes fit 31 bits: the host's condition)
+#pragma unroll
+        for(int cb = 0; cb < 2; cb++) {
+            float16_t acc[2][2];
+#pragma unroll
+            for(int i = 0; i < 2; i++)
+#pragma unroll
+                for(int j = 0; j < 2; j++)
+#pragma unroll
+                    for(int v = 0; v < 16; v++)
+                        acc[i][j][v] = 0.0f;
+#pragma unroll
+            for(int kk = 0; kk < 4; kk++)
+#pragma unroll
+                for(int i = 0; i < 2; i++)
+#pragma unroll
+                    for(int j = 0; j < 2; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[cb][kk][j], __builtin_bit_cast(half8_t, fa[kk][i]),
+                                                                           acc[i][j], 0, 0, 0);
+            unsigned soff[8];
+#pragma unroll
+            for(int it = 0; it < 8; it++)
+                soff[it] = (int64_t)strip * 64 + it * 8 + (lane >> 3) < g.M ? sconst[it] + strip_off + cb * 128 : OOB;
+            // (staged in this strip's own copy: its operands are in registers)
+            c64_epilogue<MODE>(g, acc, bnp + (half * 2 + cb) * 128, mybuf + b * C64_BUF, lane, half * 128 + cb * 64, okr, pix, soff,
+                               st[cb]);
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // (copies into this block's LDS may still be in flight)
+    if constexpr(MODE == 2) {
+        // Lane (r8, chunk) of wavefront (slot, half) holds, per channel block cb, sums over its pixels for the channels
+        // 128*half + 64*cb + 8*chunk ..+7: all of them to LDS, then one thread per channel adds its 32 partial sums
+        // (4 wavefronts x 8 lanes) in a fixed order: one row of partial sums per block.
+        float *red = (float *)smem; // [wave][cb][lane][16]
+        __syncthreads();
+#pragma unroll
+        for(int cb = 0; cb < 2; cb++)
+#pragma unroll
+            for(int e = 0; e < 16; e += 4) {
+                const float4_t v4 = {st[cb][e], st[cb][e + 1], st[cb][e + 2], st[cb][e + 3]};
+                *(float4_t *)(red + ((wave * 2 + cb) * 64 + lane) * 16 + e) = v4;
+            }
+        __syncthreads();
+        if(tid < 256) {
+            const int ch = tid & 63, hf = tid >> 7, cb = (tid >> 6) & 1;
+            float s_ = 0.0f, q_ = 0.0f;
+            for(int sl = 0; sl < 4; sl++)
+                for(int r8 = 0; r8 < 8; r8++) {
+                    const float *src = red + (((sl * 2 + hf) * 2 + cb) * 64 + r8 * 8 + (ch >> 3)) * 16 + (ch & 7);
+                    s_ += src[0];
+                    q_ += src[8];
+                }
+            typedef float float2_t __attribute__((ext_vector_type(2)));
+            const float2_t t = {s_, q_};
+            *(float2_t *)(stats + ((int64_t)blockIdx.x * g.Ngemm + tid) * 2) = t;
+        }
+    }
+}
+
+// The launch of conv1x1_c64_n256, or false when the shape is not its (SAGA_HIP_C64_WIDE=0 switches it off, =2 takes
+// it for small tensors too, where a CU gets less than eight strips per wavefront pair).
+static bool launch_c64_wide(GatherArgs &g, const CLInfo &lout, hipStream_t st, size_t stats_floats, int *rc)
+{
+    static const int mode = getenv("SAGA_HIP_C64_WIDE") ? atoi(getenv("SAGA_HIP_C64_WIDE")) : 1; // 2: also where it does not pay
+    const bool on = mode != 0;
+    const int64_t out_bytes = ((lout.rows - 1) * lout.pitch + g.Ngemm) * 2;
+    if(!on || g.R != 1 || g.S != 1 || g.stride != 1 || g.pad != 0 || g.Cred != 64 || g.Ngemm != 256 || g.beta != 0.0f ||
+       (g.lda & 7) || (g.ldo & 7) || !aligned16(g.a) || !aligned16(g.b) || !aligned16(g.out) || !g.a_bytes || !g.b_bytes ||
+       out_bytes >= 0x7fffff00 || (int64_t)g.M * g.lda * 2 >= 0x7fffff00 || g.M != lout.rows)
+        return false;
+    if(g.bn_s && (g.bn_flags & SAGA_BN_ADD) && ((g.ldz & 7) || !aligned16(g.z)))
+        return false;
+    const int nstrips = (g.M + 63) / 64;
+    const int blocks = std::min((nstrips + 3) / 4, num_cus());
+    if((nstrips < 8 * num_cus() && mode != 2) || (g.stats && (size_t)blocks * g.Ngemm * 2 > stats_floats))
+        return false;
+    static bool once = false;
+    if(!once) {
+        for(const void *k : {(const void *)conv1x1_c64_n256<0>, (const void *)conv1x1_c64_n256<1>, (const void *)conv1x1_c64_n256<2>}) {
+            const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, C64_LDS);
+            if(e != hipSuccess) {
+                *rc = (int)e;
+                return true;
+            }
+        }
+        once = true;
+    }
+    g.out_bytes = (unsigned)out_bytes;
+    g.stats_rows = blocks;
+    if(g.bn_s)
+        conv1x1_c64_n256<1><<<blocks, 512, C64_LDS, st>>>(g, nstrips);
+    else if(g.stats)
+        conv1x1_c64_n256<2><<<blocks, 512, C64_LDS, st>>>(g, nstrips);
+    else
+        conv1x1_c64_n256<0><<<blocks, 512, C64_LDS, st>>>(g, nstrips);
+    *rc = (int)hipGetLastError();
+    return true;
+}
+
 static int dma_stages()
 {
     static int v = -1;
@@ -3524,7 +3839,7 @@ int conv_mfma_fwd(const SagaTensorView *x, const SagaTensorView *w, const SagaTe
     if(!set_bn(a, bn, y, ly))
         return SAGA_HIP_EUNSUPPORTED;
     int rc = 0;
-    if(!(dma_stages() >= 2 && !pad && launch_rows64<false>(a, ly, st, stats_floats, &rc)))
+    if(!(dma_stages() >= 2 && !pad && (launch_rows64<false>(a, ly, st, stats_floats, &rc) || launch_c64_wide(a, ly, st, stats_floats, &rc))))
         rc = launch_gather<false>(a, st);
     if(stats_rows)
         *stats_rows = a.stats_rows;

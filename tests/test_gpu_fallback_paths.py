@@ -41,6 +41,9 @@ CASES = [
     # batch norm and max pooling as separate operations (forward and backward; backward only)
     ("SAGA_HIP_NO_BN_POOL_FUSE", "1", ["tests/test_gpu_networks.py", "-k", "resnet50"]),
     ("SAGA_HIP_NO_BN_POOL_BWD_FUSE", "1", ["tests/test_gpu_networks.py", "-k", "resnet50"]),
+    # 1x1 64 -> 256: through the gather kernel; through the streaming kernel also where the tensor is small
+    ("SAGA_HIP_C64_WIDE", "0", ["tests/test_gpu_ops.py", "-k", "test_conv_fwd_bwd or folded_bn or bnstats"]),
+    ("SAGA_HIP_C64_WIDE", "2", ["tests/test_gpu_ops.py", "-k", "test_conv_fwd_bwd or folded_bn or bnstats"]),
     # 3x3 / stride 2 max pooling with one thread per window instead of whole image rows in LDS
     ("SAGA_HIP_POOL_ROWS", "0", ["tests/test_gpu_ops.py", "-k", "pool"]),
 ]

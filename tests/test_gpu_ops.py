@@ -58,6 +58,10 @@ CONV_CASES = [
     # channels and a last tile of two rows; eight rows of 32 pixels per tile
     (64, 64, 30, 56, 48, 3, 1, 1, 1),
     (128, 64, 32, 32, 64, 3, 1, 1, 1),
+    # 1x1 from 64 to 256 channels: enough pixels for the streaming kernel (a partial last strip of 64), and a small
+    # ragged tensor that takes it only when SAGA_HIP_C64_WIDE=2 forces it
+    (45, 64, 56, 55, 256, 1, 0, 1, 1),
+    (3, 64, 30, 31, 256, 1, 0, 1, 1),
     # dilated (a tenth entry: dilation)
     (2, 16, 13, 12, 24, 3, 2, 1, 1, 2),
     (2, 32, 15, 15, 16, 3, 3, 2, 1, 3),
@@ -129,7 +133,10 @@ def test_conv_nonsquare_filter(R, S, layout, dtype):
                                   # 3x3 64 -> 64 with whole rows in LDS (see CONV_CASES)
                                   (37, 64, 56, 64, 3, 1, 1, 3), (130, 64, 30, 56, 3, 1, 1, 1), (40, 64, 56, 64, 3, 1, 1, 0),
                                   # 3x3 layers of the last stages: many channels, tiles with dead rows, 7x7 images
-                                  (3, 128, 14, 256, 3, 1, 1, 3), (6, 64, 7, 136, 3, 1, 1, 1), (2, 64, 28, 64, 3, 1, 1, 2)])
+                                  (3, 128, 14, 256, 3, 1, 1, 3), (6, 64, 7, 136, 3, 1, 1, 1), (2, 64, 28, 64, 3, 1, 1, 2),
+                                  # 1x1 64 -> 256 (see CONV_CASES): norm alone, with relu, with residual and relu
+                                  (45, 64, 56, 256, 1, 0, 1, 0), (43, 64, 56, 256, 1, 0, 1, 3), (3, 64, 30, 256, 1, 0, 1, 3),
+                                  (3, 64, 31, 256, 1, 0, 1, 1)])
 def test_conv_with_folded_bn_inference(case):
     """Convolution with the inference batch norm (+ residual + relu) in its epilogue against the two
     separate operators of the oracle."""
@@ -175,6 +182,9 @@ BNSTATS_CASES = [
     (3, 128, 14, 256, 3, 1, 1, True),
     (6, 64, 7, 136, 3, 1, 1, False),
     (2, 64, 56, 64, 3, 1, 1, True),
+    # 1x1 64 -> 256 (see CONV_CASES)
+    (45, 64, 56, 256, 1, 0, 1, True),
+    (3, 64, 31, 256, 1, 0, 1, False),
 ]
 
 
