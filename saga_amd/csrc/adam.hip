@@ -79,7 +79,10 @@ __global__ void __launch_bounds__(256)
     for(size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += stride) {
         const half4_t gh = ((const half4_t *)g)[i];
         half4_t wh = ((half4_t *)w)[i];
-        float4_t mm = ((float4_t *)mv)[i], vx = ((float4_t *)vv)[i], cc = ((float4_t *)cv)[i];
+        // (the moments and the fp32 master weights are touched once per step: non-temporal, so that they do not push
+        // what the next step reads first out of the last-level cache)
+        float4_t mm = __builtin_nontemporal_load((const float4_t *)mv + i), vx = __builtin_nontemporal_load((const float4_t *)vv + i),
+                 cc = __builtin_nontemporal_load((const float4_t *)cv + i);
 #pragma unroll
         for(int j = 0; j < 4; j++) {
             const half_t gj = gh[j];
@@ -103,9 +106,9 @@ __global__ void __launch_bounds__(256)
             wh[j] = (half_t)wj;
         }
         ((half4_t *)w)[i] = wh;
-        ((float4_t *)mv)[i] = mm;
-        ((float4_t *)vv)[i] = vx;
-        ((float4_t *)cv)[i] = cc;
+        __builtin_nontemporal_store(mm, (float4_t *)mv + i);
+        __builtin_nontemporal_store(vx, (float4_t *)vv + i);
+        __builtin_nontemporal_store(cc, (float4_t *)cv + i);
     }
     for(size_t i = nvec * 4 + (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
         const half_t gj = g[i];

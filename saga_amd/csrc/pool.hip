@@ -641,7 +641,8 @@ __global__ void __launch_bounds__(POOL_ROWS_NT, 1) maxpool_3x3s2_rows_k(PoolRows
             u2 packed;
             packed[0] = code[0] | code[1] << 16;
             packed[1] = code[2] | code[3] << 16;
-            *(u2 *)(t.codes + ((((size_t)n * t.P + p) * t.Q + q) * t.C + cv * 8)) = packed;
+            // (non-temporal: nobody reads the codes before the backward pass)
+            __builtin_nontemporal_store(packed, (u2 *)(t.codes + ((((size_t)n * t.P + p) * t.Q + q) * t.C + cv * 8)));
         }
     };
     // one output per thread and strip at most (the usual case): its row, column and column offsets, once
