@@ -22,7 +22,7 @@ template <> struct VecT<float, 4> { typedef float4_t type; };
 template <> struct VecT<half_t, 1> { typedef half_t type; };
 template <> struct VecT<float, 1> { typedef float type; };
 
-template <typename T, int VN> struct Ld {
+template <typename T, int VN, bool NT = true> struct Ld {
     typedef typename VecT<T, VN>::type V;
     static __device__ __forceinline__ void load(const T *p, float (&o)[VN])
     {
@@ -31,13 +31,13 @@ template <typename T, int VN> struct Ld {
         } else {
             // (non-temporal, like the stores below: these kernels read every tensor once; 9.18 -> 8.99 ms for the
             // batch-norm kernels of a ResNet-50 training step)
-            const V v = __builtin_nontemporal_load((const V *)p);
+            const V v = NT ? __builtin_nontemporal_load((const V *)p) : *(const V *)p;
 #pragma unroll
             for(int j = 0; j < VN; j++)
                 o[j] = (float)v[j];
         }
     }
-    static __device__ __forceinline__ V raw(const T *p) { return __builtin_nontemporal_load((const V *)p); }
+    static __device__ __forceinline__ V raw(const T *p) { return NT ? __builtin_nontemporal_load((const V *)p) : *(const V *)p; }
     static __device__ __forceinline__ float at(const V &v, int j)
     {
         if constexpr(VN == 1)
@@ -237,7 +237,7 @@ __global__ void __launch_bounds__(256)
     for(int j = 0; j < VN; j++)
         a0[j] = a1[j] = 0.0f;
     if(c0 < C) {
-        typedef Ld<T, VN> L;
+        typedef Ld<T, VN, false> L;
         typedef typename L::V V;
         L::load(x + c0, k);
         const RowRun rr = row_run(rows, rb, ty, cvb_);
@@ -415,7 +415,7 @@ __global__ void __launch_bounds__(256)
             sc[j] = recompute ? rs[c0 + j] * rinv[c0 + j] : 0.0f;
             sh[j] = recompute ? __builtin_fmaf(-mean[j], sc[j], rb_[c0 + j]) : 0.0f;
         }
-        typedef Ld<T, VN> L;
+        typedef Ld<T, VN, false> L;
         typedef typename L::V V;
         const RowRun rr = row_run(rows, rb, ty, cvb_);
         const int64_t stride = rr.stride;
