@@ -41,6 +41,29 @@ template <typename T, int VN> struct PV {
                 v[j] = o[j];
             *(float4_t *)p = v;
         }
+    }    // the same for data that is touched once: non-temporal
+    static __device__ __forceinline__ void load_nt(const T *p, float (&o)[VN])
+    {
+        if constexpr(VN == 8 && sizeof(T) == 2) {
+            const half8_t v = __builtin_nontemporal_load((const half8_t *)p);
+#pragma unroll
+            for(int j = 0; j < VN; j++)
+                o[j] = (float)v[j];
+        } else {
+            load(p, o);
+        }
+    }
+    static __device__ __forceinline__ void store_nt(T *p, const float (&o)[VN])
+    {
+        if constexpr(VN == 8 && sizeof(T) == 2) {
+            half8_t v;
+#pragma unroll
+            for(int j = 0; j < VN; j++)
+                v[j] = (T)o[j];
+            __builtin_nontemporal_store(v, (half8_t *)p);
+        } else {
+            store(p, o);
+        }
     }
 };
 
@@ -897,7 +920,10 @@ __global__ void __launch_bounds__(256)
                 const int h = 2 * a - 1 + (e >> 1) - pad, w = 2 * b - 1 + (e & 1) - pad;
                 in[e] = h >= 0 && h < H && w >= 0 && w < W;
                 const int hc = h < 0 ? 0 : h >= H ? H - 1 : h, wc = w < 0 ? 0 : w >= W ? W - 1 : w;
-                PV<T, VN>::load((const T *)x.ptr + off4(x, n, c, hc, wc), xv[e]);
+                if constexpr(MODE == 1) // (the second and last pass over x)
+                    PV<T, VN>::load_nt((const T *)x.ptr + off4(x, n, c, hc, wc), xv[e]);
+                else
+                    PV<T, VN>::load((const T *)x.ptr + off4(x, n, c, hc, wc), xv[e]);
             }
             auto code = [&](int e, int j) -> unsigned {
                 if constexpr(VN == 8)
@@ -942,7 +968,7 @@ __global__ void __launch_bounds__(256)
                         for(int j = 0; j < VN; j++)
                             res[j] += beta * old[j];
                     }
-                    PV<T, VN>::store(o, res);
+                    PV<T, VN>::store_nt(o, res);
                 }
             }
         }
