@@ -47,10 +47,10 @@ FAMILIES = {
 # lines, the per-kernel table and the commit the counters were taken at are in
 # profiles/resnet50_b256_fp16_hbm_counters.txt; they go stale when kernels change, hence the label.
 MEASURED_HBM_BYTES_PER_LAUNCH = {
-    "conv": 268803838,
-    "batchnorm": 415183541,
+    "conv": 255579238,
+    "batchnorm": 413304412,
 }
-TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE snapshot at commit a50fd98 (profiles/resnet50_b256_fp16_hbm_counters.txt)"
+TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE snapshot at commit 83e6fa4 (profiles/resnet50_b256_fp16_hbm_counters.txt)"
 
 
 def by_kind(rows):
