@@ -42,9 +42,10 @@ def dot(a, b):
 
 
 # Cin, H, Cout, R, stride, pad: the conv microbenchmark shape, a strided 3x3 (class-split backward
-# data), a 1x1 stride 2 (classes without taps), a deep 1x1, and the RGB stem (thin-input path)
+# data), a 1x1 stride 2 (classes without taps), a deep 1x1, the RGB stem (thin-input path) and the 1x1 that
+# widens 64 channels to 256 (the streaming kernel)
 FULL_CONVS = [(64, 56, 64, 3, 1, 1), (128, 56, 128, 3, 2, 1), (256, 56, 512, 1, 2, 0), (1024, 14, 256, 1, 1, 0),
-              (3, 224, 64, 7, 2, 3)]
+              (3, 224, 64, 7, 2, 3), (64, 56, 256, 1, 1, 0)]
 
 
 @pytest.mark.parametrize("shape", FULL_CONVS)
